@@ -1,0 +1,154 @@
+/*
+ * slimk_w2a8.h — C ABI of the MI355X (gfx950) W2A8 GEMM path.
+ *
+ * W2A8 = 2-bit weight codes, four per byte in the upstream matrix_packer.py
+ * layout, multiplied by per-token int8 activations on v_mfma_i32_16x16x64_i8,
+ * accumulated in int32 per scale group, and dequantised in a fused epilogue:
+ *
+ *   acc[m,n,g] = sum_{k in group g} q[m,k] * (code[n,k] - zp[g,n])          (int32)
+ *   out[m,n]   = cast( s_a[m] * sum_g float(acc[m,n,g]) * float(scale[g,n]) )
+ *
+ * Upstream interface this replaces: the host launcher
+ *   gemm_tn(m, n, a_k, b_k, alpha, A, ldA, B, ldB, beta, C, ldC, stream)
+ *   slimkernels/cute/gemm/wgmma_sm90_W2A8.cu:428-437
+ * (raw device pointers, explicit leading dimensions, caller-owned buffers, a
+ * stream argument) and the notebook entry wint2_gemm(activation, weight, scale)
+ * (triton.ipynb cell 1).  Upstream names the 2-bit operand "A" with m = output
+ * channels; here M = tokens, N = output channels, K = reduction length.
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer unless said otherwise.  The caller owns
+ *    all buffers; nothing here allocates or frees device memory.
+ *  - Every call only enqueues work on `stream` (a hipStream_t passed as void*;
+ *    NULL = the default stream) and returns; nothing synchronises.
+ *  - Return value: SLIMK_OK or a SLIMK_ERR_* code.  Arguments are validated on
+ *    the host before anything is launched, so a bad call never reaches the GPU.
+ *    slimk_w2a8_last_error() returns a thread-local description of the most
+ *    recent failure on the calling thread.  Nothing throws or aborts.
+ *  - Re-entrant: no mutable global state; concurrent calls from several host
+ *    threads on different streams are fine as long as they do not share a
+ *    split-K workspace.
+ *
+ * Shape limits: K % 64 == 0, group_size in {64, 128, 256}, K % group_size == 0.
+ * M, N >= 1 are otherwise arbitrary (ragged tiles are handled inside).
+ */
+#ifndef SLIMK_W2A8_H
+#define SLIMK_W2A8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SLIMK_W2A8_VERSION 100 /* major*10000 + minor*100 + patch */
+
+enum slimk_status {
+    SLIMK_OK = 0,
+    SLIMK_ERR_NULL_POINTER = 1,
+    SLIMK_ERR_BAD_SHAPE = 2,      /* non-positive size, K/group divisibility, leading dim too small */
+    SLIMK_ERR_MISALIGNED = 3,     /* a pointer or leading dimension breaks a 16-byte rule */
+    SLIMK_ERR_BAD_ENUM = 4,       /* dtype / kernel / dump selector out of range */
+    SLIMK_ERR_WORKSPACE = 5,      /* split-K requested but workspace missing or too small */
+    SLIMK_ERR_HIP = 6,            /* a HIP runtime call failed (see last_error) */
+    SLIMK_ERR_UNSUPPORTED = 7     /* valid but not implemented combination */
+};
+
+enum slimk_dtype { SLIMK_F16 = 0, SLIMK_BF16 = 1 };
+
+/* which GEMM kernel slimk_w2a8_gemm runs */
+enum slimk_kernel {
+    SLIMK_KERNEL_AUTO = 0,   /* skinny split-K for M <= 32, tiled otherwise */
+    SLIMK_KERNEL_SKINNY = 1, /* weight-streaming split-K kernel, M <= 32 */
+    SLIMK_KERNEL_TILED = 2   /* LDS double-buffered MFMA tile kernel, any M */
+};
+
+/* what the optional int32 verification buffer receives */
+enum slimk_dump {
+    SLIMK_DUMP_NONE = 0,
+    SLIMK_DUMP_GROUPS = 1, /* acc_dump[M][N][G]: every per-group accumulator */
+    SLIMK_DUMP_SUM = 2     /* acc_dump[M][N]:    sum over groups of the accumulators */
+};
+
+/* ---- queries (host only, never touch the GPU) ------------------------------------------- */
+
+/* Library version (SLIMK_W2A8_VERSION) and the one ISA the code objects were built for. */
+int slimk_w2a8_version(void);
+const char* slimk_w2a8_arch(void);
+/* Thread-local text of the last error on this thread ("" if none). */
+const char* slimk_w2a8_last_error(void);
+
+/* Byte sizes of the gfx950-private buffers slimk_w2a8_repack fills.  0 on a bad shape. */
+size_t slimk_w2a8_repacked_weight_bytes(int N, int K);
+size_t slimk_w2a8_repacked_scale_bytes(int N, int K, int group_size);
+size_t slimk_w2a8_repacked_zp_bytes(int N, int K, int group_size);
+
+/* Split-K factor slimk_w2a8_gemm would choose for this problem (1 = no workspace needed),
+ * and the workspace bytes a given split needs (0 when split_k <= 1).
+ * No upstream counterpart: upstream has no split-K launcher (the idea appears only in
+ * slimkernels/triton/gemm_splitk.ipynb cell 0). */
+int slimk_w2a8_gemm_auto_split_k(int M, int N, int K, int group_size, int kernel);
+size_t slimk_w2a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int kernel, int split_k);
+
+/* ---- device work ------------------------------------------------------------------------ */
+
+/* Zero a split-K workspace once after allocating it (a fill kernel, safe under graph capture).
+ * The GEMM leaves the workspace's counters at zero again when it finishes, so one
+ * initialisation serves any number of later calls that use the workspace one at a time. */
+int slimk_w2a8_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+
+/* Re-lay the interchange format into the gfx950 streaming layout.
+ *   w_packed [N][ldw] uint8 : matrix_packer.py:33-34 layout, ldw >= K/4 bytes per row
+ *   scales   [G][N]   fp16  : quantization.py:53 layout (G = K / group_size)
+ *   zp       [G][N]   uint8 : zero-points 0..3, or NULL for a uniform zero-point
+ *   w_r / s_r / zp_r        : outputs, sizes from the slimk_w2a8_repacked_*_bytes queries;
+ *                             zp_r may be NULL exactly when zp is NULL
+ * Replaces what upstream gets from TMA + the 128-byte shared-memory swizzle
+ * (wgmma_sm90_W2A8.cu:455-456,465-466): the bank-conflict-free operand order is
+ * baked into the stored weights instead. */
+int slimk_w2a8_repack(const uint8_t* w_packed, int ldw, const uint16_t* scales, const uint8_t* zp,
+                      int N, int K, int group_size,
+                      uint32_t* w_r, uint16_t* s_r, uint8_t* zp_r, void* stream);
+
+/* Per-token activation quantisation (no upstream counterpart; upstream feeds FP8,
+ * wgmma_sm90_W2A8.cu:533-536).
+ *   x [M][ldx] fp16 or bf16 (x_dtype)
+ *   q [M][ldq] int8     = clip(rne(x / s_a[m]), -127, 127)
+ *   s_a [M]    float32  = max(absmax_k |x[m,k]|, 1e-9) / 127
+ *   rowsum [G][ldr] int32 = sum of q over each group (needed by the GEMM to fold
+ *                           zero-points); ldr >= M, ldr % 4 == 0
+ * ldx, ldq in elements; x, q, rowsum 16-byte aligned; ldx % 8 == 0, ldq % 16 == 0. */
+int slimk_w2a8_act_quant(const void* x, int ldx, int x_dtype, int M, int K, int group_size,
+                         int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, void* stream);
+
+/* The GEMM.  Counterpart of gemm_tn (wgmma_sm90_W2A8.cu:428-437); alpha/beta, unused
+ * upstream (:408), are dropped.
+ *   q, ldq, s_a, rowsum, ldr : outputs of slimk_w2a8_act_quant
+ *   w_r, s_r, zp_r           : outputs of slimk_w2a8_repack; zp_r NULL -> every zero-point
+ *                              equals zp_const (2 for the symmetric levels {-2..1},
+ *                              1 for the upstream quantizer)
+ *   out [M][ldo]             : fp16 or bf16 (out_dtype), ldo in elements
+ *   acc_dump, dump_mode      : optional int32 verification output (see slimk_dump); NULL/0
+ *                              in production.  The dump path uses separate kernel
+ *                              instantiations so the timed kernels carry no extra code.
+ *   workspace                : required when the effective split_k > 1
+ *                              (slimk_w2a8_gemm_workspace_bytes), else may be NULL
+ *   kernel, split_k          : SLIMK_KERNEL_* and the split-K factor; 0 = choose */
+int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,
+                    const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
+                    int M, int N, int K, int group_size,
+                    void* out, int ldo, int out_dtype,
+                    int32_t* acc_dump, int dump_mode,
+                    void* workspace, size_t workspace_bytes,
+                    int kernel, int split_k, void* stream);
+
+/* Streaming-read calibration kernel: sums `bytes` (multiple of 16) of device memory into
+ * sink[0..] so that a profiler can relate its FETCH_SIZE counter to a known byte count and
+ * the benchmark can quote the achievable HBM read rate next to the GEMM's. */
+int slimk_w2a8_read_probe(const void* src, size_t bytes, uint32_t* sink, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SLIMK_W2A8_H */

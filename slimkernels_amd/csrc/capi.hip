@@ -1,0 +1,227 @@
+// C ABI of the W2A8 path (declared in include/slimk_w2a8.h): argument validation on
+// the host, kernel selection, launches.  No allocation, no synchronisation.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include <string>
+
+#include "../../include/slimk_w2a8.h"
+#include "w2a8_launch.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+int hip_result(hipError_t e, const char* what) {
+    if (e == hipSuccess) return SLIMK_OK;
+    return fail(SLIMK_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// common K / group checks; returns 0 or an error code (message set)
+int check_kg(int K, int group_size) {
+    if (K <= 0 || K % w2a8::kStepK != 0)
+        return fail(SLIMK_ERR_BAD_SHAPE, "K=%d must be a positive multiple of 64", K);
+    if (group_size != 64 && group_size != 128 && group_size != 256)
+        return fail(SLIMK_ERR_BAD_SHAPE, "group_size=%d must be 64, 128 or 256", group_size);
+    if (K % group_size != 0)
+        return fail(SLIMK_ERR_BAD_SHAPE, "K=%d is not a multiple of group_size=%d", K, group_size);
+    return SLIMK_OK;
+}
+
+bool shape_ok(int K, int group_size) {
+    return K > 0 && K % 64 == 0 && (group_size == 64 || group_size == 128 || group_size == 256) &&
+           K % group_size == 0;
+}
+
+int strips_of(int N) { return (N + w2a8::kStripN - 1) / w2a8::kStripN; }
+
+constexpr size_t kCounterBytesAlign = 256;
+
+size_t counter_bytes(int strips) {
+    size_t b = (size_t)strips * sizeof(unsigned);
+    return (b + kCounterBytesAlign - 1) / kCounterBytesAlign * kCounterBytesAlign;
+}
+
+int resolve_kernel(int M, int kernel) {
+    if (kernel == SLIMK_KERNEL_AUTO) return M <= 32 ? SLIMK_KERNEL_SKINNY : SLIMK_KERNEL_TILED;
+    return kernel;
+}
+
+// Split-K heuristic of the skinny kernel: enough workgroups to cover the 256 CUs about
+// twice, while every wave of a workgroup keeps at least one scale group.
+int auto_split(int M, int N, int K, int group_size, int kernel) {
+    (void)M;
+    if (kernel != SLIMK_KERNEL_SKINNY) return 1;
+    const int strips = strips_of(N);
+    const int G = K / group_size;
+    int split = (512 + strips - 1) / strips;
+    const int max_split = G / 4 > 0 ? G / 4 : 1;
+    if (split > max_split) split = max_split;
+    if (split > 32) split = 32;
+    if (split < 1) split = 1;
+    // drop splits that would be empty: ceil(G / split) groups each
+    const int gps = (G + split - 1) / split;
+    split = (G + gps - 1) / gps;
+    return split;
+}
+
+}  // namespace
+
+extern "C" {
+
+int slimk_w2a8_version(void) { return SLIMK_W2A8_VERSION; }
+const char* slimk_w2a8_arch(void) { return "gfx950"; }
+const char* slimk_w2a8_last_error(void) { return g_last_error.c_str(); }
+
+size_t slimk_w2a8_repacked_weight_bytes(int N, int K) {
+    if (N <= 0 || K <= 0 || K % 64 != 0) return 0;
+    return (size_t)strips_of(N) * (K / 64) * w2a8::kUnitDwords * 4;
+}
+
+size_t slimk_w2a8_repacked_scale_bytes(int N, int K, int group_size) {
+    if (N <= 0 || !shape_ok(K, group_size)) return 0;
+    return (size_t)strips_of(N) * (K / group_size) * 64 * 2;
+}
+
+size_t slimk_w2a8_repacked_zp_bytes(int N, int K, int group_size) {
+    if (N <= 0 || !shape_ok(K, group_size)) return 0;
+    return (size_t)strips_of(N) * (K / group_size) * 64;
+}
+
+int slimk_w2a8_gemm_auto_split_k(int M, int N, int K, int group_size, int kernel) {
+    if (M <= 0 || N <= 0 || !shape_ok(K, group_size)) return 0;
+    return auto_split(M, N, K, group_size, resolve_kernel(M, kernel));
+}
+
+size_t slimk_w2a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int kernel, int split_k) {
+    if (M <= 0 || N <= 0 || !shape_ok(K, group_size)) return 0;
+    const int kern = resolve_kernel(M, kernel);
+    if (split_k <= 0) split_k = auto_split(M, N, K, group_size, kern);
+    if (split_k <= 1 || kern != SLIMK_KERNEL_SKINNY) return 0;
+    const int strips = strips_of(N);
+    const size_t tile = (size_t)(M <= 16 ? 16 : 32) * w2a8::kStripN;
+    return counter_bytes(strips) + (size_t)split_k * strips * tile * sizeof(float);
+}
+
+int slimk_w2a8_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
+    if (workspace_bytes == 0) return SLIMK_OK;
+    if (!workspace) return fail(SLIMK_ERR_NULL_POINTER, "workspace is NULL");
+    if (!aligned16(workspace) || workspace_bytes % 4 != 0)
+        return fail(SLIMK_ERR_MISALIGNED, "workspace must be 16-byte aligned and a multiple of 4 bytes");
+    return hip_result(w2a8::launch_fill_zero(workspace, workspace_bytes, (hipStream_t)stream), "workspace_init");
+}
+
+int slimk_w2a8_repack(const uint8_t* w_packed, int ldw, const uint16_t* scales, const uint8_t* zp,
+                      int N, int K, int group_size,
+                      uint32_t* w_r, uint16_t* s_r, uint8_t* zp_r, void* stream) {
+    if (!w_packed || !scales || !w_r || !s_r) return fail(SLIMK_ERR_NULL_POINTER, "repack: NULL buffer");
+    if (zp && !zp_r) return fail(SLIMK_ERR_NULL_POINTER, "repack: zp given but zp_r is NULL");
+    if (N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "N=%d must be positive", N);
+    if (int rc = check_kg(K, group_size)) return rc;
+    if (ldw < K / 4) return fail(SLIMK_ERR_BAD_SHAPE, "ldw=%d is smaller than K/4=%d", ldw, K / 4);
+    if (!aligned16(w_r) || !aligned16(s_r) || (zp_r && !aligned16(zp_r)))
+        return fail(SLIMK_ERR_MISALIGNED, "repack: outputs must be 16-byte aligned");
+    return hip_result(w2a8::launch_repack(w_packed, ldw, scales, zp, N, K, group_size, w_r, s_r, zp_r,
+                                          (hipStream_t)stream),
+                      "repack");
+}
+
+int slimk_w2a8_act_quant(const void* x, int ldx, int x_dtype, int M, int K, int group_size,
+                         int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, void* stream) {
+    if (!x || !q || !s_a) return fail(SLIMK_ERR_NULL_POINTER, "act_quant: NULL buffer");
+    if (M <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "M=%d must be positive", M);
+    if (int rc = check_kg(K, group_size)) return rc;
+    if (x_dtype != SLIMK_F16 && x_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "x_dtype=%d", x_dtype);
+    if (ldx < K || ldq < K) return fail(SLIMK_ERR_BAD_SHAPE, "ldx=%d / ldq=%d smaller than K=%d", ldx, ldq, K);
+    if (rowsum && ldr < M) return fail(SLIMK_ERR_BAD_SHAPE, "ldr=%d smaller than M=%d", ldr, M);
+    if (!aligned16(x) || !aligned16(q) || ldx % 8 != 0 || ldq % 16 != 0)
+        return fail(SLIMK_ERR_MISALIGNED, "act_quant: x, q must be 16-byte aligned, ldx %% 8 == 0, ldq %% 16 == 0");
+    if (rowsum && (!aligned16(rowsum) || ldr % 4 != 0))
+        return fail(SLIMK_ERR_MISALIGNED, "act_quant: rowsum must be 16-byte aligned and ldr %% 4 == 0");
+    return hip_result(w2a8::launch_act_quant(x, ldx, x_dtype == SLIMK_BF16, M, K, group_size, q, ldq, s_a,
+                                             rowsum, ldr, (hipStream_t)stream),
+                      "act_quant");
+}
+
+int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,
+                    const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
+                    int M, int N, int K, int group_size,
+                    void* out, int ldo, int out_dtype,
+                    int32_t* acc_dump, int dump_mode,
+                    void* workspace, size_t workspace_bytes,
+                    int kernel, int split_k, void* stream) {
+    if (!q || !s_a || !rowsum || !w_r || !s_r || !out) return fail(SLIMK_ERR_NULL_POINTER, "gemm: NULL buffer");
+    if (M <= 0 || N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "M=%d, N=%d must be positive", M, N);
+    if (int rc = check_kg(K, group_size)) return rc;
+    if (out_dtype != SLIMK_F16 && out_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "out_dtype=%d", out_dtype);
+    if (kernel < SLIMK_KERNEL_AUTO || kernel > SLIMK_KERNEL_TILED) return fail(SLIMK_ERR_BAD_ENUM, "kernel=%d", kernel);
+    if (dump_mode < SLIMK_DUMP_NONE || dump_mode > SLIMK_DUMP_SUM) return fail(SLIMK_ERR_BAD_ENUM, "dump_mode=%d", dump_mode);
+    if (dump_mode != SLIMK_DUMP_NONE && !acc_dump) return fail(SLIMK_ERR_NULL_POINTER, "gemm: dump_mode set but acc_dump is NULL");
+    if (ldq < K || ldo < N || ldr < M) return fail(SLIMK_ERR_BAD_SHAPE, "gemm: ldq=%d, ldo=%d or ldr=%d too small", ldq, ldo, ldr);
+    if (zp_const < 0 || zp_const > 3) return fail(SLIMK_ERR_BAD_SHAPE, "zp_const=%d must be 0..3", zp_const);
+    if (!aligned16(q) || ldq % 16 != 0 || !aligned16(rowsum) || ldr % 4 != 0 || !aligned16(w_r) ||
+        !aligned16(s_r) || (zp_r && !aligned16(zp_r)))
+        return fail(SLIMK_ERR_MISALIGNED, "gemm: q, rowsum, w_r, s_r, zp_r must be 16-byte aligned; ldq %% 16 == 0; ldr %% 4 == 0");
+    if ((reinterpret_cast<uintptr_t>(out) & 1u) != 0) return fail(SLIMK_ERR_MISALIGNED, "gemm: out must be 2-byte aligned");
+
+    const int kern = resolve_kernel(M, kernel);
+    if (kern == SLIMK_KERNEL_SKINNY && M > 32)
+        return fail(SLIMK_ERR_UNSUPPORTED, "the skinny kernel handles M <= 32 (M=%d)", M);
+    const int G = K / group_size;
+    if (split_k <= 0) split_k = auto_split(M, N, K, group_size, kern);
+    if (kern == SLIMK_KERNEL_TILED && split_k != 1)
+        return fail(SLIMK_ERR_UNSUPPORTED, "the tiled kernel has no split-K (split_k=%d)", split_k);
+    if (split_k > G) return fail(SLIMK_ERR_BAD_SHAPE, "split_k=%d exceeds the number of groups %d", split_k, G);
+    const int gps = (G + split_k - 1) / split_k;
+    if ((G + gps - 1) / gps != split_k)
+        return fail(SLIMK_ERR_BAD_SHAPE, "split_k=%d leaves empty splits for %d groups", split_k, G);
+
+    w2a8::GemmParams p{};
+    p.q = q; p.s_a = s_a; p.rowsum = rowsum; p.w_r = w_r; p.s_r = s_r; p.zp_r = zp_r;
+    p.out = out; p.acc_dump = dump_mode != SLIMK_DUMP_NONE ? acc_dump : nullptr;
+    p.ldq = ldq; p.ldr = ldr; p.ldo = ldo;
+    p.M = M; p.N = N; p.K = K; p.G = G; p.steps = K / w2a8::kStepK; p.strips = strips_of(N);
+    p.zp_const = zp_const; p.dump_mode = dump_mode;
+    p.split = split_k; p.groups_per_split = gps;
+
+    if (split_k > 1) {
+        const size_t need = slimk_w2a8_gemm_workspace_bytes(M, N, K, group_size, kern, split_k);
+        if (!workspace) return fail(SLIMK_ERR_WORKSPACE, "split_k=%d needs a workspace of %zu bytes", split_k, need);
+        if (workspace_bytes < need)
+            return fail(SLIMK_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, need);
+        if (!aligned16(workspace)) return fail(SLIMK_ERR_MISALIGNED, "workspace must be 16-byte aligned");
+        p.ws_counter = reinterpret_cast<unsigned*>(workspace);
+        p.ws_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counter_bytes(p.strips));
+    }
+
+    hipStream_t st = (hipStream_t)stream;
+    if (dump_mode == SLIMK_DUMP_SUM) {
+        if (int rc = hip_result(w2a8::launch_fill_zero(acc_dump, (size_t)M * N * sizeof(int32_t), st), "dump clear")) return rc;
+    }
+    const int gs = group_size / w2a8::kStepK;
+    const bool asym = zp_r != nullptr;
+    const bool out_bf16 = out_dtype == SLIMK_BF16;
+    if (kern == SLIMK_KERNEL_SKINNY) return hip_result(w2a8::launch_skinny(p, gs, asym, out_bf16, st), "skinny gemm");
+    return hip_result(w2a8::launch_tiled(p, gs, asym, out_bf16, st), "tiled gemm");
+}
+
+int slimk_w2a8_read_probe(const void* src, size_t bytes, uint32_t* sink, void* stream) {
+    if (!src || !sink) return fail(SLIMK_ERR_NULL_POINTER, "read_probe: NULL buffer");
+    if (bytes == 0 || bytes % 16 != 0 || !aligned16(src))
+        return fail(SLIMK_ERR_MISALIGNED, "read_probe: bytes must be a positive multiple of 16 and src 16-byte aligned");
+    return hip_result(w2a8::launch_read_probe(src, bytes, sink, (hipStream_t)stream), "read_probe");
+}
+
+}  // extern "C"

@@ -1,0 +1,81 @@
+// Shared definitions of the gfx950 W2A8 kernels: the streaming weight layout, the
+// kernel parameter block and a few device helpers.
+//
+// Streaming weight layout ("repacked", private to this library)
+// -------------------------------------------------------------
+// The N x K code matrix is cut into units of 64 output channels (a "strip") by
+// 64 reduction elements (a "step").  One unit is 1 KiB: 64 lanes x 4 dwords, stored
+// so that lane l of a wavefront reads its 16 bytes at offset 16*l (one coalesced
+// global_load_dwordx4 / one conflict-free ds_read_b128 per wave and unit).
+//
+//   unit address   = w_r + ((strip * steps + step) * 64 + lane) * 4      [dwords]
+//   lane l         : col = l & 15, quad = l >> 4
+//   dword i, byte b, 2-bit field p of that byte (bits 2p+1:2p) holds the code of
+//       n = strip*64 + p*16 + col          k = step*64 + quad*16 + 4*i + b
+//
+// so `dword_i & (0x03030303 << 2p)` for i = 0..3 IS the 16-byte B operand of
+// v_mfma_i32_16x16x64_i8 for the 16 channels of sub-block p, scaled by 4^p, with no
+// shifts: one v_and per operand dword.  Field p = 3 sits in the sign bits of its
+// byte, so the repack stores it as (code xor 2) = two's complement of (code - 2);
+// the byte then reads as 64 * (code - 2).  The 4^p factor is divided out of the
+// fp32 scale (exact, a power of two) and the "-2" moves into the zero-point.
+//
+// Scales and zero-points are stored per (strip, group) as [16 cols][4 sub-blocks]
+// so that a lane fetches the four values it needs with one 8-byte (4-byte) load.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace w2a8 {
+
+constexpr int kStripN = 64;      // output channels per strip
+constexpr int kStepK = 64;       // reduction elements per MFMA step
+constexpr int kUnitDwords = 256; // dwords per (strip, step) unit
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+struct GemmParams {
+    const int8_t* q;        // [M][ldq]
+    const float* s_a;       // [M]
+    const int32_t* rowsum;  // [G][ldr]
+    const uint32_t* w_r;    // repacked codes
+    const uint16_t* s_r;    // [strips][G][16][4] fp16 bits
+    const uint8_t* zp_r;    // [strips][G][16][4] or nullptr
+    void* out;              // [M][ldo] fp16 / bf16 bits
+    int32_t* acc_dump;      // verification output or nullptr
+    float* ws_partial;      // split-K partial tiles
+    unsigned* ws_counter;   // split-K arrival counters (zero between calls)
+    int ldq, ldr, ldo;
+    int M, N, K;
+    int G;                  // number of scale groups = K / group_size
+    int steps;              // K / 64
+    int strips;             // ceil(N / 64)
+    int zp_const;
+    int dump_mode;
+    int split;              // split-K factor (grid.y)
+    int groups_per_split;   // ceil(G / split)
+};
+
+__device__ __forceinline__ v4i mfma_i8_16x16x64(v4i a, v4i b, v4i c) {
+    // D[i][j] += sum_k A[i][k] * B[k][j]; lane l supplies row/col (l & 15) and the
+    // 16 k-values of quarter (l >> 4); D lane l, element j = row 4*(l>>4)+j, col l&15.
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float half_bits_to_float(uint16_t h) {
+    return (float)__builtin_bit_cast(_Float16, h);
+}
+
+struct OutF16 {
+    static __device__ __forceinline__ uint16_t cast(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+};
+struct OutBF16 {
+    static __device__ __forceinline__ uint16_t cast(float v) {
+        uint32_t x = __float_as_uint(v);
+        if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
+        x += 0x7fffu + ((x >> 16) & 1u);
+        return (uint16_t)(x >> 16);
+    }
+};
+
+}  // namespace w2a8

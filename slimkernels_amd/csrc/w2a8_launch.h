@@ -1,0 +1,28 @@
+// Internal host-side launch entry points, one per kernel family.  Each validates
+// nothing (the C ABI layer did) and only enqueues on the given stream.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "w2a8_common.h"
+
+namespace w2a8 {
+
+hipError_t launch_repack(const uint8_t* w_packed, int ldw, const uint16_t* scales, const uint8_t* zp,
+                         int N, int K, int group_size, uint32_t* w_r, uint16_t* s_r, uint8_t* zp_r,
+                         hipStream_t stream);
+
+hipError_t launch_act_quant(const void* x, int ldx, bool x_bf16, int M, int K, int group_size,
+                            int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, hipStream_t stream);
+
+hipError_t launch_fill_zero(void* p, size_t bytes, hipStream_t stream);
+
+hipError_t launch_read_probe(const void* src, size_t bytes, uint32_t* sink, hipStream_t stream);
+
+// m_blocks = 1 (M <= 16) or 2 (M <= 32); gs = 64-element steps per scale group (1, 2 or 4)
+hipError_t launch_skinny(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
+
+hipError_t launch_tiled(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
+
+}  // namespace w2a8

@@ -1,0 +1,218 @@
+"""Tensor-level wrappers around the C ABI.
+
+Call pattern of the path (upstream has only the raw launcher
+gemm_tn(m, n, a_k, b_k, alpha, A, ldA, B, ldB, beta, C, ldC, stream),
+slimkernels/cute/gemm/wgmma_sm90_W2A8.cu:428-437, and the notebook entry
+wint2_gemm(activation, weight, scale), triton.ipynb cell 1):
+
+    w  = repack_w2(packed, scales, zp=None, group_size=128)   # once per weight
+    qa = quantize_act_int8(x, group_size=128)                 # per forward
+    y  = w2a8_gemm(qa, w, out_dtype=torch.float16)            # per forward
+    y  = wint2_gemm(x, packed.T, scales)                      # one-shot convenience form
+
+Every function raises if the HIP library is missing or a call fails; nothing here
+computes on the CPU.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Optional
+
+import numpy as np
+import torch
+
+from .. import _lib
+
+_DT = {torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
+
+
+def _stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_cuda(t: torch.Tensor, name: str):
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got device {t.device}); there is no CPU path")
+
+
+@dataclasses.dataclass
+class W2A8Weight:
+    """Weights of one linear layer in the gfx950 streaming layout."""
+    w_r: torch.Tensor                 # int32, repacked 2-bit codes
+    s_r: torch.Tensor                 # float16, repacked group scales
+    zp_r: Optional[torch.Tensor]      # uint8 repacked zero-points, or None (uniform)
+    zp_const: int
+    N: int
+    K: int
+    group_size: int
+    workspace: Optional[torch.Tensor] = None  # lazily created split-K workspace (uint8)
+
+    @property
+    def device(self):
+        return self.w_r.device
+
+
+@dataclasses.dataclass
+class QuantizedActivation:
+    q: torch.Tensor        # int8 [M, K]
+    s_a: torch.Tensor      # float32 [M]
+    rowsum: torch.Tensor   # int32 [G, ldr]
+    group_size: int
+
+
+def repack_w2(packed, scales, zp=None, group_size: int = 128, zp_const: int = 2,
+              device="cuda") -> W2A8Weight:
+    """Interchange format -> streaming layout, on the GPU.
+
+    packed: uint8 [N, K/4] (pack_matrix layout), scales: float16 [G, N] (quantize layout),
+    zp: uint8 [G, N] or None for a uniform zero-point ``zp_const``.  numpy arrays or tensors."""
+    L = _lib.lib()
+    dev = torch.device(device)
+    packed_t = torch.as_tensor(np.ascontiguousarray(packed) if isinstance(packed, np.ndarray) else packed)
+    scales_t = torch.as_tensor(np.ascontiguousarray(scales) if isinstance(scales, np.ndarray) else scales)
+    if packed_t.dtype != torch.uint8 or packed_t.dim() != 2:
+        raise ValueError("packed must be a 2-D uint8 array [N, K/4]")
+    if scales_t.dtype != torch.float16 or scales_t.dim() != 2:
+        raise ValueError("scales must be a 2-D float16 array [G, N]")
+    N, K = packed_t.shape[0], packed_t.shape[1] * 4
+    if K % group_size != 0 or tuple(scales_t.shape) != (K // group_size, N):
+        raise ValueError(f"scales shape {tuple(scales_t.shape)} does not match (K/group_size, N) = "
+                         f"{(K // group_size if group_size else 0, N)}")
+    packed_d = packed_t.to(dev).contiguous()
+    scales_d = scales_t.to(dev).contiguous()
+    zp_d = None
+    if zp is not None:
+        zp_t = torch.as_tensor(np.ascontiguousarray(zp) if isinstance(zp, np.ndarray) else zp)
+        if zp_t.dtype != torch.uint8 or tuple(zp_t.shape) != tuple(scales_t.shape):
+            raise ValueError("zp must be uint8 with the shape of scales")
+        zp_d = zp_t.to(dev).contiguous()
+    wb = L.slimk_w2a8_repacked_weight_bytes(N, K)
+    sb = L.slimk_w2a8_repacked_scale_bytes(N, K, group_size)
+    if wb == 0 or sb == 0:
+        raise ValueError(f"unsupported shape N={N}, K={K}, group_size={group_size} "
+                         "(K % 64 == 0, group_size in (64, 128, 256), K % group_size == 0)")
+    w_r = torch.empty(wb // 4, dtype=torch.int32, device=dev)
+    s_r = torch.empty(sb // 2, dtype=torch.float16, device=dev)
+    zp_r = torch.empty(L.slimk_w2a8_repacked_zp_bytes(N, K, group_size), dtype=torch.uint8, device=dev) \
+        if zp_d is not None else None
+    with torch.cuda.device(dev):
+        _lib.check(L.slimk_w2a8_repack(packed_d.data_ptr(), packed_d.stride(0), scales_d.data_ptr(),
+                                       zp_d.data_ptr() if zp_d is not None else None, N, K, group_size,
+                                       w_r.data_ptr(), s_r.data_ptr(),
+                                       zp_r.data_ptr() if zp_r is not None else None, _stream_ptr(dev)))
+        # packed_d / scales_d are consumed by the enqueued kernels: keep them alive until done
+        torch.cuda.current_stream(dev).synchronize()
+    return W2A8Weight(w_r, s_r, zp_r, int(zp_const), N, K, group_size)
+
+
+def quantize_act_int8(x: torch.Tensor, group_size: int = 128) -> QuantizedActivation:
+    """Per-token symmetric int8 quantisation: x [M, K] fp16/bf16 -> q, s_a, per-group row sums."""
+    L = _lib.lib()
+    _require_cuda(x, "x")
+    if x.dim() != 2 or x.dtype not in _DT:
+        raise ValueError("x must be a 2-D float16 or bfloat16 tensor")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    M, K = x.shape
+    ldr = (M + 3) // 4 * 4
+    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    s_a = torch.empty((M,), dtype=torch.float32, device=x.device)
+    rowsum = torch.empty((max(K // group_size, 1), ldr), dtype=torch.int32, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(L.slimk_w2a8_act_quant(x.data_ptr(), x.stride(0), _DT[x.dtype], M, K, group_size,
+                                          q.data_ptr(), q.stride(0), s_a.data_ptr(), rowsum.data_ptr(), ldr,
+                                          _stream_ptr(x.device)))
+    return QuantizedActivation(q, s_a, rowsum, group_size)
+
+
+def _workspace(w: W2A8Weight, nbytes: int) -> Optional[torch.Tensor]:
+    if nbytes == 0:
+        return None
+    if w.workspace is None or w.workspace.numel() < nbytes:
+        w.workspace = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+        _lib.check(_lib.lib().slimk_w2a8_workspace_init(w.workspace.data_ptr(), w.workspace.numel(),
+                                                       _stream_ptr(w.device)))
+    return w.workspace
+
+
+def w2a8_gemm(qa: QuantizedActivation, w: W2A8Weight, out_dtype=torch.float16, *, kernel: str = "auto",
+              split_k: int = 0, dump: Optional[str] = None, out: Optional[torch.Tensor] = None):
+    """out[M, N] = dequant( q @ (codes - zp)^T ).  Returns out, or (out, acc) when ``dump`` is
+    "groups" (int32 [M, N, G]) or "sum" (int32 [M, N])."""
+    L = _lib.lib()
+    kern = {"auto": _lib.KERNEL_AUTO, "skinny": _lib.KERNEL_SKINNY, "tiled": _lib.KERNEL_TILED}[kernel]
+    M, K = qa.q.shape
+    if K != w.K or qa.group_size != w.group_size:
+        raise ValueError(f"activation K={K}/group {qa.group_size} does not match weight K={w.K}/group {w.group_size}")
+    if out_dtype not in _DT:
+        raise ValueError("out_dtype must be torch.float16 or torch.bfloat16")
+    dev = qa.q.device
+    if out is None:
+        out = torch.empty((M, w.N), dtype=out_dtype, device=dev)
+    G = K // w.group_size
+    acc, mode = None, _lib.DUMP_NONE
+    if dump == "groups":
+        acc, mode = torch.empty((M, w.N, G), dtype=torch.int32, device=dev), _lib.DUMP_GROUPS
+    elif dump == "sum":
+        acc, mode = torch.empty((M, w.N), dtype=torch.int32, device=dev), _lib.DUMP_SUM
+    elif dump is not None:
+        raise ValueError("dump must be None, 'groups' or 'sum'")
+    with torch.cuda.device(dev):
+        ws_bytes = L.slimk_w2a8_gemm_workspace_bytes(M, w.N, K, w.group_size, kern, split_k)
+        ws = _workspace(w, ws_bytes)
+        _lib.check(L.slimk_w2a8_gemm(
+            qa.q.data_ptr(), qa.q.stride(0), qa.s_a.data_ptr(), qa.rowsum.data_ptr(), qa.rowsum.stride(0),
+            w.w_r.data_ptr(), w.s_r.data_ptr(), w.zp_r.data_ptr() if w.zp_r is not None else None, w.zp_const,
+            M, w.N, K, w.group_size, out.data_ptr(), out.stride(0), _DT[out.dtype],
+            acc.data_ptr() if acc is not None else None, mode,
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+            kern, split_k, _stream_ptr(dev)))
+    return (out, acc) if acc is not None else out
+
+
+def wint2_gemm(activation: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, zp=None,
+               group_size: Optional[int] = None, zp_const: int = 2, out_dtype=None) -> torch.Tensor:
+    """One-shot form with the argument order of the upstream notebook entry
+    wint2_gemm(activation, weight, scale) (triton.ipynb cell 1): ``activation`` [M, K]
+    fp16/bf16, ``weight`` the packed matrix transposed, [K/4, N] uint8 (upstream passes
+    ``packed_weight.T``), ``scale`` [G, N] fp16.  Repacks on every call — use
+    repack_w2 + w2a8_gemm or W2A8Linear in a real loop."""
+    _require_cuda(activation, "activation")
+    packed = weight.t().contiguous()
+    K = packed.shape[1] * 4
+    if group_size is None:
+        group_size = K // scale.shape[0]
+    w = repack_w2(packed, scale, zp, group_size, zp_const, device=activation.device)
+    qa = quantize_act_int8(activation, group_size)
+    return w2a8_gemm(qa, w, out_dtype or activation.dtype)
+
+
+class W2A8Linear(torch.nn.Module):
+    """y = x @ W^T with W held as 2-bit codes (+ optional bias), a swap-in for nn.Linear."""
+
+    def __init__(self, weight: W2A8Weight, bias: Optional[torch.Tensor] = None, out_dtype=torch.float16):
+        super().__init__()
+        self.weight = weight
+        self.bias = bias
+        self.out_dtype = out_dtype
+        self.in_features, self.out_features = weight.K, weight.N
+
+    @classmethod
+    def from_float(cls, weight_nk, group_size=128, mode="sym", bias=None, out_dtype=torch.float16, device="cuda"):
+        from ..quantization import prepare_w2
+        w_np = weight_nk.detach().float().cpu().numpy() if isinstance(weight_nk, torch.Tensor) else np.asarray(weight_nk)
+        packed, scales, zero = prepare_w2(w_np, group_size, mode)
+        uniform = {"sym": 2, "ref": 1}.get(mode)
+        w = repack_w2(packed, scales, None if uniform is not None else zero, group_size,
+                      zp_const=uniform if uniform is not None else 0, device=device)
+        return cls(w, bias, out_dtype)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, x.shape[-1])
+        if x2.dtype not in _DT:
+            x2 = x2.to(self.out_dtype)
+        y = w2a8_gemm(quantize_act_int8(x2, self.weight.group_size), self.weight, self.out_dtype)
+        if self.bias is not None:
+            y = y + self.bias
+        return y.reshape(*lead, self.out_features)

@@ -1,0 +1,80 @@
+"""Shared helpers of the GPU parity tests."""
+import functools
+
+import numpy as np
+import torch
+
+from slimkernels_amd import workloads
+
+
+def bits_to_f32(bits: np.ndarray, bf16: bool) -> np.ndarray:
+    bits = np.ascontiguousarray(bits).view(np.uint16)
+    if bf16:
+        return (bits.astype(np.uint32) << 16).view(np.float32)
+    return bits.view(np.float16).astype(np.float32)
+
+
+def ulp_of(ref_f32: np.ndarray, bf16: bool) -> np.ndarray:
+    """Spacing of the output type at |ref| (fp16: 10 explicit mantissa bits, bf16: 7)."""
+    mant = 7 if bf16 else 10
+    min_exp = -126 if bf16 else -14
+    a = np.abs(ref_f32).astype(np.float64)
+    e = np.floor(np.log2(np.maximum(a, 2.0 ** min_exp)))
+    return 2.0 ** (e - mant)
+
+
+def out_tensor_bits(t: torch.Tensor) -> np.ndarray:
+    return t.detach().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def assert_out_close(gpu_bits, ref_bits, bf16, reorder_bound=None, what=""):
+    """The output criterion of the path: every element within 1 ULP of the output type OR within
+    rtol 1e-3 of the oracle.  `reorder_bound` (optional, per element) additionally admits the fp32
+    rounding noise of summing the per-group terms in another order (split-K), which is what limits
+    elements whose terms cancel to almost zero."""
+    g, r = bits_to_f32(gpu_bits, bf16), bits_to_f32(ref_bits, bf16)
+    assert np.isfinite(g).all(), f"{what}: non-finite GPU output"
+    diff = np.abs(g.astype(np.float64) - r.astype(np.float64))
+    tol = np.maximum(ulp_of(r, bf16), 1e-3 * np.abs(r))
+    if reorder_bound is not None:
+        tol = np.maximum(tol, reorder_bound)
+    bad = diff > tol
+    assert not bad.any(), (f"{what}: {int(bad.sum())} of {bad.size} outputs off; worst |diff|/tol = "
+                           f"{float((diff / tol).max()):.3g} at {np.unravel_index(np.argmax(diff / tol), diff.shape)}")
+    return float((np.ascontiguousarray(gpu_bits).view(np.uint16) == np.ascontiguousarray(ref_bits).view(np.uint16)).mean())
+
+
+def reorder_bound(acc: np.ndarray, scale_half: np.ndarray, s_a: np.ndarray) -> np.ndarray:
+    """G * 2^-24 * s_a[m] * sum_g |acc[m,n,g]| * scale[g,n]: worst-case drift of an fp32 sum of the
+    per-group terms under re-association."""
+    s = np.asarray(scale_half, np.float16).astype(np.float64)
+    mag = np.einsum("mng,gn->mn", np.abs(acc).astype(np.float64), s)
+    return acc.shape[2] * 2.0 ** -24 * mag * np.asarray(s_a, np.float64)[:, None]
+
+
+@functools.lru_cache(maxsize=8)
+def _quantized_weight(n, k, g, mode, dist, seed):
+    return workloads.make_quantized_weight(workloads.Case("w", 1, n, k, group_size=g, mode=mode, weight_dist=dist, seed=seed))
+
+
+def quantized_weight(case):
+    """make_quantized_weight, memoised on everything the weight depends on (M does not matter)."""
+    return _quantized_weight(case.N, case.K, case.group_size, case.mode, case.weight_dist, case.seed)
+
+
+def device_inputs(ops, case, packed, scales, zero, x_half):
+    """Upload one case: returns (W2A8Weight, x tensor)."""
+    uniform = case.zp_const
+    w = ops.repack_w2(packed, scales, None if uniform is not None else zero, case.group_size,
+                      zp_const=uniform if uniform is not None else 0)
+    x = torch.from_numpy(x_half).cuda()
+    return w, x
+
+
+def torch_dtype(case):
+    return torch.bfloat16 if case.out_dtype == "bfloat16" else torch.float16
+
+
+def small_case(M, N, K, g, mode, seed, out_dtype="float16", outliers=False):
+    return workloads.Case("t", M, N, K, group_size=g, mode=mode, out_dtype=out_dtype,
+                          weight_dist="uniform" if mode == "asym" else "normal", outliers=outliers, seed=seed)

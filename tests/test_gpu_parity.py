@@ -1,0 +1,169 @@
+"""GPU parity: the HIP kernels (through the C ABI) against the CPU oracle on the same seeded
+inputs.  int8 / int32 / index results must be bit-exact; fp16 / bf16 outputs within
+rtol 1e-3 or 1 ULP of the output type (the tiled kernel, which sums groups in the oracle's
+order with the same fused multiply-add, is additionally required to be bit-identical)."""
+import numpy as np
+import pytest
+import torch
+
+from slimkernels_amd import layout, workloads
+import parity_utils as pu
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+# ------------------------------------------------------------------ repack
+@pytest.mark.parametrize("N,K,g,with_zp", [(64, 64, 64, False), (100, 256, 128, True), (4096, 4096, 128, False),
+                                           (1000, 512, 256, True), (16, 128, 64, True)])
+def test_repack_matches_layout_definition(gpu_ops, N, K, g, with_zp):
+    _say("repack", N, K, g, with_zp)
+    rng = np.random.default_rng(N + K)
+    packed = rng.integers(0, 256, (N, K // 4), dtype=np.uint8)
+    scales = rng.uniform(0.001, 0.03, (K // g, N)).astype(np.float16)
+    zp = rng.integers(0, 4, (K // g, N), dtype=np.uint8) if with_zp else None
+    w = gpu_ops.repack_w2(packed, scales, zp, g)
+    strips, steps = -(-N // 64), K // 64
+    got = w.w_r.cpu().numpy().view(np.uint32).reshape(strips, steps, 64, 4)
+    np.testing.assert_array_equal(got, layout.repack_codes(packed))
+    np.testing.assert_array_equal(layout.unrepack_codes(got, N, K), packed)
+    np.testing.assert_array_equal(w.s_r.cpu().numpy().reshape(strips, K // g, 16, 4), layout.repack_group_values(scales))
+    if with_zp:
+        np.testing.assert_array_equal(w.zp_r.cpu().numpy().reshape(strips, K // g, 16, 4), layout.repack_group_values(zp))
+
+
+# ------------------------------------------------------------------ activation quantisation
+@pytest.mark.parametrize("M,K,g,bf16,outliers", [(1, 4096, 128, False, True), (16, 4096, 128, False, True),
+                                                 (77, 4096, 128, False, False), (3, 13824, 128, False, False),
+                                                 (5, 8192, 64, True, False), (33, 256, 256, False, False),
+                                                 (2, 64, 64, False, False)])
+def test_act_quant_bit_exact(gpu_ops, oracle, M, K, g, bf16, outliers):
+    _say("act_quant", M, K, g, bf16)
+    case = pu.small_case(M, 64, K, g, "sym", seed=M * 7 + K, outliers=outliers)
+    x = workloads.make_activation(case)
+    x[min(1, M - 1), : min(K, 70)] = 0.0
+    if M > 2:
+        x[2] = 0.0  # an all-zero token
+    if bf16:
+        xt = torch.from_numpy(x.astype(np.float32)).to(torch.bfloat16)
+        bits = xt.view(torch.int16).numpy().view(np.uint16)
+        q, s_a, rs = oracle.c_act_quant(bits, g, is_bf16=True)
+    else:
+        xt = torch.from_numpy(x)
+        q, s_a, rs = oracle.c_act_quant(x, g)
+    qa = gpu_ops.quantize_act_int8(xt.cuda(), g)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(qa.s_a.cpu().numpy(), s_a)
+    np.testing.assert_array_equal(qa.q.cpu().numpy(), q)
+    np.testing.assert_array_equal(qa.rowsum.cpu().numpy()[:, :M], rs)
+
+
+# ------------------------------------------------------------------ GEMM on small and ragged shapes
+def _run_case(gpu_ops, oracle, case, kernel, split_k=0, dump="groups", exact_out=False):
+    _say("gemm", case.name, kernel, "split", split_k, "dump", dump)
+    packed, scales, zero = pu.quantized_weight(case)
+    x = workloads.make_activation(case)
+    bf16 = case.out_dtype == "bfloat16"
+    ref = oracle.reference_forward(x, packed, scales, zero, case.group_size, out_bf16=bf16, want_acc=True)
+    w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, x)
+    qa = gpu_ops.quantize_act_int8(xd, case.group_size)
+    out, acc = gpu_ops.w2a8_gemm(qa, w, pu.torch_dtype(case), kernel=kernel, split_k=split_k, dump=dump)
+    out2 = gpu_ops.w2a8_gemm(qa, w, pu.torch_dtype(case), kernel=kernel, split_k=split_k)  # production instantiation
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(qa.q.cpu().numpy(), ref["q"])
+    if dump == "groups":
+        np.testing.assert_array_equal(acc.cpu().numpy(), ref["acc"])
+    else:
+        np.testing.assert_array_equal(acc.cpu().numpy(), ref["acc"].sum(axis=2))
+    bound = pu.reorder_bound(ref["acc"], scales, ref["s_a"])
+    for o in (out, out2):
+        bits = pu.out_tensor_bits(o)
+        if exact_out:
+            np.testing.assert_array_equal(bits, ref["out_bits"])
+        else:
+            pu.assert_out_close(bits, ref["out_bits"], bf16, bound, case.name)
+    np.testing.assert_array_equal(pu.out_tensor_bits(out), pu.out_tensor_bits(out2))
+
+
+SMALL = [
+    # M, N, K, g, mode, out
+    (1, 64, 128, 64, "sym", "float16"),
+    (16, 128, 512, 128, "sym", "float16"),
+    (7, 100, 256, 128, "asym", "float16"),
+    (32, 192, 1024, 256, "sym", "bfloat16"),
+    (17, 70, 768, 64, "asym", "bfloat16"),
+    (3, 4096, 256, 128, "ref", "float16"),
+]
+
+
+@pytest.mark.parametrize("M,N,K,g,mode,out", SMALL)
+def test_skinny_small(gpu_ops, oracle, M, N, K, g, mode, out):
+    case = pu.small_case(M, N, K, g, mode, seed=M + N, out_dtype=out)
+    _run_case(gpu_ops, oracle, case, "skinny", split_k=1)
+    _run_case(gpu_ops, oracle, case, "skinny", split_k=0, dump="sum")
+    G = K // g
+    if G >= 2:
+        _run_case(gpu_ops, oracle, case, "skinny", split_k=2)
+
+
+@pytest.mark.parametrize("M,N,K,g,mode,out", SMALL + [
+    (77, 200, 512, 128, "asym", "float16"),
+    (129, 130, 320, 64, "sym", "float16"),
+    (300, 64, 256, 128, "sym", "bfloat16"),
+])
+def test_tiled_small(gpu_ops, oracle, M, N, K, g, mode, out):
+    case = pu.small_case(M, N, K, g, mode, seed=M + N + 1, out_dtype=out)
+    _run_case(gpu_ops, oracle, case, "tiled", dump="groups", exact_out=True)
+    _run_case(gpu_ops, oracle, case, "tiled", dump="sum", exact_out=True)
+
+
+def test_split_k_is_deterministic_and_workspace_reusable(gpu_ops, oracle):
+    case = pu.small_case(16, 256, 2048, 128, "sym", seed=5)
+    packed, scales, zero = pu.quantized_weight(case)
+    x = workloads.make_activation(case)
+    w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, x)
+    qa = gpu_ops.quantize_act_int8(xd, 128)
+    outs = [pu.out_tensor_bits(gpu_ops.w2a8_gemm(qa, w, kernel="skinny", split_k=4)) for _ in range(5)]
+    for o in outs[1:]:
+        np.testing.assert_array_equal(o, outs[0])
+    ref = oracle.reference_forward(x, packed, scales, zero, 128)
+    pu.assert_out_close(outs[0], ref["out_bits"], False, pu.reorder_bound(ref["acc"], scales, ref["s_a"]), "split4")
+
+
+# ------------------------------------------------------------------ the configured workloads
+def test_config_c1(gpu_ops, oracle):
+    case = workloads.config_cases("c1")[0]
+    _run_case(gpu_ops, oracle, case, "auto")
+    _run_case(gpu_ops, oracle, case, "tiled", exact_out=True)
+
+
+@pytest.mark.parametrize("shape", ["qo", "kv", "gate_up", "down"])
+@pytest.mark.parametrize("M", [1, 8, 32])
+def test_config_c2_decode(gpu_ops, oracle, shape, M):
+    N, K = workloads.LLAMA8B_LINEARS[shape]
+    case = workloads.Case("c2", M, N, K, outliers=True)
+    _run_case(gpu_ops, oracle, case, "auto")
+
+
+def test_config_c5_asym_ragged(gpu_ops, oracle):
+    a, b = workloads.config_cases("c5")
+    _run_case(gpu_ops, oracle, a, "auto", exact_out=True)  # M = 77 -> tiled
+    _run_case(gpu_ops, oracle, b, "auto")                  # M = 1  -> skinny split-K
+
+
+def test_wint2_gemm_and_linear_entry_points(gpu_ops, oracle):
+    case = pu.small_case(5, 128, 256, 128, "sym", seed=9)
+    packed, scales, zero = pu.quantized_weight(case)
+    x = workloads.make_activation(case)
+    ref = oracle.reference_forward(x, packed, scales, zero, 128)
+    xd = torch.from_numpy(x).cuda()
+    y = gpu_ops.wint2_gemm(xd, torch.from_numpy(packed).cuda().t(), torch.from_numpy(scales).cuda())
+    pu.assert_out_close(pu.out_tensor_bits(y), ref["out_bits"], False,
+                        pu.reorder_bound(ref["acc"], scales, ref["s_a"]), "wint2_gemm")
+    lin = gpu_ops.W2A8Linear.from_float(workloads.make_weight(case).astype(np.float32), 128, "sym")
+    y2 = lin(xd.reshape(1, 5, 256))
+    assert y2.shape == (1, 5, 128)
+    np.testing.assert_array_equal(pu.out_tensor_bits(y2.reshape(5, 128)), pu.out_tensor_bits(y))
