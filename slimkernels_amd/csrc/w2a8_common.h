@@ -66,8 +66,13 @@ __device__ __forceinline__ float half_bits_to_float(uint16_t h) {
     return (float)__builtin_bit_cast(_Float16, h);
 }
 
+// The output is defined as cast(fp32 product): the empty asm keeps the compiler from folding the
+// caller's fp32 multiply into a v_fma_mixlo_f16, which would round the exact product once.
 struct OutF16 {
-    static __device__ __forceinline__ uint16_t cast(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+    static __device__ __forceinline__ uint16_t cast(float v) {
+        asm volatile("" : "+v"(v));
+        return __builtin_bit_cast(uint16_t, (_Float16)v);
+    }
 };
 struct OutBF16 {
     static __device__ __forceinline__ uint16_t cast(float v) {
