@@ -1,0 +1,302 @@
+#!/usr/bin/env python3
+"""Benchmark of the W2A8 GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload (config "c2", the decode regime the headline metric is quoted on): one step =
+24 skinny split-K GEMM launches, M in {1,2,4,8,16,32} over the four Llama-3-8B linear
+shapes (4096x4096, 1024x4096, 14336x4096, 4096x14336), 2-bit symmetric group-128 weights,
+per-token int8 activations with 0.1 % outlier channels, fp16 out.  Inputs are resident in
+HBM before the timed region; every launch reads a different copy of its weight matrix so
+that the stream comes from HBM and not from the 256 MiB Infinity Cache ("cold").  The step
+is replayed from a HIP graph so that host launch cost does not pace microsecond kernels.
+
+value  = algorithmic bytes of all GEMMs / wall time      (GB/s, higher is better)
+roofline.achieved = mean algorithmic bytes per launch / mean launch duration, HIP events
+                    on the launch stream, against the 8 TB/s HBM3E peak.
+cpu_baseline = the same GEMMs (bounded sample) through the CPU oracle's restatement of the
+               reference CPU path (numpy quantiser/packer output + torch CPU int matmul).
+Activation quantisation is timed separately (detail.act_quant).  detail also carries the
+per-shape cold/warm table, the prefill (int8-MFMA-bound) TOPS of the tiled kernel and a
+plain streaming-read calibration.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published
+INT8_PEAK_TOPS = 5000.0       # MI355X dense int8 MFMA, published (5.0 POP/s)
+COLD_FOOTPRINT = 640 << 20    # bytes of distinct weight copies between two uses of one copy
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this command, scaled by what the same counters read for the read-probe kernel of known size.
+# None until measured.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=40)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--skip-detail", action="store_true", help="only the headline line (no per-shape table, prefill, CPU baseline)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (the W2A8 path has no multi-GPU part); "
+              f"--gpus {args.gpus} is not supported", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from slimkernels_amd import torch as ops   # raises if the HIP library is missing: no fallback
+    from slimkernels_amd import _lib, workloads
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L = _lib.lib()
+
+    # ------------------------------------------------------------------ inputs (resident in HBM)
+    def n_copies(nbytes, uses_per_cycle):
+        return max(uses_per_cycle, -(-COLD_FOOTPRINT // nbytes))
+
+    class Shape:
+        pass
+
+    cases = workloads.config_cases("c2")
+    shapes = {}
+    for name, (N, K) in workloads.LLAMA8B_LINEARS.items():
+        sh = Shape()
+        sh.name, sh.N, sh.K = name, N, K
+        c0 = workloads.Case("c2", 1, N, K, outliers=True)
+        packed, scales, zero = workloads.make_quantized_weight(c0)
+        base = ops.repack_w2(packed, scales, None, 128, zp_const=2)
+        sh.base = base
+        sh.host = (packed, scales, zero)
+        sh.copies = [base]
+        shapes[name] = sh
+    total_w = sum(s.base.w_r.numel() * 4 + s.base.s_r.numel() * 2 for s in shapes.values())
+    # every launch of a step cycle uses the next copy; one copy is reused only after all copies of
+    # all shapes have been streamed (>= COLD_FOOTPRINT of other traffic in between)
+    for sh in shapes.values():
+        nb = sh.base.w_r.numel() * 4 + sh.base.s_r.numel() * 2
+        want = n_copies(nb, len(workloads.DECODE_M))
+        for _ in range(want - 1):
+            sh.copies.append(ops.W2A8Weight(sh.base.w_r.clone(), sh.base.s_r.clone(), None, 2, sh.N, sh.K, 128))
+        sh.next = 0
+
+    acts = {}
+    for c in cases:
+        x = torch.from_numpy(workloads.make_activation(c)).to(dev)
+        qa = ops.quantize_act_int8(x, 128)
+        out = torch.empty((c.M, c.N), dtype=torch.float16, device=dev)
+        acts[(c.N, c.K, c.M)] = (x, qa, out)
+    name_of = {(N, K): n for n, (N, K) in workloads.LLAMA8B_LINEARS.items()}
+
+    def launch_step(warm=False):
+        for c in cases:
+            sh = shapes[name_of[(c.N, c.K)]]
+            w = sh.copies[0] if warm else sh.copies[sh.next % len(sh.copies)]
+            if not warm:
+                sh.next += 1
+            _, qa, out = acts[(c.N, c.K, c.M)]
+            ops.w2a8_gemm(qa, w, torch.float16, out=out)
+
+    # touch every copy once eagerly: creates and zeroes the split-K workspaces outside any capture
+    for sh in shapes.values():
+        for w in sh.copies:
+            _, qa, out = acts[(sh.N, sh.K, 16)]
+            ops.w2a8_gemm(qa, w, torch.float16, out=out)
+    torch.cuda.synchronize()
+
+    def capture(n_steps, warm=False):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(n_steps):
+                launch_step(warm)
+        return g
+
+    # ------------------------------------------------------------------ timed region
+    UNROLL = 8
+    graphs = {}
+
+    def run_steps(k):
+        full, rem = divmod(k, UNROLL)
+        if full and UNROLL not in graphs:
+            graphs[UNROLL] = capture(UNROLL)
+        if rem and rem not in graphs:
+            graphs[rem] = capture(rem)
+        return full, rem
+
+    full_w, rem_w = run_steps(args.warmup)
+    full_k, rem_k = run_steps(args.steps)
+    torch.cuda.synchronize()
+    for _ in range(full_w):
+        graphs[UNROLL].replay()
+    if rem_w:
+        graphs[rem_w].replay()
+    torch.cuda.synchronize()
+
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(full_k):
+        graphs[UNROLL].replay()
+    if rem_k:
+        graphs[rem_k].replay()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ev_ms = e0.elapsed_time(e1)
+
+    step_bytes = sum(workloads.algorithmic_bytes(c) for c in cases)
+    step_ops = sum(workloads.algorithmic_ops(c) for c in cases)
+    launches = len(cases) * args.steps
+    ms_per_step = wall * 1e3 / args.steps
+    value = step_bytes * args.steps / wall / 1e9
+    avg_launch_us = ev_ms * 1e3 / launches
+    achieved = (step_bytes / len(cases)) / (avg_launch_us * 1e-6) / 1e9
+
+    result = {
+        "metric": "W2A8 GEMM TOPS + HBM GB/s (% roofline) at M=1..4096, 1 MI355X",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "c2 decode sweep: M in {1,2,4,8,16,32} x Llama-3-8B linears "
+                               "(4096x4096, 1024x4096, 14336x4096, 4096x14336), W2 sym g128, A8 per-token, "
+                               "fp16 out; 24 skinny split-K GEMM launches per step, cold HBM (rotating weight copies)",
+                   "launches_per_step": len(cases), "algorithmic_bytes_per_step": step_bytes,
+                   "ops_per_step": step_ops, "timing": "HIP graph replay, inputs resident in HBM"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
+                     "kernel": "w2a8::skinny_kernel", "avg_launch_us": round(avg_launch_us, 3),
+                     "algorithmic_bytes_per_launch": step_bytes // len(cases)},
+    }
+
+    detail = {"tops_decode": round(step_ops * args.steps / wall / 1e12, 3)}
+    if not args.skip_detail:
+        detail.update(collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, dev))
+        result["cpu_baseline"] = cpu_baseline(np, workloads, shapes)
+    else:
+        result["cpu_baseline"] = None
+    result["detail"] = detail
+    print(json.dumps(result))
+
+
+def _lib_check(rc):
+    from slimkernels_amd import _lib
+    _lib.check(rc)
+
+
+def time_graph(torch, fn, launches_in_graph, replays=6):
+    """Mean microseconds per launch of `fn` (which enqueues `launches_in_graph` launches)."""
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (replays * launches_in_graph)
+
+
+def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, dev):
+    detail = {}
+    # ---- streaming-read calibration: what a plain 16-byte-per-lane read kernel reaches on this box
+    buf = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    buf.zero_()
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+
+    def probe():
+        st = torch.cuda.current_stream().cuda_stream  # the capture stream while a graph records
+        for _ in range(4):
+            _lib_check(L.slimk_w2a8_read_probe(buf.data_ptr(), buf.numel(), sink.data_ptr(), st))
+    us = time_graph(torch, probe, 4)
+    detail["read_probe_GBps_1GiB"] = round(buf.numel() / (us * 1e-6) / 1e9, 1)
+    del buf
+
+    # ---- per-(shape, M) decode table, cold (rotating copies) and warm (one copy, cache resident)
+    table = []
+    for c in cases:
+        sh = shapes[name_of[(c.N, c.K)]]
+        _, qa, out = acts[(c.N, c.K, c.M)]
+        nb = workloads.algorithmic_bytes(c)
+        row = {"shape": f"{c.N}x{c.K}", "M": c.M, "bytes": nb,
+               "split_k": L.slimk_w2a8_gemm_auto_split_k(c.M, c.N, c.K, 128, 0)}
+        for label, ws in (("cold", sh.copies), ("warm", sh.copies[:1] * 16)):
+            def fn(ws=ws):
+                for w in ws:
+                    ops.w2a8_gemm(qa, w, torch.float16, out=out)
+            us = time_graph(torch, fn, len(ws), replays=3 if label == "cold" else 10)
+            row[f"{label}_us"] = round(us, 2)
+            row[f"{label}_GBps"] = round(nb / (us * 1e-6) / 1e9, 1)
+        row["cold_frac_hbm"] = round(row["cold_GBps"] / HBM_PEAK_GBPS, 4)
+        table.append(row)
+    detail["decode"] = table
+
+    # ---- activation quantisation, timed on its own (bytes: 2MK read + MK + 4M + 4MG written)
+    aq = []
+    for (N, K, M) in ((4096, 4096, 1), (4096, 4096, 32), (4096, 14336, 32)):
+        x, _, _ = acts[(N, K, M)]
+        us = time_graph(torch, lambda: [ops.quantize_act_int8(x, 128) for _ in range(8)], 8)
+        aq.append({"M": M, "K": K, "us": round(us, 2), "GBps": round((3 * M * K + 4 * M + 4 * M * (K // 128)) / (us * 1e-6) / 1e9, 1)})
+    detail["act_quant"] = aq
+
+    # ---- prefill regime (c3): tiled int8-MFMA kernel
+    pre = []
+    for (N, K) in ((14336, 4096), (4096, 14336)):
+        w = shapes[name_of[(N, K)]].base
+        for M in (512, 2048, 4096):
+            c = workloads.Case("c3", M, N, K)
+            x = torch.from_numpy(workloads.make_activation(c)).to(dev)
+            qa = ops.quantize_act_int8(x, 128)
+            out = torch.empty((M, N), dtype=torch.float16, device=dev)
+            ops.w2a8_gemm(qa, w, torch.float16, out=out)
+            us = time_graph(torch, lambda: [ops.w2a8_gemm(qa, w, torch.float16, out=out) for _ in range(4)], 4)
+            tops = workloads.algorithmic_ops(c) / (us * 1e-6) / 1e12
+            pre.append({"shape": f"{N}x{K}", "M": M, "us": round(us, 1), "TOPS": round(tops, 1),
+                        "frac_int8_mfma": round(tops / INT8_PEAK_TOPS, 4)})
+    detail["prefill"] = pre
+    return detail
+
+
+def cpu_baseline(np, workloads, shapes):
+    """The reference CPU path on a bounded sample of the same workload: the four Llama linears at
+    M in {1, 16, 32}, through the oracle's torch-CPU-int-matmul restatement, on this box's host cores."""
+    import torch
+    from oracle import w2a8_oracle as orc
+    torch.set_num_threads(min(16, os.cpu_count() or 1))
+    tot_bytes, tot_s, c_port_s = 0, 0.0, 0.0
+    for name, M in [(n, m) for n in workloads.LLAMA8B_LINEARS for m in (1, 16, 32)]:
+        N, K = workloads.LLAMA8B_LINEARS[name]
+        c = workloads.Case("c2", M, N, K, outliers=True)
+        packed, scales, zero = shapes[name].host
+        x = workloads.make_activation(c)
+        t0 = time.perf_counter()
+        orc.torch_reference_forward(x, packed, scales, zero, 128)
+        tot_s += time.perf_counter() - t0
+        q, s_a, _ = orc.c_act_quant(x, 128)
+        t0 = time.perf_counter()
+        orc.c_gemm_fused(q, s_a, packed, scales, zero, 128)
+        c_port_s += time.perf_counter() - t0
+        tot_bytes += workloads.algorithmic_bytes(c)
+    return {"value": round(tot_bytes / tot_s / 1e9, 4), "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": "the four c2 shapes at M in {1,16,32} once each (act-quant + unpack + torch CPU int32 matmul per group + "
+                      "fp32 epilogue); algorithmic bytes / wall seconds",
+            "seconds": round(tot_s, 3), "host_cpus": os.cpu_count(),
+            "scalar_c_port_1core_GBps": round(tot_bytes / c_port_s / 1e9, 4)}
+
+
+if __name__ == "__main__":
+    main()

@@ -134,7 +134,8 @@ int slimk_w2a8_act_quant(const void* x, int ldx, int x_dtype, int M, int K, int 
  *                              instantiations so the timed kernels carry no extra code.
  *   workspace                : required when the effective split_k > 1
  *                              (slimk_w2a8_gemm_workspace_bytes), else may be NULL
- *   kernel, split_k          : SLIMK_KERNEL_* and the split-K factor; 0 = choose */
+ *   kernel, split_k          : SLIMK_KERNEL_* and the split-K factor; 0 = choose.  split_k is an upper
+ *                              bound: a split owns whole 256-element chunks of K, so fewer may be used */
 int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,
                     const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
                     int M, int N, int K, int group_size,

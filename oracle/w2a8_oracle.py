@@ -285,3 +285,23 @@ def reference_forward(x_half: np.ndarray, packed: np.ndarray, scale_half: np.nda
         acc, out_f32 = None, None
         out_bits, _ = c_gemm_fused(q, s_a, packed, scale_half, zp, group_size, out_bf16)
     return dict(q=q, s_a=s_a, rowsum=rs, acc=acc, out_bits=out_bits, out_f32=out_f32)
+
+
+def torch_reference_forward(x_half: np.ndarray, packed: np.ndarray, scale_half: np.ndarray, zp: np.ndarray,
+                            group_size: int, out_bf16: bool = False):
+    """The CPU path as the task statement words it: numpy quantiser/packer output fed to a
+    torch CPU integer matmul, then the float epilogue.  Used for the timed CPU baseline; its
+    result agrees with c_gemm_acc exactly (int32) and with c_epilogue to float32 rounding
+    (the group sum here is a plain torch sum, not the fused chain)."""
+    import torch
+    q, s_a, _ = np_act_quant(x_half, group_size)
+    M, K = q.shape
+    N = packed.shape[0]
+    G = K // group_size
+    codes = torch.from_numpy(np_unpack(packed)).to(torch.int32).reshape(N, G, group_size)
+    w = codes - torch.from_numpy(np.ascontiguousarray(zp.T)).to(torch.int32)[:, :, None]
+    acc = torch.einsum("mgk,ngk->mng", torch.from_numpy(q).to(torch.int32).reshape(M, G, group_size), w)
+    s = torch.from_numpy(np.ascontiguousarray(np.asarray(scale_half, np.float16).T)).to(torch.float32)  # [N, G]
+    t = (acc.to(torch.float32) * s[None]).sum(dim=2) * torch.from_numpy(s_a)[:, None]
+    out = t.to(torch.bfloat16 if out_bf16 else torch.float16)
+    return acc.numpy(), out

@@ -2,6 +2,7 @@
 // the host, kernel selection, launches.  No allocation, no synchronisation.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 
 #include <string>
 
@@ -59,22 +60,49 @@ int resolve_kernel(int M, int kernel) {
     return kernel;
 }
 
-// Split-K heuristic of the skinny kernel: enough workgroups to cover the 256 CUs about
-// twice, while every wave of a workgroup keeps at least one scale group.
+// The skinny kernel partitions K in chunks of four 64-element steps; a split owns whole chunks.
+int chunk_groups(int group_size) { return group_size >= 256 ? 1 : 256 / group_size; }
+
+// Groups per split for a requested split factor, rounded up to whole chunks; the effective split
+// (number of non-empty splits) is ceil(G / groups_per_split) <= requested.
+int groups_per_split(int G, int group_size, int split) {
+    const int cg = chunk_groups(group_size);
+    int gps = (G + split - 1) / split;
+    return (gps + cg - 1) / cg * cg;
+}
+
+// Split-K heuristic of the skinny kernel (measured on MI355X, cold weights).  One workgroup per
+// 64-channel strip already covers the chip when there are >= 192 strips, and a matrix of a few
+// MiB is latency-bound whatever is done, so both run unsplit: the cross-workgroup reduction
+// costs about 3 us.  Only a large matrix with few strips (small N, long K) is split, up to about
+// 256 workgroups, because a quarter of the CUs cannot pull full HBM bandwidth.
 int auto_split(int M, int N, int K, int group_size, int kernel) {
     (void)M;
     if (kernel != SLIMK_KERNEL_SKINNY) return 1;
     const int strips = strips_of(N);
     const int G = K / group_size;
-    int split = (512 + strips - 1) / strips;
-    const int max_split = G / 4 > 0 ? G / 4 : 1;
+    const int chunks = (K / 64 + 3) / 4;
+    const size_t weight_bytes = (size_t)strips * 64 * (K / 4);
+    int split = 1;
+    if (strips < 192 && weight_bytes > (size_t)6 << 20) split = (256 + strips - 1) / strips;
+    const int max_split = chunks / 4 > 0 ? chunks / 4 : 1;
     if (split > max_split) split = max_split;
     if (split > 32) split = 32;
-    if (split < 1) split = 1;
-    // drop splits that would be empty: ceil(G / split) groups each
-    const int gps = (G + split - 1) / split;
-    split = (G + gps - 1) / gps;
-    return split;
+    const int gps = groups_per_split(G, group_size, split);
+    return (G + gps - 1) / gps;
+}
+
+// Wavefronts per workgroup of the skinny kernel (the in-workgroup split of K).
+// SLIMK_W2A8_SKINNY_WAVES overrides the choice (read once; a tuning aid, not an interface).
+int skinny_waves(int M, int split) {
+    static const int forced = [] {
+        const char* e = getenv("SLIMK_W2A8_SKINNY_WAVES");
+        return e ? atoi(e) : 0;
+    }();
+    if (forced) return forced;
+    // split runs are the long-K ones: more waves per workgroup keep more loads in flight per CU
+    if (split > 1) return M <= 16 ? 16 : 8;
+    return 4;
 }
 
 }  // namespace
@@ -184,9 +212,8 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
     if (kern == SLIMK_KERNEL_TILED && split_k != 1)
         return fail(SLIMK_ERR_UNSUPPORTED, "the tiled kernel has no split-K (split_k=%d)", split_k);
     if (split_k > G) return fail(SLIMK_ERR_BAD_SHAPE, "split_k=%d exceeds the number of groups %d", split_k, G);
-    const int gps = (G + split_k - 1) / split_k;
-    if ((G + gps - 1) / gps != split_k)
-        return fail(SLIMK_ERR_BAD_SHAPE, "split_k=%d leaves empty splits for %d groups", split_k, G);
+    const int gps = groups_per_split(G, group_size, split_k);
+    split_k = (G + gps - 1) / gps;  // effective split: the request is an upper bound (whole chunks per split)
 
     w2a8::GemmParams p{};
     p.q = q; p.s_a = s_a; p.rowsum = rowsum; p.w_r = w_r; p.s_r = s_r; p.zp_r = zp_r;
@@ -213,7 +240,8 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
     const int gs = group_size / w2a8::kStepK;
     const bool asym = zp_r != nullptr;
     const bool out_bf16 = out_dtype == SLIMK_BF16;
-    if (kern == SLIMK_KERNEL_SKINNY) return hip_result(w2a8::launch_skinny(p, gs, asym, out_bf16, st), "skinny gemm");
+    if (kern == SLIMK_KERNEL_SKINNY)
+        return hip_result(w2a8::launch_skinny(p, gs, skinny_waves(M, split_k), asym, out_bf16, st), "skinny gemm");
     return hip_result(w2a8::launch_tiled(p, gs, asym, out_bf16, st), "tiled gemm");
 }
 

@@ -51,7 +51,8 @@ __global__ __launch_bounds__(256) void tiled_kernel(const GemmParams p) {
     }
     const int b_strip = strip0 + (wave & 1);
     const bool b_ok = b_strip < p.strips;
-    const uint32_t* b_src = p.w_r + ((size_t)(b_ok ? b_strip : 0) * p.steps + (wave >> 1)) * kUnitDwords + lane * 4;
+    const uint32_t* b_src = p.w_r + ((size_t)(wave >> 1) * p.strips + (b_ok ? b_strip : 0)) * kUnitDwords + lane * 4;
+    const size_t b_step_stride = (size_t)p.strips * kUnitDwords;  // dwords between consecutive steps of a strip
 
     auto fetch = [&](int stage) {
         const int step0 = stage * kStageSteps;
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(256) void tiled_kernel(const GemmParams p) {
         }
         const int bstep = step0 + (wave >> 1);
         gb = v4i{0, 0, 0, 0};
-        if (b_ok && bstep < p.steps) gb = *reinterpret_cast<const v4i*>(b_src + (size_t)step0 * kUnitDwords);
+        if (b_ok && bstep < p.steps) gb = *reinterpret_cast<const v4i*>(b_src + (size_t)step0 * b_step_stride);
     };
     auto stash = [&](int buf) {
 #pragma unroll
@@ -83,13 +84,13 @@ __global__ __launch_bounds__(256) void tiled_kernel(const GemmParams p) {
             for (int j = 0; j < 4; ++j) t[mb][pp][j] = 0.0f;
         }
 
-    const size_t sg_base = (size_t)(strip_ok ? strip : 0) * p.G;
+    const size_t sg_strip = (size_t)(strip_ok ? strip : 0);
     const int m_wave = m_tile + wm * 64;  // first token row of this wave
 
     auto group_begin = [&](int g) {
         int zpe[4];
         if (ASYM) {
-            const uint32_t zraw = *reinterpret_cast<const uint32_t*>(p.zp_r + ((sg_base + g) * 16 + col) * 4);
+            const uint32_t zraw = *reinterpret_cast<const uint32_t*>(p.zp_r + (((size_t)g * p.strips + sg_strip) * 16 + col) * 4);
             zpe[0] = (int)(zraw & 0xffu);
             zpe[1] = (int)((zraw >> 8) & 0xffu) * 4;
             zpe[2] = (int)((zraw >> 16) & 0xffu) * 16;
@@ -110,7 +111,7 @@ __global__ __launch_bounds__(256) void tiled_kernel(const GemmParams p) {
         }
     };
     auto group_end = [&](int g) {
-        const uint2 sraw = *reinterpret_cast<const uint2*>(p.s_r + ((sg_base + g) * 16 + col) * 4);
+        const uint2 sraw = *reinterpret_cast<const uint2*>(p.s_r + (((size_t)g * p.strips + sg_strip) * 16 + col) * 4);
         float sc[4];
         sc[0] = half_bits_to_float((uint16_t)(sraw.x & 0xffffu));
         sc[1] = half_bits_to_float((uint16_t)(sraw.x >> 16)) * 0.25f;

@@ -8,15 +8,15 @@ namespace w2a8 {
 // interchange layout (matrix_packer.py:33-34: byte j of row n holds k = 4j..4j+3,
 // k = 4j in bits 7:6).  See w2a8_common.h for the target layout.
 __global__ __launch_bounds__(256) void repack_codes_kernel(const uint8_t* __restrict__ w_packed, int ldw,
-                                                           int N, int steps, size_t total_dwords,
+                                                           int N, int strips, size_t total_dwords,
                                                            uint32_t* __restrict__ w_r) {
     size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total_dwords) return;
     const int i = (int)(idx & 3);
     const int lane = (int)((idx >> 2) & 63);
     const size_t unit = idx >> 8;
-    const int step = (int)(unit % (size_t)steps);
-    const int strip = (int)(unit / (size_t)steps);
+    const int strip = (int)(unit % (size_t)strips);
+    const int step = (int)(unit / (size_t)strips);
     const int col = lane & 15, quad = lane >> 4;
     const int src_byte = step * 16 + quad * 4 + i;  // (step*64 + quad*16 + 4*i) / 4
     uint32_t out = 0;
@@ -34,9 +34,9 @@ __global__ __launch_bounds__(256) void repack_codes_kernel(const uint8_t* __rest
     w_r[idx] = out;
 }
 
-// scales [G][N] fp16 -> s_r [strips][G][16][4]; zero-points likewise (one byte each).
+// scales [G][N] fp16 -> s_r [G][strips][16][4]; zero-points likewise (one byte each).
 __global__ __launch_bounds__(256) void repack_scales_kernel(const uint16_t* __restrict__ scales,
-                                                            const uint8_t* __restrict__ zp, int N, int G,
+                                                            const uint8_t* __restrict__ zp, int N, int strips,
                                                             size_t total, uint16_t* __restrict__ s_r,
                                                             uint8_t* __restrict__ zp_r) {
     size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -44,8 +44,8 @@ __global__ __launch_bounds__(256) void repack_scales_kernel(const uint16_t* __re
     const int p = (int)(idx & 3);
     const int col = (int)((idx >> 2) & 15);
     const size_t sg = idx >> 6;
-    const int g = (int)(sg % (size_t)G);
-    const int strip = (int)(sg / (size_t)G);
+    const int strip = (int)(sg % (size_t)strips);
+    const int g = (int)(sg / (size_t)strips);
     const int n = strip * kStripN + p * 16 + col;
     s_r[idx] = (n < N) ? scales[(size_t)g * N + n] : (uint16_t)0;
     if (zp_r) zp_r[idx] = (n < N) ? zp[(size_t)g * N + n] : (uint8_t)0;
@@ -59,10 +59,10 @@ hipError_t launch_repack(const uint8_t* w_packed, int ldw, const uint16_t* scale
     const int G = K / group_size;
     const size_t total = (size_t)strips * steps * kUnitDwords;
     repack_codes_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream>>>(
-        w_packed, ldw, N, steps, total, w_r);
+        w_packed, ldw, N, strips, total, w_r);
     const size_t stotal = (size_t)strips * G * 64;
     repack_scales_kernel<<<dim3((unsigned)((stotal + 255) / 256)), dim3(256), 0, stream>>>(
-        scales, zp, N, G, stotal, s_r, zp ? zp_r : nullptr);
+        scales, zp, N, strips, stotal, s_r, zp ? zp_r : nullptr);
     return hipGetLastError();
 }
 

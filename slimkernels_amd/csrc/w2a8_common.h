@@ -8,7 +8,10 @@
 // so that lane l of a wavefront reads its 16 bytes at offset 16*l (one coalesced
 // global_load_dwordx4 / one conflict-free ds_read_b128 per wave and unit).
 //
-//   unit address   = w_r + ((strip * steps + step) * 64 + lane) * 4      [dwords]
+//   unit address   = w_r + ((step * strips + strip) * 64 + lane) * 4     [dwords]
+//   (step-major: the units that all strips need at the same moment are contiguous, so the
+//    chip reads one sequential band per step instead of `strips` power-of-two-strided
+//    streams that pile onto a few HBM channels)
 //   lane l         : col = l & 15, quad = l >> 4
 //   dword i, byte b, 2-bit field p of that byte (bits 2p+1:2p) holds the code of
 //       n = strip*64 + p*16 + col          k = step*64 + quad*16 + 4*i + b
@@ -20,8 +23,9 @@
 // the byte then reads as 64 * (code - 2).  The 4^p factor is divided out of the
 // fp32 scale (exact, a power of two) and the "-2" moves into the zero-point.
 //
-// Scales and zero-points are stored per (strip, group) as [16 cols][4 sub-blocks]
-// so that a lane fetches the four values it needs with one 8-byte (4-byte) load.
+// Scales and zero-points are stored per (group, strip) as [16 cols][4 sub-blocks]
+// (index (group * strips + strip) * 64 + col * 4 + p) so that a lane fetches the four
+// values it needs with one 8-byte (4-byte) load.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -39,8 +43,8 @@ struct GemmParams {
     const float* s_a;       // [M]
     const int32_t* rowsum;  // [G][ldr]
     const uint32_t* w_r;    // repacked codes
-    const uint16_t* s_r;    // [strips][G][16][4] fp16 bits
-    const uint8_t* zp_r;    // [strips][G][16][4] or nullptr
+    const uint16_t* s_r;    // [G][strips][16][4] fp16 bits
+    const uint8_t* zp_r;    // [G][strips][16][4] or nullptr
     void* out;              // [M][ldo] fp16 / bf16 bits
     int32_t* acc_dump;      // verification output or nullptr
     float* ws_partial;      // split-K partial tiles

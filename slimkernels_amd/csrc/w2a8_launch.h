@@ -20,8 +20,8 @@ hipError_t launch_fill_zero(void* p, size_t bytes, hipStream_t stream);
 
 hipError_t launch_read_probe(const void* src, size_t bytes, uint32_t* sink, hipStream_t stream);
 
-// m_blocks = 1 (M <= 16) or 2 (M <= 32); gs = 64-element steps per scale group (1, 2 or 4)
-hipError_t launch_skinny(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
+// gs = 64-element steps per scale group (1, 2 or 4); waves = wavefronts per workgroup (4, 8, 16)
+hipError_t launch_skinny(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, hipStream_t stream);
 
 hipError_t launch_tiled(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
 

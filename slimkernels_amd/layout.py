@@ -6,8 +6,9 @@ repacked buffer can be turned back into the interchange format (``unrepack_codes
 e.g. when persisting weights.  Nothing here is used by the GEMM.
 
 Layout: the [N, K] code matrix is cut into units of 64 channels (strip) x 64 reduction
-elements (step); unit (strip, step) is 64 lanes x 4 dwords at dword offset
-((strip * steps + step) * 64 + lane) * 4.  With col = lane & 15, quad = lane >> 4, the
+elements (step); unit (step, strip) is 64 lanes x 4 dwords at dword offset
+((step * strips + strip) * 64 + lane) * 4 (step-major, so that what all strips read at
+the same time is one contiguous band).  With col = lane & 15, quad = lane >> 4, the
 2-bit field p (bits 2p+1:2p) of byte b of dword i holds the code of
 
     n = strip*64 + p*16 + col        k = step*64 + quad*16 + 4*i + b
@@ -22,7 +23,7 @@ STEP_K = 64
 
 
 def repack_codes(packed: np.ndarray) -> np.ndarray:
-    """uint8 [N, K/4] interchange bytes -> uint32 [strips, steps, 64, 4] streaming layout."""
+    """uint8 [N, K/4] interchange bytes -> uint32 [steps, strips, 64, 4] streaming layout."""
     packed = np.asarray(packed, np.uint8)
     N, K = packed.shape[0], packed.shape[1] * 4
     if K % STEP_K:
@@ -40,13 +41,13 @@ def repack_codes(packed: np.ndarray) -> np.ndarray:
         for b in range(4):
             # c[:, p, :, :, :, :, b] has axes strip, col, step, quad, i
             out |= c[:, p, :, :, :, :, b].transpose(0, 2, 3, 1, 4) << np.uint32(8 * b + 2 * p)
-    return out.reshape(strips, steps, 64, 4)
+    return np.ascontiguousarray(out.reshape(strips, steps, 64, 4).transpose(1, 0, 2, 3))
 
 
 def unrepack_codes(w_r: np.ndarray, N: int, K: int) -> np.ndarray:
     """Inverse of :func:`repack_codes`: streaming layout -> uint8 [N, K/4] interchange bytes."""
     strips, steps = -(-N // STRIP_N), K // STEP_K
-    w = np.asarray(w_r, np.uint32).reshape(strips, steps, 4, 16, 4)  # strip, step, quad, col, i
+    w = np.asarray(w_r, np.uint32).reshape(steps, strips, 4, 16, 4).transpose(1, 0, 2, 3, 4)  # strip, step, quad, col, i
     codes = np.zeros((strips, 4, 16, steps, 4, 4, 4), np.uint8)       # strip, p, col, step, quad, i, b
     for p in range(4):
         for b in range(4):
@@ -60,11 +61,11 @@ def unrepack_codes(w_r: np.ndarray, N: int, K: int) -> np.ndarray:
 
 
 def repack_group_values(values_gn: np.ndarray) -> np.ndarray:
-    """[G, N] per-(group, channel) values (scales or zero-points) -> [strips, G, 16, 4]
-    (strip, group, col, sub-block p), zero-filled past N."""
+    """[G, N] per-(group, channel) values (scales or zero-points) -> [G, strips, 16, 4]
+    (group, strip, col, sub-block p), zero-filled past N."""
     v = np.asarray(values_gn)
     G, N = v.shape
     strips = -(-N // STRIP_N)
     full = np.zeros((G, strips * STRIP_N), v.dtype)
     full[:, :N] = v
-    return np.ascontiguousarray(full.reshape(G, strips, 4, 16).transpose(1, 0, 3, 2))
+    return np.ascontiguousarray(full.reshape(G, strips, 4, 16).transpose(0, 1, 3, 2))

@@ -36,10 +36,10 @@ def wave_strip_groups(q, rowsum, w_r, s_r, zp_r, zp_const, strip, groups, gs, M)
     t = np.zeros((64, 4, 4), np.float32)  # lane, p, j
     acc_out = np.zeros((16, 64, len(groups)), np.int32)
     for gi, g in enumerate(groups):
-        sraw = s_r[strip, g][col]                         # [64, 4] fp16 (lane, p)
+        sraw = s_r[g, strip][col]                         # [64, 4] fp16 (lane, p)
         sc = sraw.astype(np.float32) * np.array([1, 0.25, 0.0625, 0.015625], np.float32)
         if zp_r is not None:
-            z = zp_r[strip, g][col].astype(np.int32)
+            z = zp_r[g, strip][col].astype(np.int32)
         else:
             z = np.full((64, 4), zp_const, np.int32)
         zpe = np.stack([z[:, 0], z[:, 1] * 4, z[:, 2] * 16, (z[:, 3] - 2) * 64], axis=1)
@@ -51,7 +51,7 @@ def wave_strip_groups(q, rowsum, w_r, s_r, zp_r, zp_const, strip, groups, gs, M)
                 acc[l, p] = -zpe[l, p] * rs
         for s in range(gs):
             step = g * gs + s
-            w = w_r[strip, step]                          # uint32 [64, 4]
+            w = w_r[step, strip]                          # uint32 [64, 4]
             a = np.zeros((64, 16), np.int8)
             for l in range(64):
                 m = col[l]

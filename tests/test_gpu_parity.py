@@ -27,12 +27,12 @@ def test_repack_matches_layout_definition(gpu_ops, N, K, g, with_zp):
     zp = rng.integers(0, 4, (K // g, N), dtype=np.uint8) if with_zp else None
     w = gpu_ops.repack_w2(packed, scales, zp, g)
     strips, steps = -(-N // 64), K // 64
-    got = w.w_r.cpu().numpy().view(np.uint32).reshape(strips, steps, 64, 4)
+    got = w.w_r.cpu().numpy().view(np.uint32).reshape(steps, strips, 64, 4)
     np.testing.assert_array_equal(got, layout.repack_codes(packed))
     np.testing.assert_array_equal(layout.unrepack_codes(got, N, K), packed)
-    np.testing.assert_array_equal(w.s_r.cpu().numpy().reshape(strips, K // g, 16, 4), layout.repack_group_values(scales))
+    np.testing.assert_array_equal(w.s_r.cpu().numpy().reshape(K // g, strips, 16, 4), layout.repack_group_values(scales))
     if with_zp:
-        np.testing.assert_array_equal(w.zp_r.cpu().numpy().reshape(strips, K // g, 16, 4), layout.repack_group_values(zp))
+        np.testing.assert_array_equal(w.zp_r.cpu().numpy().reshape(K // g, strips, 16, 4), layout.repack_group_values(zp))
 
 
 # ------------------------------------------------------------------ activation quantisation

@@ -11,7 +11,7 @@ def test_repack_roundtrip(N, K):
     rng = np.random.default_rng(N * 1000 + K)
     packed = rng.integers(0, 256, (N, K // 4), dtype=np.uint8)
     w_r = layout.repack_codes(packed)
-    assert w_r.shape == (-(-N // 64), K // 64, 64, 4)
+    assert w_r.shape == (K // 64, -(-N // 64), 64, 4)
     np.testing.assert_array_equal(layout.unrepack_codes(w_r, N, K), packed)
 
 
@@ -27,18 +27,18 @@ def test_repack_field_definition():
         n, k = int(rng.integers(N)), int(rng.integers(K))
         strip, p, col = n // 64, (n % 64) // 16, n % 16
         step, quad, i, b = k // 64, (k % 64) // 16, (k % 16) // 4, k % 4
-        f = (int(w_r[strip, step, quad * 16 + col, i]) >> (8 * b + 2 * p)) & 3
+        f = (int(w_r[step, strip, quad * 16 + col, i]) >> (8 * b + 2 * p)) & 3
         assert (f ^ 2 if p == 3 else f) == codes[n, k]
 
 
 def test_group_value_layout():
     v = np.arange(3 * 70, dtype=np.float16).reshape(3, 70)
     r = layout.repack_group_values(v)
-    assert r.shape == (2, 3, 16, 4)
+    assert r.shape == (3, 2, 16, 4)
     for n in (0, 15, 16, 63, 64, 69):
         for g in range(3):
-            assert r[n // 64, g, n % 16, (n % 64) // 16] == v[g, n]
-    assert r[1, 0, 6, 0] == 0  # n = 70 is padding
+            assert r[g, n // 64, n % 16, (n % 64) // 16] == v[g, n]
+    assert r[0, 1, 6, 0] == 0  # n = 70 is padding
 
 
 @pytest.mark.parametrize("mode,gs", [("sym", 2), ("asym", 1), ("asym", 2)])
