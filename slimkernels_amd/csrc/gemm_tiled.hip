@@ -1,180 +1,217 @@
-// Tiled W2A8 GEMM for gfx950 (any M; the int8-MFMA-bound prefill regime).
+// Fast tiled W2A8 GEMM for gfx950: the int8-MFMA-bound prefill regime, uniform zero-point 2
+// (the symmetric levels {-2..1}), group size 64 or 128, K a multiple of 128.
 //
-// Workgroup = 4 wavefronts as 2 (tokens) x 2 (channels); workgroup tile 128 tokens x
-// 128 channels (two weight strips); wave tile 64 x 64 = 4 x 4 MFMA blocks of
-// v_mfma_i32_16x16x64_i8.  The reduction runs in stages of two 64-element steps.
-// Both operands are staged in LDS in MFMA-operand order: every 16-row x 64-k
-// activation block and every weight unit is 1 KiB laid out lane-major, so each
-// fragment read is one ds_read_b128 per lane at offset 16*lane (conflict-free by
-// construction) and every global->LDS transfer is a 16-byte-per-lane copy.  Two LDS
-// buffers: the next stage is fetched into registers while the current one is
-// multiplied, then written to the other buffer; one barrier per stage.
-// At each scale-group boundary the int32 accumulators are folded into fp32 running
-// sums (v_cvt_f32_i32 + v_fma_f32 per element) and restarted at -zp * rowsum.
+// Workgroup = 4 wavefronts side by side along the channels; workgroup tile 128 tokens x 256
+// channels (four weight strips); wave tile 128 x 64 = 8 x 4 blocks of v_mfma_i32_16x16x64_i8.
+// A wide-in-N tile is the cheap one here: per reduction element a tile fetches BM bytes of
+// activations but only BN/4 bytes of 2-bit weights.
+//
+// What bounds the kernel is the vector ALU next to the matrix core, not the matrix core: every
+// accumulator must be drained into an fp32 running sum once per scale group (v_cvt_f32_i32 +
+// v_fma_f32 per element per group -- at group 128 that is as many VALU cycles as MFMA cycles).
+// Everything else is arranged to add as little VALU work as possible:
+//  * the high bit of every 2-bit field is flipped (one v_xor per dword) and the field moved to
+//    the top of its byte (v_lshlrev + v_and), so each operand byte reads as 64 * (code - 2):
+//    the zero-point is gone before the MFMA and no row-sum term is needed; the factor 64 is
+//    divided out of the fp32 scale;
+//  * the unpacked weight operand of a wave (one strip) is reused by its eight token blocks;
+//  * activations sit in LDS in MFMA-operand order (1 KiB per 16-row x 64-k block, lane-major),
+//    so every fragment read is one conflict-free ds_read_b128 and the global->LDS transfer is a
+//    16-byte-per-lane copy; two LDS buffers, one barrier per 128-element stage;
+//  * a wave's weights are its own strip and nobody else's, so they never touch LDS: each wave
+//    loads its 2 KiB of packed codes per stage straight into registers one stage ahead.
+#include <stdlib.h>
+
 #include "w2a8_launch.h"
 
 namespace w2a8 {
 
-constexpr int kBM = 128, kBN = 128;
+namespace fast {
+constexpr int kBM = 128, kBN = 256;
 constexpr int kStageSteps = 2;
-constexpr int kABlocks = (kBM / 16) * kStageSteps;        // 16 activation blocks per stage
-constexpr int kBUnits = (kBN / kStripN) * kStageSteps;    // 4 weight units per stage
-constexpr int kStageDwords = (kABlocks + kBUnits) * 256;  // 20 KiB per stage
+constexpr int kMB = kBM / 16;                              // 8 token blocks per wave
+constexpr int kStrips = kBN / kStripN;                     // 4 strips per workgroup, one per wave
+constexpr int kABlocks = kMB * kStageSteps;                // 16 activation blocks per stage
+constexpr int kStageDwords = kABlocks * 256;               // 16 KiB of activations per stage
+constexpr int kAQueue = 4;                                 // activation fragments kept in flight from LDS
+}  // namespace fast
 
-template <int GS, bool ASYM, bool DUMP, typename OutT>
-__global__ __launch_bounds__(256) void tiled_kernel(const GemmParams p) {
+template <int GS, typename OutT>
+__global__ __launch_bounds__(256, 2) void tiled_kernel(const GemmParams p) {
+    using namespace fast;
     __shared__ __attribute__((aligned(16))) uint32_t lds[2][kStageDwords];
+    constexpr int kGroupsPerStage = kStageSteps / GS;  // 2 (group 64) or 1 (group 128)
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 15, quad = lane >> 4;
-    const int wm = wave >> 1, wn = wave & 1;  // wave position inside the workgroup tile
-    const int m_tile = blockIdx.y * kBM;
-    const int strip0 = blockIdx.x * (kBN / kStripN);
-    const int strip = strip0 + wn;                 // strip of this wave
-    const bool strip_ok = strip < p.strips;
-    const int n_stages = (p.steps + kStageSteps - 1) / kStageSteps;
 
-    // ---- global -> register staging assignment
-    // activation blocks: wave w fetches blocks w, w+4, w+8, w+12 (block = step_in_stage*8 + mb)
-    // weight units:      wave w fetches unit w (unit = step_in_stage*2 + strip_in_tile)
-    v4i ga[4], gb;
-    const int8_t* a_src[4];
-    bool a_ok[4];
+    // Tile order: consecutive workgroup ids land on different XCDs (id % 8), each with its own
+    // L2.  Give every XCD one contiguous run of tiles, channel tile fastest, so that the tiles
+    // an XCD works on at the same time share their activation rows in that L2.
+    const int tiles_n = (p.strips + kStrips - 1) / kStrips;
+    const int tiles_m = (p.M + kBM - 1) / kBM;
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    const int tile = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if (tile >= total) return;
+    const int m_tile = (tile / tiles_n) * kBM;
+    const int strip0 = (tile % tiles_n) * kStrips;
+    const int strip = min(strip0 + wave, p.strips - 1);  // clamped: a surplus wave recomputes the last strip, stores nothing
+    const bool strip_ok = strip0 + wave < p.strips;
+    const int n_stages = p.steps / kStageSteps;
+
+    // ---- loads, one stage ahead, all through buffer instructions: a wave-uniform descriptor plus a
+    // scalar offset that advances per stage, so no vector ALU work goes into addresses, and rows
+    // past M read as zero (out-of-range buffer reads return 0).
+    //  * activations: wave w copies blocks w, w+4, w+8, w+12 (block = step_in_stage * 8 + token block)
+    //    straight from global memory into LDS (buffer_load_dwordx4 ... lds: lane l lands at 16*l);
+    //  * weights: the two units of the wave's own strip (one per step) go to registers;
+    //  * scales: the lane's four sub-block scales of each group of the stage.
+    const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int8_t*>(p.q), 0, (int)min((size_t)p.M * p.ldq, (size_t)0x7fffffff), 0x00020000);
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(p.w_r), 0, (int)min((size_t)p.strips * p.steps * (kUnitDwords * 4), (size_t)0x7fffffff), 0x00020000);
+    const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(p.s_r), 0, (int)min((size_t)p.strips * p.G * 128, (size_t)0x7fffffff), 0x00020000);
+    uint32_t a_off[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int blk = wave + 4 * i;
-        const int mb = blk & 7;
-        const int m = m_tile + mb * 16 + col;
-        a_ok[i] = m < p.M;
-        a_src[i] = p.q + (size_t)(a_ok[i] ? m : 0) * p.ldq + (blk >> 3) * kStepK + quad * 16;
+        a_off[i] = (uint32_t)(m_tile + (blk & 7) * 16 + col) * (uint32_t)p.ldq + (blk >> 3) * kStepK + quad * 16;
     }
-    const int b_strip = strip0 + (wave & 1);
-    const bool b_ok = b_strip < p.strips;
-    const uint32_t* b_src = p.w_r + ((size_t)(wave >> 1) * p.strips + (b_ok ? b_strip : 0)) * kUnitDwords + lane * 4;
-    const size_t b_step_stride = (size_t)p.strips * kUnitDwords;  // dwords between consecutive steps of a strip
-
-    auto fetch = [&](int stage) {
-        const int step0 = stage * kStageSteps;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int step = step0 + ((wave + 4 * i) >> 3);
-            ga[i] = v4i{0, 0, 0, 0};
-            if (a_ok[i] && step < p.steps) ga[i] = *reinterpret_cast<const v4i*>(a_src[i] + (size_t)step0 * kStepK);
-        }
-        const int bstep = step0 + (wave >> 1);
-        gb = v4i{0, 0, 0, 0};
-        if (b_ok && bstep < p.steps) gb = *reinterpret_cast<const v4i*>(b_src + (size_t)step0 * b_step_stride);
-    };
-    auto stash = [&](int buf) {
+    const uint32_t b_step_stride = (uint32_t)p.strips * (kUnitDwords * 4);  // bytes between steps of a strip
+    const uint32_t b_strip_off = (uint32_t)strip * (kUnitDwords * 4);
+    const uint32_t s_lane_off = (uint32_t)(strip * 16 + col) * 8;
+    const uint32_t s_group_stride = (uint32_t)p.strips * 128;               // bytes between groups of a strip
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    typedef unsigned v2u __attribute__((ext_vector_type(2)));
+    v4u gb[kStageSteps];
+    v2u sraw[kGroupsPerStage];
+    auto fetch = [&](int stage, int buf) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            *reinterpret_cast<v4i*>(&lds[buf][(wave + 4 * i) * 256 + lane * 4]) = ga[i];
-        *reinterpret_cast<v4i*>(&lds[buf][(kABlocks + wave) * 256 + lane * 4]) = gb;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                q_rsrc, (__attribute__((address_space(3))) void*)&lds[buf][(wave + 4 * i) * 256], 16, a_off[i],
+                stage * (kStageSteps * kStepK), 0, 0);
+#pragma unroll
+        for (int s = 0; s < kStageSteps; ++s)
+            gb[s] = __builtin_amdgcn_raw_buffer_load_b128(
+                w_rsrc, lane * 16, (stage * kStageSteps + s) * b_step_stride + b_strip_off, 0);
+#pragma unroll
+        for (int gi = 0; gi < kGroupsPerStage; ++gi)
+            sraw[gi] = __builtin_amdgcn_raw_buffer_load_b64(
+                s_rsrc, s_lane_off, (stage * kGroupsPerStage + gi) * s_group_stride, 0);
+    };
+    auto land = [&]() {  // every load of this wave has arrived (LDS-direct ones included), then meet the others
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
     };
 
-    float t[4][4][4];
-    v4i acc[4][4];
+    float t[kMB][4][4];
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
+    for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
-        for (int pp = 0; pp < 4; ++pp) {
-            acc[mb][pp] = v4i{0, 0, 0, 0};
+        for (int pp = 0; pp < 4; ++pp)
 #pragma unroll
             for (int j = 0; j < 4; ++j) t[mb][pp][j] = 0.0f;
-        }
 
-    const size_t sg_strip = (size_t)(strip_ok ? strip : 0);
-    const int m_wave = m_tile + wm * 64;  // first token row of this wave
+    fetch(0, 0);
+    land();
 
-    auto group_begin = [&](int g) {
-        int zpe[4];
-        if (ASYM) {
-            const uint32_t zraw = *reinterpret_cast<const uint32_t*>(p.zp_r + (((size_t)g * p.strips + sg_strip) * 16 + col) * 4);
-            zpe[0] = (int)(zraw & 0xffu);
-            zpe[1] = (int)((zraw >> 8) & 0xffu) * 4;
-            zpe[2] = (int)((zraw >> 16) & 0xffu) * 16;
-            zpe[3] = ((int)(zraw >> 24) - 2) * 64;
-        } else {
-            zpe[0] = p.zp_const;
-            zpe[1] = p.zp_const * 4;
-            zpe[2] = p.zp_const * 16;
-            zpe[3] = (p.zp_const - 2) * 64;
-        }
+    // accumulator sets (two, alternating) and the scale of the unit carried over a stage boundary;
+    // zero to start with, so the first carried drain adds nothing
+    v4i acc[2][4];
+    float sc_prev[4];
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb) {
-            const int m0 = m_wave + mb * 16 + quad * 4;
-            v4i rs = {0, 0, 0, 0};
-            if (m0 < p.M) rs = *reinterpret_cast<const v4i*>(p.rowsum + (size_t)g * p.ldr + m0);
-#pragma unroll
-            for (int pp = 0; pp < 4; ++pp) acc[mb][pp] = rs * (-zpe[pp]);
-        }
-    };
-    auto group_end = [&](int g) {
-        const uint2 sraw = *reinterpret_cast<const uint2*>(p.s_r + (((size_t)g * p.strips + sg_strip) * 16 + col) * 4);
-        float sc[4];
-        sc[0] = half_bits_to_float((uint16_t)(sraw.x & 0xffffu));
-        sc[1] = half_bits_to_float((uint16_t)(sraw.x >> 16)) * 0.25f;
-        sc[2] = half_bits_to_float((uint16_t)(sraw.y & 0xffffu)) * 0.0625f;
-        sc[3] = half_bits_to_float((uint16_t)(sraw.y >> 16)) * 0.015625f;
-#pragma unroll
-        for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-            for (int pp = 0; pp < 4; ++pp)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    t[mb][pp][j] = __builtin_fmaf((float)acc[mb][pp][j], sc[pp], t[mb][pp][j]);
-                    if (DUMP) {
-                        const int m = m_wave + mb * 16 + quad * 4 + j;
-                        const int n = strip * kStripN + pp * 16 + col;
-                        if (strip_ok && m < p.M && n < p.N) {
-                            const int v = acc[mb][pp][j] >> (2 * pp);
-                            if (p.dump_mode == 1)
-                                p.acc_dump[((size_t)m * p.N + n) * p.G + g] = v;
-                            else
-                                p.acc_dump[(size_t)m * p.N + n] += v;  // one wave owns (m, n): no race
-                        }
-                    }
-                }
-    };
-
-    fetch(0);
-    stash(0);
-    __syncthreads();
+    for (int pp = 0; pp < 4; ++pp) {
+        acc[0][pp] = v4i{0, 0, 0, 0};
+        acc[1][pp] = v4i{0, 0, 0, 0};
+        sc_prev[pp] = 0.0f;
+    }
 
     for (int stage = 0; stage < n_stages; ++stage) {
         const int buf = stage & 1;
-        if (stage + 1 < n_stages) fetch(stage + 1);
+        const uint32_t* la = &lds[buf][lane * 4];
+        auto lds_a = [&](int r) {  // r-th fragment in consumption order: token block r / 2, step r % 2
+            return *reinterpret_cast<const v4i*>(la + ((r % kStageSteps) * kMB + r / kStageSteps) * 256);
+        };
+        v4i aq[kAQueue];
+#pragma unroll
+        for (int r = 0; r < kAQueue; ++r) aq[r] = lds_a(r);
+
+        float sc[kGroupsPerStage][4];
+#pragma unroll
+        for (int gi = 0; gi < kGroupsPerStage; ++gi) {
+            // operand bytes are 64 * (code - 2): fold 1/64 into the scale (exact)
+            sc[gi][0] = half_bits_to_float((uint16_t)(sraw[gi].x & 0xffffu)) * 0.015625f;
+            sc[gi][1] = half_bits_to_float((uint16_t)(sraw[gi].x >> 16)) * 0.015625f;
+            sc[gi][2] = half_bits_to_float((uint16_t)(sraw[gi].y & 0xffffu)) * 0.015625f;
+            sc[gi][3] = half_bits_to_float((uint16_t)(sraw[gi].y >> 16)) * 0.015625f;
+        }
+
+        // unpack this wave's strip for both steps of the stage (loaded during the previous stage)
+        v4i b[kStageSteps][4];
 #pragma unroll
         for (int s = 0; s < kStageSteps; ++s) {
-            const int step = stage * kStageSteps + s;
-            if (step < p.steps) {
-                if (step % GS == 0) group_begin(step / GS);
-                const v4i w = *reinterpret_cast<const v4i*>(&lds[buf][(kABlocks + s * 2 + wn) * 256 + lane * 4]);
-                v4i b[4];
+            const v4i w = __builtin_bit_cast(v4i, gb[s]);
+            const v4i wf = w ^ (int)0x2a2a2a2au;  // flip the high bit of fields 0..2: code -> two's complement of code - 2
 #pragma unroll
-                for (int pp = 0; pp < 4; ++pp) b[pp] = w & (int)(0x03030303u << (2 * pp));
-#pragma unroll
-                for (int mb = 0; mb < 4; ++mb) {
-                    const v4i a = *reinterpret_cast<const v4i*>(&lds[buf][(s * 8 + wm * 4 + mb) * 256 + lane * 4]);
-#pragma unroll
-                    for (int pp = 0; pp < 4; ++pp) acc[mb][pp] = mfma_i8_16x16x64(a, b[pp], acc[mb][pp]);
-                }
-                if (step % GS == GS - 1) group_end(step / GS);
-            }
+            for (int pp = 0; pp < 3; ++pp) b[s][pp] = (wf << (6 - 2 * pp)) & (int)0xc0c0c0c0u;
+            b[s][3] = w & (int)0xc0c0c0c0u;  // field 3 is stored already flipped
         }
-        if (stage + 1 < n_stages) stash(buf ^ 1);
-        __syncthreads();
+
+        // next stage (the last iteration re-reads its own stage into the idle buffer: harmless)
+        fetch(min(stage + 1, n_stages - 1), buf ^ 1);
+
+        // Work units in order: (token block, group of the stage).  The MFMAs of unit u go into
+        // accumulator set u & 1 and are written before the drain of unit u - 1, so the matrix core
+        // works on one unit while the vector ALU folds the previous one; the last unit of a stage
+        // is drained at the top of the next stage (or after the loop).
+        constexpr int kUnits = kMB * kGroupsPerStage;
+#pragma unroll
+        for (int u = 0; u < kUnits; ++u) {
+            const int mb = u / kGroupsPerStage, gi = u % kGroupsPerStage;
+#pragma unroll
+            for (int s = 0; s < GS; ++s) {
+                const int r = mb * kStageSteps + gi * GS + s;  // fragment index in consumption order
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp)
+                    acc[u & 1][pp] = mfma_i8_16x16x64(aq[r % kAQueue], b[gi * GS + s][pp],
+                                                      s == 0 ? v4i{0, 0, 0, 0} : acc[u & 1][pp]);
+                if (r + kAQueue < kABlocks) aq[r % kAQueue] = lds_a(r + kAQueue);
+            }
+            // drain the previous unit (for u == 0: the last unit of the previous stage, scale sc_prev)
+            const int pu = (u + kUnits - 1) % kUnits;
+            const int pmb = pu / kGroupsPerStage, pgi = pu % kGroupsPerStage;
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    t[pmb][pp][j] = __builtin_fmaf((float)acc[(u & 1) ^ 1][pp][j], u == 0 ? sc_prev[pp] : sc[pgi][pp],
+                                                   t[pmb][pp][j]);
+        }
+#pragma unroll
+        for (int pp = 0; pp < 4; ++pp) sc_prev[pp] = sc[kGroupsPerStage - 1][pp];
+
+        land();
     }
+    // the last unit of the last stage
+#pragma unroll
+    for (int pp = 0; pp < 4; ++pp)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            t[kMB - 1][pp][j] = __builtin_fmaf((float)acc[1][pp][j], sc_prev[pp], t[kMB - 1][pp][j]);
 
     // ---- epilogue: out = cast(t * s_a[m])
     if (!strip_ok) return;
     uint16_t* out = reinterpret_cast<uint16_t*>(p.out);
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
+    for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int m = m_wave + mb * 16 + quad * 4 + j;
+            const int m = m_tile + mb * 16 + quad * 4 + j;
             if (m >= p.M) continue;
             const float sa = p.s_a[m];
 #pragma unroll
@@ -185,31 +222,23 @@ __global__ __launch_bounds__(256) void tiled_kernel(const GemmParams p) {
         }
 }
 
-template <int GS, bool ASYM, bool DUMP>
-static void launch_out(const GemmParams& p, bool out_bf16, hipStream_t stream) {
-    const dim3 grid((p.strips + 1) / 2, (p.M + kBM - 1) / kBM), block(256);
-    if (out_bf16)
-        tiled_kernel<GS, ASYM, DUMP, OutBF16><<<grid, block, 0, stream>>>(p);
-    else
-        tiled_kernel<GS, ASYM, DUMP, OutF16><<<grid, block, 0, stream>>>(p);
-}
-
-template <int GS>
-static void launch_flags(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
+bool tiled_fast_supported(const GemmParams& p, int gs, bool asym) {
     const bool dump = p.acc_dump != nullptr && p.dump_mode != 0;
-    if (asym) {
-        if (dump) launch_out<GS, true, true>(p, out_bf16, stream);
-        else launch_out<GS, true, false>(p, out_bf16, stream);
-    } else {
-        if (dump) launch_out<GS, false, true>(p, out_bf16, stream);
-        else launch_out<GS, false, false>(p, out_bf16, stream);
-    }
+    return !asym && !dump && p.zp_const == 2 && (gs == 1 || gs == 2) && p.steps % fast::kStageSteps == 0;
 }
 
 hipError_t launch_tiled(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream) {
-    if (gs == 1) launch_flags<1>(p, asym, out_bf16, stream);
-    else if (gs == 2) launch_flags<2>(p, asym, out_bf16, stream);
-    else launch_flags<4>(p, asym, out_bf16, stream);
+    if (!tiled_fast_supported(p, gs, asym)) return launch_tiled_generic(p, gs, asym, out_bf16, stream);
+    const int tiles = ((p.strips + fast::kStrips - 1) / fast::kStrips) * ((p.M + fast::kBM - 1) / fast::kBM);
+    const dim3 grid((tiles + 7) / 8 * 8), block(256);
+    static const int pad = [] { const char* e = getenv("SLIMK_W2A8_TILED_LDS_PAD"); return e ? atoi(e) : 0; }();
+    if (gs == 1) {
+        if (out_bf16) tiled_kernel<1, OutBF16><<<grid, block, pad, stream>>>(p);
+        else tiled_kernel<1, OutF16><<<grid, block, pad, stream>>>(p);
+    } else {
+        if (out_bf16) tiled_kernel<2, OutBF16><<<grid, block, pad, stream>>>(p);
+        else tiled_kernel<2, OutF16><<<grid, block, pad, stream>>>(p);
+    }
     return hipGetLastError();
 }
 
