@@ -4,16 +4,20 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 Workload (config "c2", the decode regime the headline metric is quoted on): one step =
-24 skinny split-K GEMM launches, M in {1,2,4,8,16,32} over the four Llama-3-8B linear
+the 24 independent GEMMs of the sweep, M in {1,2,4,8,16,32} over the four Llama-3-8B linear
 shapes (4096x4096, 1024x4096, 14336x4096, 4096x14336), 2-bit symmetric group-128 weights,
-per-token int8 activations with 0.1 % outlier channels, fp16 out.  Inputs are resident in
-HBM before the timed region; every launch reads a different copy of its weight matrix so
-that the stream comes from HBM and not from the 256 MiB Infinity Cache ("cold").  The step
-is replayed from a HIP graph so that host launch cost does not pace microsecond kernels.
+per-token int8 activations with 0.1 % outlier channels, fp16 out, issued as ONE grouped
+launch of the skinny kernel (slimk_w2a8_gemm_grouped).  Inputs are resident in HBM before
+the timed region; every GEMM of every step reads a different copy of its weight matrix, so
+the stream comes from HBM and not from the 256 MiB Infinity Cache ("cold").  Steps are
+replayed from a HIP graph so that host launch cost does not pace the GPU.
 
 value  = algorithmic bytes of all GEMMs / wall time      (GB/s, higher is better)
-roofline.achieved = mean algorithmic bytes per launch / mean launch duration, HIP events
-                    on the launch stream, against the 8 TB/s HBM3E peak.
+roofline.achieved = algorithmic bytes per launch / mean launch duration, HIP events on the
+                    launch stream, against the 8 TB/s HBM3E peak.
+detail.single_launch repeats the same step as 24 separate launches (one GEMM each): those are
+latency-bound (5-10 us per launch whatever the size) and are reported per shape in
+detail.decode.
 cpu_baseline = the same GEMMs (bounded sample) through the CPU oracle's restatement of the
                reference CPU path (numpy quantiser/packer output + torch CPU int matmul).
 Activation quantisation is timed separately (detail.act_quant).  detail also carries the
@@ -99,14 +103,20 @@ def main():
         acts[(c.N, c.K, c.M)] = (x, qa, out)
     name_of = {(N, K): n for n, (N, K) in workloads.LLAMA8B_LINEARS.items()}
 
-    def launch_step(warm=False):
+    def launch_step(warm=False, grouped=True):
+        probs = []
         for c in cases:
             sh = shapes[name_of[(c.N, c.K)]]
             w = sh.copies[0] if warm else sh.copies[sh.next % len(sh.copies)]
             if not warm:
                 sh.next += 1
             _, qa, out = acts[(c.N, c.K, c.M)]
-            ops.w2a8_gemm(qa, w, torch.float16, out=out)
+            if grouped:
+                probs.append((qa, w, out))
+            else:
+                ops.w2a8_gemm(qa, w, torch.float16, out=out)
+        if grouped:
+            ops.w2a8_gemm_grouped(probs, torch.float16)
 
     # touch every copy once eagerly: creates and zeroes the split-K workspaces outside any capture
     for sh in shapes.values():
@@ -115,53 +125,56 @@ def main():
             ops.w2a8_gemm(qa, w, torch.float16, out=out)
     torch.cuda.synchronize()
 
-    def capture(n_steps, warm=False):
+    def capture(n_steps, warm=False, grouped=True):
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             for _ in range(n_steps):
-                launch_step(warm)
+                launch_step(warm, grouped)
         return g
 
     # ------------------------------------------------------------------ timed region
     UNROLL = 8
-    graphs = {}
 
-    def run_steps(k):
-        full, rem = divmod(k, UNROLL)
-        if full and UNROLL not in graphs:
-            graphs[UNROLL] = capture(UNROLL)
-        if rem and rem not in graphs:
-            graphs[rem] = capture(rem)
-        return full, rem
+    def timed_run(grouped):
+        """W warm-up steps, then exactly K timed steps; returns (wall seconds, HIP-event milliseconds)."""
+        graphs = {}
 
-    full_w, rem_w = run_steps(args.warmup)
-    full_k, rem_k = run_steps(args.steps)
-    torch.cuda.synchronize()
-    for _ in range(full_w):
-        graphs[UNROLL].replay()
-    if rem_w:
-        graphs[rem_w].replay()
-    torch.cuda.synchronize()
+        def plan(k):
+            full, rem = divmod(k, UNROLL)
+            if full and UNROLL not in graphs:
+                graphs[UNROLL] = capture(UNROLL, grouped=grouped)
+            if rem and rem not in graphs:
+                graphs[rem] = capture(rem, grouped=grouped)
+            return full, rem
 
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for _ in range(full_k):
-        graphs[UNROLL].replay()
-    if rem_k:
-        graphs[rem_k].replay()
-    e1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ev_ms = e0.elapsed_time(e1)
+        full_w, rem_w = plan(args.warmup)
+        full_k, rem_k = plan(args.steps)
+        torch.cuda.synchronize()
+        for _ in range(full_w):
+            graphs[UNROLL].replay()
+        if rem_w:
+            graphs[rem_w].replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(full_k):
+            graphs[UNROLL].replay()
+        if rem_k:
+            graphs[rem_k].replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, e0.elapsed_time(e1)
+
+    wall, ev_ms = timed_run(grouped=True)
 
     step_bytes = sum(workloads.algorithmic_bytes(c) for c in cases)
     step_ops = sum(workloads.algorithmic_ops(c) for c in cases)
-    launches = len(cases) * args.steps
+    launches = args.steps                       # one grouped launch per step
     ms_per_step = wall * 1e3 / args.steps
     value = step_bytes * args.steps / wall / 1e9
     avg_launch_us = ev_ms * 1e3 / launches
-    achieved = (step_bytes / len(cases)) / (avg_launch_us * 1e-6) / 1e9
+    achieved = step_bytes / (avg_launch_us * 1e-6) / 1e9
 
     result = {
         "metric": "W2A8 GEMM TOPS + HBM GB/s (% roofline) at M=1..4096, 1 MI355X",
@@ -170,17 +183,25 @@ def main():
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": "c2 decode sweep: M in {1,2,4,8,16,32} x Llama-3-8B linears "
                                "(4096x4096, 1024x4096, 14336x4096, 4096x14336), W2 sym g128, A8 per-token, "
-                               "fp16 out; 24 skinny split-K GEMM launches per step, cold HBM (rotating weight copies)",
-                   "launches_per_step": len(cases), "algorithmic_bytes_per_step": step_bytes,
+                               "fp16 out; the 24 GEMMs of a step issued as one grouped skinny-kernel launch, "
+                               "cold HBM (rotating weight copies)",
+                   "launches_per_step": 1, "gemms_per_step": len(cases), "algorithmic_bytes_per_step": step_bytes,
                    "ops_per_step": step_ops, "timing": "HIP graph replay, inputs resident in HBM"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "w2a8::skinny_kernel", "avg_launch_us": round(avg_launch_us, 3),
-                     "algorithmic_bytes_per_launch": step_bytes // len(cases)},
+                     "kernel": "w2a8::skinny_grouped_kernel", "avg_launch_us": round(avg_launch_us, 3),
+                     "algorithmic_bytes_per_launch": step_bytes},
     }
 
     detail = {"tops_decode": round(step_ops * args.steps / wall / 1e12, 3)}
     if not args.skip_detail:
+        wall1, ev1 = timed_run(grouped=False)
+        us1 = ev1 * 1e3 / (len(cases) * args.steps)
+        detail["single_launch"] = {
+            "what": "the same steps as 24 separate launches, one GEMM each (w2a8::skinny_kernel)",
+            "GBps": round(step_bytes * args.steps / wall1 / 1e9, 2), "ms_per_step": round(wall1 * 1e3 / args.steps, 5),
+            "avg_launch_us": round(us1, 3),
+            "frac_hbm": round(step_bytes / len(cases) / (us1 * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
         detail.update(collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, dev))
         result["cpu_baseline"] = cpu_baseline(np, workloads, shapes)
     else:

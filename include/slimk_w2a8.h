@@ -144,6 +144,33 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
                     void* workspace, size_t workspace_bytes,
                     int kernel, int split_k, void* stream);
 
+/* One problem of a grouped launch: the arguments of slimk_w2a8_gemm that describe data. */
+typedef struct slimk_w2a8_problem {
+    const int8_t* q;
+    const float* s_a;
+    const int32_t* rowsum;
+    const uint32_t* w_r;
+    const uint16_t* s_r;
+    const uint8_t* zp_r; /* NULL: uniform zero-point zp_const */
+    void* out;
+    int ldq, ldr, ldo;
+    int M, N, K;
+    int zp_const;
+} slimk_w2a8_problem;
+
+#define SLIMK_W2A8_MAX_GROUP 24
+
+/* Several independent skinny (M <= 32) GEMMs in ONE kernel launch.  A decode step issues many
+ * small GEMMs whose individual run time is a few microseconds of mostly launch and memory
+ * latency; run together they fill the chip and stream from HBM at full rate.
+ * `problems` is a HOST array of `count` (1..SLIMK_W2A8_MAX_GROUP) entries, copied into the
+ * kernel arguments (so the call is graph-capturable and the array may be reused at once).
+ * All problems share group_size, out_dtype and the zero-point mode (all zp_r NULL with
+ * zp_const == 2, all zp_r NULL with other constants, or all zp_r non-NULL); M, N, K may
+ * differ.  No split-K, no workspace.  No upstream counterpart. */
+int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int group_size, int out_dtype,
+                            void* stream);
+
 /* Streaming-read calibration kernel: sums `bytes` (multiple of 16) of device memory into
  * sink[0..] so that a profiler can relate its FETCH_SIZE counter to a known byte count and
  * the benchmark can quote the achievable HBM read rate next to the GEMM's. */

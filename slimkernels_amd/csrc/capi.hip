@@ -245,6 +245,57 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
     return hip_result(w2a8::launch_tiled(p, gs, asym, out_bf16, st), "tiled gemm");
 }
 
+int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int group_size, int out_dtype,
+                            void* stream) {
+    if (!problems) return fail(SLIMK_ERR_NULL_POINTER, "gemm_grouped: problems is NULL");
+    if (count < 1 || count > SLIMK_W2A8_MAX_GROUP)
+        return fail(SLIMK_ERR_BAD_SHAPE, "gemm_grouped: count=%d must be 1..%d", count, SLIMK_W2A8_MAX_GROUP);
+    if (out_dtype != SLIMK_F16 && out_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "out_dtype=%d", out_dtype);
+    if (group_size != 64 && group_size != 128 && group_size != 256)
+        return fail(SLIMK_ERR_BAD_SHAPE, "group_size=%d must be 64, 128 or 256", group_size);
+    // longest reductions first: their workgroups run longest and should not start last
+    int order[SLIMK_W2A8_MAX_GROUP];
+    for (int i = 0; i < count; ++i) order[i] = i;
+    for (int i = 1; i < count; ++i)
+        for (int j = i; j > 0 && problems[order[j]].K > problems[order[j - 1]].K; --j) {
+            const int t = order[j]; order[j] = order[j - 1]; order[j - 1] = t;
+        }
+    static_assert(SLIMK_W2A8_MAX_GROUP == w2a8::kMaxGroup, "group limit");
+    w2a8::GroupedParams gp{};
+    gp.count = count;
+    int zm = -1, wgs = 0;
+    for (int i = 0; i < count; ++i) {
+        const slimk_w2a8_problem& pr = problems[order[i]];
+        if (!pr.q || !pr.s_a || !pr.rowsum || !pr.w_r || !pr.s_r || !pr.out)
+            return fail(SLIMK_ERR_NULL_POINTER, "gemm_grouped: problem %d has a NULL buffer", order[i]);
+        if (pr.M <= 0 || pr.N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "gemm_grouped: problem %d: M=%d, N=%d", order[i], pr.M, pr.N);
+        if (pr.M > 32) return fail(SLIMK_ERR_UNSUPPORTED, "gemm_grouped: problem %d has M=%d > 32", order[i], pr.M);
+        if (int rc = check_kg(pr.K, group_size)) return rc;
+        if (pr.ldq < pr.K || pr.ldo < pr.N || pr.ldr < pr.M)
+            return fail(SLIMK_ERR_BAD_SHAPE, "gemm_grouped: problem %d: a leading dimension is too small", order[i]);
+        if (pr.zp_const < 0 || pr.zp_const > 3) return fail(SLIMK_ERR_BAD_SHAPE, "gemm_grouped: problem %d: zp_const=%d", order[i], pr.zp_const);
+        if (!aligned16(pr.q) || pr.ldq % 16 != 0 || !aligned16(pr.rowsum) || pr.ldr % 4 != 0 || !aligned16(pr.w_r) ||
+            !aligned16(pr.s_r) || (pr.zp_r && !aligned16(pr.zp_r)) || (reinterpret_cast<uintptr_t>(pr.out) & 1u))
+            return fail(SLIMK_ERR_MISALIGNED, "gemm_grouped: problem %d breaks an alignment rule of slimk_w2a8_gemm", order[i]);
+        const int this_zm = pr.zp_r ? 2 : (pr.zp_const == 2 ? 0 : 1);
+        if (zm >= 0 && this_zm != zm)
+            return fail(SLIMK_ERR_UNSUPPORTED, "gemm_grouped: problems mix zero-point modes");
+        zm = this_zm;
+        w2a8::GemmParams& g = gp.prob[i];
+        g.q = pr.q; g.s_a = pr.s_a; g.rowsum = pr.rowsum; g.w_r = pr.w_r; g.s_r = pr.s_r; g.zp_r = pr.zp_r;
+        g.out = pr.out; g.ldq = pr.ldq; g.ldr = pr.ldr; g.ldo = pr.ldo;
+        g.M = pr.M; g.N = pr.N; g.K = pr.K; g.G = pr.K / group_size; g.steps = pr.K / w2a8::kStepK;
+        g.strips = strips_of(pr.N); g.zp_const = pr.zp_const;
+        g.split = 1; g.groups_per_split = groups_per_split(g.G, group_size, 1);
+        gp.wg_begin[i] = wgs;
+        wgs += g.strips;
+    }
+    gp.wg_begin[count] = wgs;
+    return hip_result(w2a8::launch_skinny_grouped(gp, group_size / w2a8::kStepK, zm, out_dtype == SLIMK_BF16,
+                                                  (hipStream_t)stream),
+                      "grouped skinny gemm");
+}
+
 int slimk_w2a8_read_probe(const void* src, size_t bytes, uint32_t* sink, void* stream) {
     if (!src || !sink) return fail(SLIMK_ERR_NULL_POINTER, "read_probe: NULL buffer");
     if (bytes == 0 || bytes % 16 != 0 || !aligned16(src))

@@ -44,11 +44,11 @@ struct SkinnySmem {
 // ZM = zero-point mode: 0 uniform zero-point 2 (the symmetric levels; folded with shifts),
 // 1 any other uniform zero-point, 2 per-(group, channel) zero-points read from zp_r.
 template <int MB, int J, int GS, int NW, int ZM, bool DUMP, typename OutT>
-__global__ __launch_bounds__(NW * 64) void skinny_kernel(const GemmParams p) {
+__device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip, const int split,
+                                            SkinnySmem<MB, NW>& sm) {
     constexpr bool ASYM = ZM == 2;
     constexpr bool SYM2 = ZM == 0;
     constexpr int kThreads = NW * 64;
-    __shared__ __attribute__((aligned(16))) SkinnySmem<MB, NW> sm;
     constexpr int kGroupsPerChunk = kDepth / GS;
     constexpr int kTile = MB * 16 * kStripN;  // elements of the workgroup's output tile
     constexpr int kOutPerThread = (kTile + kThreads - 1) / kThreads;
@@ -57,8 +57,6 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const GemmParams p) {
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps ranges and bases in SGPRs
     const int col = lane & 15, quad = lane >> 4;
-    const int strip = blockIdx.x;
-    const int split = blockIdx.y;
 
     // token scales for the epilogue (element e = tid + kThreads*i -> row e >> 6), fetched first
     float sa[kOutPerThread];
@@ -298,6 +296,36 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const GemmParams p) {
     if (tid == 0) __hip_atomic_store(p.ws_counter + strip, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+template <int MB, int J, int GS, int NW, int ZM, bool DUMP, typename OutT>
+__global__ __launch_bounds__(NW * 64) void skinny_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(16))) SkinnySmem<MB, NW> sm;
+    skinny_body<MB, J, GS, NW, ZM, DUMP, OutT>(p, blockIdx.x, blockIdx.y, sm);
+}
+
+// Several independent skinny GEMMs in one launch: workgroup ids are cut into runs, one run per
+// problem (one workgroup per strip, no split-K: together the problems fill the chip), and each
+// workgroup runs the single-problem body on its problem.  All problems share the group size,
+// the zero-point mode and the output type; M may differ (the three row-count variants live side
+// by side in the kernel).  The problem table travels in the kernel arguments.
+#ifndef SLIMK_GROUPED_WAVES_PER_SIMD
+#define SLIMK_GROUPED_WAVES_PER_SIMD 2
+#endif
+template <int GS, int ZM, typename OutT>
+__global__ __launch_bounds__(256, SLIMK_GROUPED_WAVES_PER_SIMD) void skinny_grouped_kernel(const GroupedParams gp) {
+    __shared__ __attribute__((aligned(16))) union {
+        SkinnySmem<1, 4> one;
+        SkinnySmem<2, 4> two;
+    } sm;
+    const int wg = blockIdx.x;
+    int i = 0;
+    while (i + 1 < gp.count && wg >= gp.wg_begin[i + 1]) ++i;
+    const GemmParams& p = gp.prob[i];
+    const int strip = wg - gp.wg_begin[i];
+    if (p.M == 1) skinny_body<1, 1, GS, 4, ZM, false, OutT>(p, strip, 0, sm.one);
+    else if (p.M <= 16) skinny_body<1, 4, GS, 4, ZM, false, OutT>(p, strip, 0, sm.one);
+    else skinny_body<2, 4, GS, 4, ZM, false, OutT>(p, strip, 0, sm.two);
+}
+
 template <int MB, int J, int GS, int NW, int ZM, bool DUMP>
 static void launch_out(const GemmParams& p, bool out_bf16, hipStream_t stream) {
     const dim3 grid(p.strips, p.split), block(NW * 64);
@@ -338,6 +366,27 @@ static void launch_gs(const GemmParams& p, int gs, int waves, bool asym, bool ou
     if (gs == 1) launch_nw<MB, 1>(p, waves, asym, out_bf16, stream);
     else if (gs == 2) launch_nw<MB, 2>(p, waves, asym, out_bf16, stream);
     else launch_nw<MB, 4>(p, waves, asym, out_bf16, stream);
+}
+
+template <int GS, int ZM>
+static void launch_grouped_out(const GroupedParams& gp, int total_wgs, bool out_bf16, hipStream_t stream) {
+    if (out_bf16) skinny_grouped_kernel<GS, ZM, OutBF16><<<dim3(total_wgs), dim3(256), 0, stream>>>(gp);
+    else skinny_grouped_kernel<GS, ZM, OutF16><<<dim3(total_wgs), dim3(256), 0, stream>>>(gp);
+}
+
+template <int GS>
+static void launch_grouped_zm(const GroupedParams& gp, int total_wgs, int zm, bool out_bf16, hipStream_t stream) {
+    if (zm == 0) launch_grouped_out<GS, 0>(gp, total_wgs, out_bf16, stream);
+    else if (zm == 1) launch_grouped_out<GS, 1>(gp, total_wgs, out_bf16, stream);
+    else launch_grouped_out<GS, 2>(gp, total_wgs, out_bf16, stream);
+}
+
+hipError_t launch_skinny_grouped(const GroupedParams& gp, int gs, int zm, bool out_bf16, hipStream_t stream) {
+    const int total_wgs = gp.wg_begin[gp.count];
+    if (gs == 1) launch_grouped_zm<1>(gp, total_wgs, zm, out_bf16, stream);
+    else if (gs == 2) launch_grouped_zm<2>(gp, total_wgs, zm, out_bf16, stream);
+    else launch_grouped_zm<4>(gp, total_wgs, zm, out_bf16, stream);
+    return hipGetLastError();
 }
 
 hipError_t launch_skinny(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, hipStream_t stream) {

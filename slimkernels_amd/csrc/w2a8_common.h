@@ -60,6 +60,14 @@ struct GemmParams {
     int groups_per_split;   // ceil(G / split)
 };
 
+// Problem table of a grouped skinny launch; passed by value in the kernel arguments (< 4 KiB).
+constexpr int kMaxGroup = 24;
+struct GroupedParams {
+    GemmParams prob[kMaxGroup];
+    int wg_begin[kMaxGroup + 1];  // problem i owns workgroups wg_begin[i] .. wg_begin[i+1]-1 (one per strip)
+    int count;
+};
+
 __device__ __forceinline__ v4i mfma_i8_16x16x64(v4i a, v4i b, v4i c) {
     // D[i][j] += sum_k A[i][k] * B[k][j]; lane l supplies row/col (l & 15) and the
     // 16 k-values of quarter (l >> 4); D lane l, element j = row 4*(l>>4)+j, col l&15.

@@ -15,6 +15,7 @@ computes on the CPU.
 """
 from __future__ import annotations
 
+import ctypes
 import dataclasses
 from typing import Optional
 
@@ -168,6 +169,40 @@ def w2a8_gemm(qa: QuantizedActivation, w: W2A8Weight, out_dtype=torch.float16, *
             ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
             kern, split_k, _stream_ptr(dev)))
     return (out, acc) if acc is not None else out
+
+
+def w2a8_gemm_grouped(problems, out_dtype=torch.float16):
+    """Several independent skinny (M <= 32) GEMMs in one kernel launch.
+
+    ``problems`` is a sequence of (QuantizedActivation, W2A8Weight) or (qa, w, out) tuples that
+    share group size and zero-point mode; returns the list of outputs.  More than 24 problems are
+    issued as several launches."""
+    L = _lib.lib()
+    probs = [(p[0], p[1], p[2] if len(p) > 2 else None) for p in problems]
+    if not probs:
+        return []
+    dev = probs[0][0].q.device
+    g = probs[0][1].group_size
+    outs = []
+    with torch.cuda.device(dev):
+        for lo in range(0, len(probs), _lib.MAX_GROUP):
+            chunk = probs[lo:lo + _lib.MAX_GROUP]
+            arr = (_lib.Problem * len(chunk))()
+            for i, (qa, w, out) in enumerate(chunk):
+                M, K = qa.q.shape
+                if K != w.K or qa.group_size != w.group_size or w.group_size != g:
+                    raise ValueError("grouped problems must share the group size and match their weights' K")
+                if out is None:
+                    out = torch.empty((M, w.N), dtype=out_dtype, device=dev)
+                if out.dtype != out_dtype:
+                    raise ValueError("every output must have dtype out_dtype")
+                outs.append(out)
+                arr[i] = _lib.Problem(qa.q.data_ptr(), qa.s_a.data_ptr(), qa.rowsum.data_ptr(), w.w_r.data_ptr(),
+                                      w.s_r.data_ptr(), w.zp_r.data_ptr() if w.zp_r is not None else None,
+                                      out.data_ptr(), qa.q.stride(0), qa.rowsum.stride(0), out.stride(0),
+                                      M, w.N, K, w.zp_const)
+            _lib.check(L.slimk_w2a8_gemm_grouped(ctypes.byref(arr), len(chunk), g, _DT[out_dtype], _stream_ptr(dev)))
+    return outs
 
 
 def wint2_gemm(activation: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, zp=None,

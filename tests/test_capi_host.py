@@ -1,0 +1,145 @@
+"""Host-side checks of the C ABI (no GPU): the library loads, exports every symbol the header
+declares, answers its size queries, and rejects bad arguments with the documented codes before
+anything could be launched."""
+import ctypes
+import os
+import re
+import threading
+
+import pytest
+
+from slimkernels_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "slimk_w2a8.h")
+FAKE = 0x10000  # a non-NULL, 16-byte aligned value: validation never dereferences pointers
+
+
+@pytest.fixture(scope="module")
+def L():
+    return _lib.lib()
+
+
+def declared_symbols():
+    text = open(HEADER, encoding="utf-8").read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(slimk_w2a8_\w+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound(L):
+    names = declared_symbols()
+    assert len(names) >= 12
+    for n in names:
+        assert hasattr(L, n), f"{n} is declared in the header but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
+    assert set(_lib.SIGNATURES) == set(names)
+
+
+def test_version_arch_and_sizes(L):
+    assert L.slimk_w2a8_version() == 100
+    assert L.slimk_w2a8_arch() == b"gfx950"
+    assert L.slimk_w2a8_repacked_weight_bytes(4096, 4096) == 4096 * 4096 // 4
+    assert L.slimk_w2a8_repacked_weight_bytes(100, 128) == 2 * 2 * 1024     # two strips (N padded to 128) x two steps
+    assert L.slimk_w2a8_repacked_scale_bytes(4096, 4096, 128) == 2 * 4096 * 32
+    assert L.slimk_w2a8_repacked_zp_bytes(4096, 4096, 128) == 4096 * 32
+    assert L.slimk_w2a8_repacked_weight_bytes(4096, 100) == 0               # K % 64
+    assert L.slimk_w2a8_repacked_scale_bytes(4096, 4096, 96) == 0           # group size
+    assert L.slimk_w2a8_repacked_scale_bytes(4096, 4096 + 64, 128) == 0     # K % group
+
+
+def test_split_heuristic_and_workspace(L):
+    # unsplit: many strips, or a matrix of a few MiB
+    assert L.slimk_w2a8_gemm_auto_split_k(16, 14336, 4096, 128, _lib.KERNEL_AUTO) == 1
+    assert L.slimk_w2a8_gemm_auto_split_k(1, 4096, 4096, 128, _lib.KERNEL_AUTO) == 1
+    assert L.slimk_w2a8_gemm_workspace_bytes(16, 14336, 4096, 128, _lib.KERNEL_AUTO, 0) == 0
+    # few strips, long K: split to about 256 workgroups
+    s = L.slimk_w2a8_gemm_auto_split_k(16, 4096, 14336, 128, _lib.KERNEL_AUTO)
+    assert s == 4
+    ws = L.slimk_w2a8_gemm_workspace_bytes(16, 4096, 14336, 128, _lib.KERNEL_AUTO, 0)
+    assert ws == 256 + s * 64 * (16 * 64) * 4     # counters + split x strips x (16 x 64 fp32 tile)
+    assert L.slimk_w2a8_gemm_workspace_bytes(32, 4096, 14336, 128, _lib.KERNEL_AUTO, 4) == 256 + 4 * 64 * (32 * 64) * 4
+    # the tiled kernel never splits
+    assert L.slimk_w2a8_gemm_auto_split_k(512, 4096, 14336, 128, _lib.KERNEL_AUTO) == 1
+    assert L.slimk_w2a8_gemm_auto_split_k(0, 4096, 4096, 128, 0) == 0
+
+
+def _gemm(L, **kw):
+    a = dict(q=FAKE, ldq=4096, s_a=FAKE, rowsum=FAKE, ldr=16, w_r=FAKE, s_r=FAKE, zp_r=None, zp_const=2,
+             M=16, N=4096, K=4096, g=128, out=FAKE, ldo=4096, odt=0, acc=None, dump=0, ws=None, wsb=0,
+             kernel=0, split=0, stream=None)
+    a.update(kw)
+    return L.slimk_w2a8_gemm(a["q"], a["ldq"], a["s_a"], a["rowsum"], a["ldr"], a["w_r"], a["s_r"], a["zp_r"],
+                             a["zp_const"], a["M"], a["N"], a["K"], a["g"], a["out"], a["ldo"], a["odt"], a["acc"],
+                             a["dump"], a["ws"], a["wsb"], a["kernel"], a["split"], a["stream"])
+
+
+def test_gemm_argument_validation(L):
+    assert _gemm(L, q=None) == 1 and b"NULL" in L.slimk_w2a8_last_error()
+    assert _gemm(L, out=None) == 1
+    assert _gemm(L, M=0) == 2
+    assert _gemm(L, K=4000) == 2 and b"multiple of 64" in L.slimk_w2a8_last_error()
+    assert _gemm(L, g=96) == 2
+    assert _gemm(L, K=4096 + 64) == 2
+    assert _gemm(L, ldq=100) == 2
+    assert _gemm(L, ldo=8) == 2
+    assert _gemm(L, ldr=8) == 2
+    assert _gemm(L, zp_const=7) == 2
+    assert _gemm(L, q=FAKE + 4) == 3
+    assert _gemm(L, ldq=4096 + 8) == 3
+    assert _gemm(L, ldr=18) == 3
+    assert _gemm(L, odt=5) == 4
+    assert _gemm(L, kernel=9) == 4
+    assert _gemm(L, dump=3) == 4
+    assert _gemm(L, dump=1, acc=None) == 1
+    assert _gemm(L, M=64, ldr=64, kernel=_lib.KERNEL_SKINNY) == 7
+    assert _gemm(L, M=64, ldr=64, kernel=_lib.KERNEL_TILED, split=2) == 7
+    # split-K without / with too small a workspace (N = 4096, K = 14336 wants split 4)
+    assert _gemm(L, K=14336, ldq=14336) == 5 and b"workspace" in L.slimk_w2a8_last_error()
+    assert _gemm(L, K=14336, ldq=14336, ws=FAKE, wsb=1024) == 5
+    assert _gemm(L, split=64) == 2                                     # more splits than groups
+
+
+def test_repack_and_act_quant_validation(L):
+    r = L.slimk_w2a8_repack
+    assert r(None, 1024, FAKE, None, 4096, 4096, 128, FAKE, FAKE, None, None) == 1
+    assert r(FAKE, 1024, FAKE, FAKE, 4096, 4096, 128, FAKE, FAKE, None, None) == 1     # zp without zp_r
+    assert r(FAKE, 100, FAKE, None, 4096, 4096, 128, FAKE, FAKE, None, None) == 2      # ldw < K/4
+    assert r(FAKE, 1024, FAKE, None, 4096, 4096, 100, FAKE, FAKE, None, None) == 2
+    assert r(FAKE, 1024, FAKE, None, 4096, 4096, 128, FAKE + 8, FAKE, None, None) == 3
+    a = L.slimk_w2a8_act_quant
+    assert a(None, 4096, 0, 1, 4096, 128, FAKE, 4096, FAKE, FAKE, 4, None) == 1
+    assert a(FAKE, 4096, 0, 0, 4096, 128, FAKE, 4096, FAKE, FAKE, 4, None) == 2
+    assert a(FAKE, 4096, 3, 1, 4096, 128, FAKE, 4096, FAKE, FAKE, 4, None) == 4
+    assert a(FAKE, 100, 0, 1, 4096, 128, FAKE, 4096, FAKE, FAKE, 4, None) == 2
+    assert a(FAKE, 4096 + 4, 0, 1, 4096, 128, FAKE, 4096, FAKE, FAKE, 4, None) == 3
+    assert a(FAKE, 4096, 0, 5, 4096, 128, FAKE, 4096, FAKE, FAKE, 4, None) == 2        # ldr < M
+    assert L.slimk_w2a8_workspace_init(None, 64, None) == 1
+    assert L.slimk_w2a8_workspace_init(FAKE, 0, None) == 0                             # nothing to do
+    assert L.slimk_w2a8_read_probe(FAKE, 24, FAKE, None) == 3
+
+
+def test_last_error_is_thread_local(L):
+    assert _gemm(L, g=96) == 2
+    mine = L.slimk_w2a8_last_error()
+    seen = {}
+
+    def other():
+        seen["before"] = L.slimk_w2a8_last_error()
+        _gemm(L, q=None)
+        seen["after"] = L.slimk_w2a8_last_error()
+
+    t = threading.Thread(target=other)
+    t.start()
+    t.join()
+    assert seen["before"] == b"" and b"NULL" in seen["after"]
+    assert L.slimk_w2a8_last_error() == mine
+
+
+def test_python_entry_refuses_cpu_tensors():
+    import torch
+    from slimkernels_amd import torch as ops
+    with pytest.raises(ValueError, match="no CPU path"):
+        ops.quantize_act_int8(torch.zeros(2, 64, dtype=torch.float16))
+    with pytest.raises(ValueError):
+        ops.wint2_gemm(torch.zeros(2, 64, dtype=torch.float16), torch.zeros(16, 8, dtype=torch.uint8),
+                       torch.zeros(1, 8, dtype=torch.float16))

@@ -1,0 +1,91 @@
+"""GPU parity at the full sizes of the prefill (c3) and 70B-class (c4) configurations.
+
+The CPU oracle cannot form every accumulator of a 4096 x 14336 x 4096 problem in seconds, so
+each case is checked three ways:
+  * sampled tokens: per-token quantisation makes rows independent, so the oracle is run on a
+    random subset of the rows and compared bit for bit (int8 q, int32 group sums, fp16/bf16 out);
+  * a checksum over ALL rows: sum_n acc_sum[m, n] must equal q[m, :] . colsum, where
+    colsum[k] = sum_n (code[n, k] - zp) is formed once on the host in int64;
+  * structure: a zero token gives a zero output row, duplicate tokens give identical rows.
+"""
+import numpy as np
+import pytest
+import torch
+
+from slimkernels_amd import workloads
+import parity_utils as pu
+
+pytestmark = pytest.mark.gpu
+
+
+def _colsum(packed, zero, g):
+    codes = np.empty((packed.shape[0], packed.shape[1] * 4), np.uint8)
+    for i, sh in enumerate((6, 4, 2, 0)):
+        codes[:, i::4] = (packed >> sh) & 3
+    K = codes.shape[1]
+    cs = codes.sum(axis=0, dtype=np.int64)                       # [K]
+    zs = zero.astype(np.int64).sum(axis=1)                       # [G]  sum_n zp[g, n]
+    return cs - np.repeat(zs, g)
+
+
+def _check_case(gpu_ops, oracle, case, sample_rows, seed=0):
+    print("config", case.name, "sampled rows", sample_rows, flush=True)
+    packed, scales, zero = pu.quantized_weight(case)
+    x = workloads.make_activation(case)
+    M = case.M
+    if M >= 8:  # structural rows
+        x[3] = 0
+        x[5] = x[4]
+    bf16 = case.out_dtype == "bfloat16"
+    w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, x)
+    qa = gpu_ops.quantize_act_int8(xd, case.group_size)
+    odt = pu.torch_dtype(case)
+    out = gpu_ops.w2a8_gemm(qa, w, odt)
+    _, acc_sum = gpu_ops.w2a8_gemm(qa, w, odt, dump="sum")
+    torch.cuda.synchronize()
+
+    # ---- checksum over every row (int64 on the host)
+    q_all = qa.q.cpu().numpy()
+    want = q_all.astype(np.int64) @ _colsum(packed, zero, case.group_size)
+    got = acc_sum.sum(dim=1, dtype=torch.int64).cpu().numpy()
+    np.testing.assert_array_equal(got, want)
+
+    # ---- sampled rows against the oracle, bit for bit
+    rng = np.random.default_rng(seed)
+    rows = np.sort(rng.choice(M, size=min(sample_rows, M), replace=False))
+    if M >= 8:
+        rows = np.unique(np.concatenate([rows, [3, 4, 5]]))
+    ref_bits, ref_sum = None, None
+    q_ref, s_ref, _ = oracle.c_act_quant(np.ascontiguousarray(x[rows]), case.group_size)
+    np.testing.assert_array_equal(q_all[rows], q_ref)
+    np.testing.assert_array_equal(qa.s_a.cpu().numpy()[rows], s_ref)
+    ref_bits, ref_sum = oracle.c_gemm_fused(q_ref, s_ref, packed, scales, zero, case.group_size, bf16, want_acc_sum=True)
+    rows_t = torch.from_numpy(rows).cuda()
+    np.testing.assert_array_equal(acc_sum[rows_t].cpu().numpy(), ref_sum)
+    got_bits = pu.out_tensor_bits(out[rows_t])
+    if M > 32:      # tiled kernel: same summation order as the oracle
+        np.testing.assert_array_equal(got_bits, ref_bits)
+    else:           # skinny split-K: the output criterion (1 ULP or rtol 1e-3, plus fp32 re-association noise)
+        g, r = pu.bits_to_f32(got_bits, bf16), pu.bits_to_f32(ref_bits, bf16)
+        # bound the re-association noise by G * 2^-24 * s_a * sum_g |acc_g| * scale <= G * 2^-24 * s_a * K * 127 * 3 * max scale
+        smax = float(scales.astype(np.float32).max())
+        bound = (case.K // case.group_size) * 2.0 ** -24 * s_ref[:, None] * (np.abs(q_ref).astype(np.float64).sum(axis=1)[:, None] * 2 * smax)
+        pu.assert_out_close(got_bits, ref_bits, bf16, bound, case.name)
+    # ---- structure
+    if M >= 8:
+        ob = pu.out_tensor_bits(out[3:6])
+        assert not (ob[0] & 0x7fff).any(), "zero token must give a zero output row"
+        np.testing.assert_array_equal(ob[1], ob[2])
+
+
+@pytest.mark.parametrize("N,K", [(14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("M", [512, 2048, 4096])
+def test_config_c3_prefill(gpu_ops, oracle, N, K, M):
+    _check_case(gpu_ops, oracle, workloads.Case("c3", M, N, K), sample_rows=48 if M > 512 else 96)
+
+
+@pytest.mark.parametrize("N,K", [(28672, 8192), (8192, 28672)])
+@pytest.mark.parametrize("M", [1, 16, 128, 2048])
+def test_config_c4_large(gpu_ops, oracle, N, K, M):
+    case = workloads.Case("c4", M, N, K, group_size=64, out_dtype="bfloat16")
+    _check_case(gpu_ops, oracle, case, sample_rows=16)

@@ -167,3 +167,34 @@ def test_wint2_gemm_and_linear_entry_points(gpu_ops, oracle):
     y2 = lin(xd.reshape(1, 5, 256))
     assert y2.shape == (1, 5, 128)
     np.testing.assert_array_equal(pu.out_tensor_bits(y2.reshape(5, 128)), pu.out_tensor_bits(y))
+
+
+def test_grouped_launch_matches_single_launches(gpu_ops, oracle):
+    """One grouped launch over problems of different M, N, K == the same problems launched one by one
+    with split_k = 1 (same kernel body, same summation order: bit-identical), and == the oracle."""
+    shapes = [(1, 256, 512), (5, 100, 1024), (16, 512, 256), (32, 192, 768), (2, 64, 2048)]
+    probs, singles, refs = [], [], []
+    for i, (M, N, K) in enumerate(shapes):
+        case = pu.small_case(M, N, K, 128, "sym", seed=50 + i)
+        packed, scales, zero = pu.quantized_weight(case)
+        x = workloads.make_activation(case)
+        w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, x)
+        qa = gpu_ops.quantize_act_int8(xd, 128)
+        probs.append((qa, w))
+        singles.append(gpu_ops.w2a8_gemm(qa, w, kernel="skinny", split_k=1))
+        refs.append((oracle.reference_forward(x, packed, scales, zero, 128), scales))
+    outs = gpu_ops.w2a8_gemm_grouped(probs)
+    torch.cuda.synchronize()
+    for o, s, (ref, scales) in zip(outs, singles, refs):
+        np.testing.assert_array_equal(pu.out_tensor_bits(o), pu.out_tensor_bits(s))
+        pu.assert_out_close(pu.out_tensor_bits(o), ref["out_bits"], False,
+                            pu.reorder_bound(ref["acc"], scales, ref["s_a"]), "grouped")
+    # asymmetric group, bf16
+    case = pu.small_case(7, 130, 512, 64, "asym", seed=77, out_dtype="bfloat16")
+    packed, scales, zero = pu.quantized_weight(case)
+    x = workloads.make_activation(case)
+    w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, x)
+    qa = gpu_ops.quantize_act_int8(xd, 64)
+    (o,) = gpu_ops.w2a8_gemm_grouped([(qa, w)], torch.bfloat16)
+    ref = oracle.reference_forward(x, packed, scales, zero, 64, out_bf16=True)
+    pu.assert_out_close(pu.out_tensor_bits(o), ref["out_bits"], True, pu.reorder_bound(ref["acc"], scales, ref["s_a"]), "grouped asym")
