@@ -37,10 +37,11 @@ HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0       # MI355X dense int8 MFMA, published (5.0 POP/s)
 COLD_FOOTPRINT = 640 << 20    # bytes of distinct weight copies between two uses of one copy
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this command, scaled by what the same counters read for the read-probe kernel of known size.
-# None until measured.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = None
+# HBM bytes per launch of the dominant kernel from two rocprofv3 --pmc runs of
+# `python3 bench.py --skip-detail` (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same
+# counter reads for this file's 256 MiB calibration read (read_probe_kernel: 131080 -> x2.0) and
+# calibration fill (fill_zero_kernel: 262144 -> x1.0):  (114780 * 2.0 + 2898 * 1.0) KiB.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = int((114780 * 2.0 + 2898 * 1.0) * 1024)
 
 
 def main():
@@ -165,6 +166,16 @@ def main():
         e1.record()
         torch.cuda.synchronize()
         return time.perf_counter() - t0, e0.elapsed_time(e1)
+
+    # counter calibration: a plain read and a plain fill of known size (256 MiB each), so that a
+    # rocprofv3 --pmc run of this command can scale FETCH_SIZE / WRITE_SIZE of the GEMM kernel
+    cal = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    for _ in range(3):
+        _lib.check(L.slimk_w2a8_workspace_init(cal.data_ptr(), cal.numel(), torch.cuda.current_stream().cuda_stream))
+        _lib.check(L.slimk_w2a8_read_probe(cal.data_ptr(), cal.numel(), sink.data_ptr(), torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    del cal
 
     wall, ev_ms = timed_run(grouped=True)
 

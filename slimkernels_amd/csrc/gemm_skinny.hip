@@ -24,15 +24,14 @@
 namespace w2a8 {
 
 // NW = wavefronts per workgroup (the split of K inside a workgroup).
-constexpr int kDepth = 4;  // ring depth in steps = steps per metadata chunk = granule of the K partition
-
-template <int MB, int NW>
+// D = ring depth in steps = steps per metadata chunk = granule of the K partition (4 or 8).
+template <int MB, int NW, int D>
 struct SkinnySmem {
     union {
         struct {
-            uint16_t scale[NW][kDepth][16][4];  // [wave][group in chunk][col][sub-block]
-            uint8_t zp[NW][kDepth][16][4];
-            int32_t rowsum[NW][kDepth][MB * 16];
+            uint16_t scale[NW][D][16][4];  // [wave][group in chunk][col][sub-block]
+            uint8_t zp[NW][D][16][4];
+            int32_t rowsum[NW][D][MB * 16];
         } meta;
         float red[NW][MB * 16][kStripN + 1];
     };
@@ -43,9 +42,9 @@ struct SkinnySmem {
 // block is a real token, so three quarters of the drain arithmetic can be dropped).
 // ZM = zero-point mode: 0 uniform zero-point 2 (the symmetric levels; folded with shifts),
 // 1 any other uniform zero-point, 2 per-(group, channel) zero-points read from zp_r.
-template <int MB, int J, int GS, int NW, int ZM, bool DUMP, typename OutT>
+template <int MB, int J, int GS, int NW, int ZM, bool DUMP, typename OutT, int kDepth>
 __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip, const int split,
-                                            SkinnySmem<MB, NW>& sm) {
+                                            SkinnySmem<MB, NW, kDepth>& sm) {
     constexpr bool ASYM = ZM == 2;
     constexpr bool SYM2 = ZM == 0;
     constexpr int kThreads = NW * 64;
@@ -63,8 +62,8 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
 #pragma unroll
     for (int i = 0; i < kOutPerThread; ++i) sa[i] = p.s_a[min((tid + kThreads * i) >> 6, p.M - 1)];
 
-    // Step range of this workgroup (groups_per_split is a multiple of kGroupsPerChunk), then of this
-    // wave, in whole chunks of kDepth steps; only the very last chunk of K can be ragged.
+    // Step range of this workgroup (groups_per_split is a multiple of a 4-step chunk's groups), then
+    // of this wave, in whole chunks of kDepth steps; only a range's last chunk can be ragged.
     const int wg_s0 = min(split * p.groups_per_split, p.G) * GS;
     const int wg_s1 = min((split + 1) * p.groups_per_split, p.G) * GS;
     const int wg_chunks = (wg_s1 - wg_s0 + kDepth - 1) / kDepth;
@@ -231,6 +230,7 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
 
     // ---- meet the workgroup's waves in LDS (the metadata area is dead once every wave is here)
     __syncthreads();
+
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
@@ -298,8 +298,8 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
 
 template <int MB, int J, int GS, int NW, int ZM, bool DUMP, typename OutT>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const GemmParams p) {
-    __shared__ __attribute__((aligned(16))) SkinnySmem<MB, NW> sm;
-    skinny_body<MB, J, GS, NW, ZM, DUMP, OutT>(p, blockIdx.x, blockIdx.y, sm);
+    __shared__ __attribute__((aligned(16))) SkinnySmem<MB, NW, 4> sm;
+    skinny_body<MB, J, GS, NW, ZM, DUMP, OutT, 4>(p, blockIdx.x, blockIdx.y, sm);
 }
 
 // Several independent skinny GEMMs in one launch: workgroup ids are cut into runs, one run per
@@ -313,17 +313,17 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const GemmParams p) {
 template <int GS, int ZM, typename OutT>
 __global__ __launch_bounds__(256, SLIMK_GROUPED_WAVES_PER_SIMD) void skinny_grouped_kernel(const GroupedParams gp) {
     __shared__ __attribute__((aligned(16))) union {
-        SkinnySmem<1, 4> one;
-        SkinnySmem<2, 4> two;
+        SkinnySmem<1, 4, 4> one;
+        SkinnySmem<2, 4, 4> two;
     } sm;
     const int wg = blockIdx.x;
     int i = 0;
     while (i + 1 < gp.count && wg >= gp.wg_begin[i + 1]) ++i;
     const GemmParams& p = gp.prob[i];
     const int strip = wg - gp.wg_begin[i];
-    if (p.M == 1) skinny_body<1, 1, GS, 4, ZM, false, OutT>(p, strip, 0, sm.one);
-    else if (p.M <= 16) skinny_body<1, 4, GS, 4, ZM, false, OutT>(p, strip, 0, sm.one);
-    else skinny_body<2, 4, GS, 4, ZM, false, OutT>(p, strip, 0, sm.two);
+    if (p.M == 1) skinny_body<1, 1, GS, 4, ZM, false, OutT, 4>(p, strip, 0, sm.one);
+    else if (p.M <= 16) skinny_body<1, 4, GS, 4, ZM, false, OutT, 4>(p, strip, 0, sm.one);
+    else skinny_body<2, 4, GS, 4, ZM, false, OutT, 4>(p, strip, 0, sm.two);
 }
 
 template <int MB, int J, int GS, int NW, int ZM, bool DUMP>
