@@ -41,6 +41,15 @@ int check_kg(int K, int group_size) {
     return SLIMK_OK;
 }
 
+// The kernels address weights and activations through 32-bit buffer offsets.
+int check_extent(int M, int N, int K, int ldq) {
+    const size_t wbytes = (size_t)((N + w2a8::kStripN - 1) / w2a8::kStripN) * (size_t)(K / w2a8::kStepK) * (w2a8::kUnitDwords * 4);
+    const size_t qbytes = (size_t)M * (size_t)ldq;
+    if (wbytes > 0x7fffffffu || qbytes > 0x7fffffffu)
+        return fail(SLIMK_ERR_UNSUPPORTED, "repacked weights (%zu bytes) or activations (%zu bytes) exceed 2 GiB", wbytes, qbytes);
+    return SLIMK_OK;
+}
+
 bool shape_ok(int K, int group_size) {
     return K > 0 && K % 64 == 0 && (group_size == 64 || group_size == 128 || group_size == 256) &&
            K % group_size == 0;
@@ -101,7 +110,8 @@ int skinny_waves(int M, int split) {
     }();
     if (forced) return forced;
     // split runs are the long-K ones: more waves per workgroup keep more loads in flight per CU
-    if (split > 1) return M <= 16 ? 16 : 8;
+    (void)M;
+    if (split > 1) return 16;
     return 4;
 }
 
@@ -139,8 +149,9 @@ size_t slimk_w2a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int 
     if (split_k <= 0) split_k = auto_split(M, N, K, group_size, kern);
     if (split_k <= 1 || kern != SLIMK_KERNEL_SKINNY) return 0;
     const int strips = strips_of(N);
-    const size_t tile = (size_t)(M <= 16 ? 16 : 32) * w2a8::kStripN;
-    return counter_bytes(strips) + (size_t)split_k * strips * tile * sizeof(float);
+    const int mblocks = (M + 15) / 16;  // one tile and one arrival counter per (strip, block of 16 rows)
+    const size_t tile = (size_t)16 * w2a8::kStripN;
+    return counter_bytes(strips * mblocks) + (size_t)split_k * strips * mblocks * tile * sizeof(float);
 }
 
 int slimk_w2a8_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
@@ -199,6 +210,7 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
     if (dump_mode != SLIMK_DUMP_NONE && !acc_dump) return fail(SLIMK_ERR_NULL_POINTER, "gemm: dump_mode set but acc_dump is NULL");
     if (ldq < K || ldo < N || ldr < M) return fail(SLIMK_ERR_BAD_SHAPE, "gemm: ldq=%d, ldo=%d or ldr=%d too small", ldq, ldo, ldr);
     if (zp_const < 0 || zp_const > 3) return fail(SLIMK_ERR_BAD_SHAPE, "zp_const=%d must be 0..3", zp_const);
+    if (int rc = check_extent(M, N, K, ldq)) return rc;
     if (!aligned16(q) || ldq % 16 != 0 || !aligned16(rowsum) || ldr % 4 != 0 || !aligned16(w_r) ||
         !aligned16(s_r) || (zp_r && !aligned16(zp_r)))
         return fail(SLIMK_ERR_MISALIGNED, "gemm: q, rowsum, w_r, s_r, zp_r must be 16-byte aligned; ldq %% 16 == 0; ldr %% 4 == 0");
@@ -230,7 +242,7 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
             return fail(SLIMK_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, need);
         if (!aligned16(workspace)) return fail(SLIMK_ERR_MISALIGNED, "workspace must be 16-byte aligned");
         p.ws_counter = reinterpret_cast<unsigned*>(workspace);
-        p.ws_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counter_bytes(p.strips));
+        p.ws_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counter_bytes(p.strips * ((M + 15) / 16)));
     }
 
     hipStream_t st = (hipStream_t)stream;
@@ -264,6 +276,9 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
     w2a8::GroupedParams gp{};
     gp.count = count;
     int zm = -1, wgs = 0;
+    // A workgroup of eight waves covers 8 strips x all of K, 4 strips x 2 halves or 2 strips x 4 quarters:
+    // whichever keeps a wave's run at roughly 48..96 steps.
+    const auto kparts_of = [](int steps) { return steps > 192 ? 4 : (steps > 96 ? 2 : 1); };
     for (int i = 0; i < count; ++i) {
         const slimk_w2a8_problem& pr = problems[order[i]];
         if (!pr.q || !pr.s_a || !pr.rowsum || !pr.w_r || !pr.s_r || !pr.out)
@@ -274,12 +289,13 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
         if (pr.ldq < pr.K || pr.ldo < pr.N || pr.ldr < pr.M)
             return fail(SLIMK_ERR_BAD_SHAPE, "gemm_grouped: problem %d: a leading dimension is too small", order[i]);
         if (pr.zp_const < 0 || pr.zp_const > 3) return fail(SLIMK_ERR_BAD_SHAPE, "gemm_grouped: problem %d: zp_const=%d", order[i], pr.zp_const);
+        if (int rc = check_extent(pr.M, pr.N, pr.K, pr.ldq)) return rc;
         if (!aligned16(pr.q) || pr.ldq % 16 != 0 || !aligned16(pr.rowsum) || pr.ldr % 4 != 0 || !aligned16(pr.w_r) ||
             !aligned16(pr.s_r) || (pr.zp_r && !aligned16(pr.zp_r)) || (reinterpret_cast<uintptr_t>(pr.out) & 1u))
             return fail(SLIMK_ERR_MISALIGNED, "gemm_grouped: problem %d breaks an alignment rule of slimk_w2a8_gemm", order[i]);
-        const int this_zm = pr.zp_r ? 2 : (pr.zp_const == 2 ? 0 : 1);
+        const int this_zm = pr.zp_r ? 1 : 0;
         if (zm >= 0 && this_zm != zm)
-            return fail(SLIMK_ERR_UNSUPPORTED, "gemm_grouped: problems mix zero-point modes");
+            return fail(SLIMK_ERR_UNSUPPORTED, "gemm_grouped: problems mix uniform and per-group zero-points");
         zm = this_zm;
         w2a8::GemmParams& g = gp.prob[i];
         g.q = pr.q; g.s_a = pr.s_a; g.rowsum = pr.rowsum; g.w_r = pr.w_r; g.s_r = pr.s_r; g.zp_r = pr.zp_r;
@@ -288,10 +304,14 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
         g.strips = strips_of(pr.N); g.zp_const = pr.zp_const;
         g.split = 1; g.groups_per_split = groups_per_split(g.G, group_size, 1);
         gp.wg_begin[i] = wgs;
-        wgs += g.strips;
+        gp.kparts[i] = kparts_of(g.steps);
+        // units (sets of 8, 4 or 2 strips) in whole sets of eight, times the row blocks of 16 tokens
+        const int per_unit = 8 / gp.kparts[i];
+        const int units = (g.strips + per_unit - 1) / per_unit;
+        wgs += (units + 7) / 8 * 8 * ((pr.M + 15) / 16);
     }
     gp.wg_begin[count] = wgs;
-    return hip_result(w2a8::launch_skinny_grouped(gp, group_size / w2a8::kStepK, zm, out_dtype == SLIMK_BF16,
+    return hip_result(w2a8::launch_skinny_grouped(gp, group_size / w2a8::kStepK, zm == 1, out_dtype == SLIMK_BF16,
                                                   (hipStream_t)stream),
                       "grouped skinny gemm");
 }

@@ -23,72 +23,117 @@
 
 namespace w2a8 {
 
-// NW = wavefronts per workgroup (the split of K inside a workgroup).
-// D = ring depth in steps = steps per metadata chunk = granule of the K partition (4 or 8).
-template <int MB, int NW, int D>
+constexpr int kDepth = 4;  // ring depth in steps = steps per metadata chunk = granule of the K partition
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+
+// NWP = wavefronts per workgroup.  Each wave owns a private metadata area; the reduction tile
+// reuses the same memory once every wave has left its loop.
+struct SkinnyMeta {
+    uint16_t scale[kDepth][16][4];  // [group in chunk][col][sub-block]
+    uint8_t zp[kDepth][16][4];
+    int32_t rowsum[kDepth][16];
+};
+
+template <int NWP>
 struct SkinnySmem {
     union {
-        struct {
-            uint16_t scale[NW][D][16][4];  // [wave][group in chunk][col][sub-block]
-            uint8_t zp[NW][D][16][4];
-            int32_t rowsum[NW][D][MB * 16];
-        } meta;
-        float red[NW][MB * 16][kStripN + 1];
+        SkinnyMeta meta[NWP];
+        float red[NWP][16][kStripN + 1];
     };
     int last;
 };
 
-// J = live rows per lane of a D fragment: 4 in general, 1 when M == 1 (only row 0 of the 16x16
-// block is a real token, so three quarters of the drain arithmetic can be dropped).
-// ZM = zero-point mode: 0 uniform zero-point 2 (the symmetric levels; folded with shifts),
-// 1 any other uniform zero-point, 2 per-(group, channel) zero-points read from zp_r.
-template <int MB, int J, int GS, int NW, int ZM, bool DUMP, typename OutT, int kDepth>
-__device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip, const int split,
-                                            SkinnySmem<MB, NW, kDepth>& sm) {
-    constexpr bool ASYM = ZM == 2;
-    constexpr bool SYM2 = ZM == 0;
-    constexpr int kThreads = NW * 64;
+// One wave's share of one strip and one block of 16 token rows (a problem with 17..32 rows is
+// run as two row blocks by two sets of waves: the second read of the weights comes from L2, and
+// the small register footprint of a single block is what lets four waves share a SIMD).
+//   J     live rows per lane of a D fragment: 4 in general, 1 when M == 1 (only row 0 of the 16x16
+//         block is a real token, so three quarters of the drain arithmetic are dropped)
+//   GS    steps per scale group
+//   NWK   waves that split the workgroup's K range among them (1: the wave owns all of it and
+//         stores its results itself; NWP: all the workgroup's waves, meeting in LDS)
+//   ASYM  per-(group, channel) zero-points from zp_r instead of the uniform zp_const
+//   DUMP  verification build: exact int32 group sums are written out
+//
+// Zero-points.  The MFMA operand of field p is code * 4^p (p < 3) or 64 * (code - 2) (p = 3), so
+// a group's true sum is raw - zpe * rowsum with zpe = zp * 4^p resp. (zp - 2) * 64.  The timed
+// kernels never form that integer: the term -zpe * scale * rowsum is itself a small matrix
+// product over the groups (16 tokens x 16 channels x up to 4 groups of a chunk) and goes through
+// one v_mfma_f32_16x16x4_f32 per chunk and sub-block, accumulating straight into the fp32 running
+// sums (same D layout as the int8 MFMA).  The verification build folds it in integers instead.
+template <int J, int GS, int NWK, int NWP, bool ASYM, bool DUMP, typename OutT>
+__device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip, const int split, const int mblk,
+                                            const int kwave, const int pwave, SkinnySmem<NWP>& sm) {
+    constexpr int MB = 1;
+    static_assert(NWK == 1 || NWK == NWP, "K is split over one wave or over the whole workgroup");
+    constexpr int kThreads = NWP * 64;
     constexpr int kGroupsPerChunk = kDepth / GS;
-    constexpr int kTile = MB * 16 * kStripN;  // elements of the workgroup's output tile
-    constexpr int kOutPerThread = (kTile + kThreads - 1) / kThreads;
+    constexpr int kTile = MB * 16 * kStripN;                 // elements of a strip's output tile (workspace pitch)
+    constexpr int kLive = (J == 1 ? 1 : MB * 16) * kStripN;  // elements of it that can hold real tokens
+    constexpr int kOutPerThread = (kLive + kThreads - 1) / kThreads;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps ranges and bases in SGPRs
     const int col = lane & 15, quad = lane >> 4;
+    SkinnyMeta& meta = sm.meta[pwave];
 
-    // token scales for the epilogue (element e = tid + kThreads*i -> row e >> 6), fetched first
-    float sa[kOutPerThread];
+    // this row block's view of the per-token operands
+    const int m0 = mblk * 16;
+    const int M = min(16, p.M - m0);
+    const int8_t* const qp = p.q + (size_t)m0 * p.ldq;
+    const float* const sap = p.s_a + m0;
+    const int32_t* const rsp = p.rowsum + m0;
+    const int ldr = p.ldr - m0;
+    uint16_t* const out = reinterpret_cast<uint16_t*>(p.out) + (size_t)m0 * p.ldo;
+    const int mblocks = (p.M + 15) >> 4;
+    const int tile_id = strip * mblocks + mblk;  // index of this (strip, row block) in the split-K workspace
+
+    // token scales for the epilogue, fetched first
+    float sa[NWK == 1 ? MB * J : kOutPerThread];
+    if (NWK == 1) {  // this wave stores D fragments itself: rows mb*16 + quad*4 + j
 #pragma unroll
-    for (int i = 0; i < kOutPerThread; ++i) sa[i] = p.s_a[min((tid + kThreads * i) >> 6, p.M - 1)];
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int j = 0; j < J; ++j) sa[mb * J + j] = sap[min(mb * 16 + quad * 4 + j, M - 1)];
+    } else {  // element e = tid + kThreads*i of the reduced tile -> row e >> 6
+#pragma unroll
+        for (int i = 0; i < kOutPerThread; ++i) sa[i] = sap[min((tid + kThreads * i) >> 6, M - 1)];
+    }
 
-    // Step range of this workgroup (groups_per_split is a multiple of a 4-step chunk's groups), then
-    // of this wave, in whole chunks of kDepth steps; only a range's last chunk can be ragged.
+    // Step range of this workgroup (groups_per_split is a multiple of a chunk's groups), then of this
+    // wave, in whole chunks of kDepth steps; only a range's last chunk can be ragged.
     const int wg_s0 = min(split * p.groups_per_split, p.G) * GS;
     const int wg_s1 = min((split + 1) * p.groups_per_split, p.G) * GS;
     const int wg_chunks = (wg_s1 - wg_s0 + kDepth - 1) / kDepth;
-    const int per_wave = (wg_chunks + NW - 1) / NW;
-    const int s0 = min(wg_s0 + wave * per_wave * kDepth, wg_s1);
+    const int per_wave = (wg_chunks + NWK - 1) / NWK;
+    const int s0 = min(wg_s0 + kwave * per_wave * kDepth, wg_s1);
     const int s1 = min(s0 + per_wave * kDepth, wg_s1);
     const int g1 = s1 / GS;
-    const int s_last = s1 - 1;
+    const int len = s1 - s0;
+    auto stepof = [&](int it) { return s0 + min(it, len - 1); };  // iterations past the end repeat the last step
 
-    // Addressing: wave-uniform 64-bit bases (SGPRs) plus 32-bit per-lane offsets.  No load is
-    // predicated or sits under a branch: out-of-range rows, groups and steps are clamped onto valid
-    // addresses instead, so the number of loads in flight is the same on every path and the
-    // s_waitcnt the compiler places before each use waits for exactly that load (a token row >= M
-    // only ever feeds output rows >= M, which are not stored; a clamped step or group is never used).
-    const char* wb = reinterpret_cast<const char*>(p.w_r) + (size_t)strip * (kUnitDwords * 4);
-    const size_t wstride = (size_t)p.strips * (kUnitDwords * 4);  // bytes between consecutive steps of a strip
+    // Addressing: buffer descriptors with a per-lane offset fixed for the whole kernel and a scalar
+    // offset per step, so no vector ALU work goes into addresses.  No load is predicated or sits
+    // under a branch: out-of-range rows, groups and steps are clamped onto valid ones instead, so the
+    // number of loads in flight is the same on every path and the s_waitcnt the compiler places
+    // before each use waits for exactly that load (a token row >= M only ever feeds output rows >= M,
+    // which are not stored; a clamped step or group is never used).
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(p.w_r), 0, (int)((size_t)p.strips * p.steps * (kUnitDwords * 4)), 0x00020000);
+    const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int8_t*>(qp), 0, (int)((size_t)(M - 1) * p.ldq + p.K), 0x00020000);
+    const uint32_t wstride = (uint32_t)p.strips * (kUnitDwords * 4);  // bytes between consecutive steps of a strip
+    const uint32_t wbase = (uint32_t)strip * (kUnitDwords * 4);
     const uint32_t wlane = lane * 16;
-    const char* qb = reinterpret_cast<const char*>(p.q);
     uint32_t aoff[MB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) aoff[mb] = (uint32_t)min(mb * 16 + col, p.M - 1) * (uint32_t)p.ldq + quad * 16;
+    for (int mb = 0; mb < MB; ++mb) aoff[mb] = (uint32_t)min(mb * 16 + col, M - 1) * (uint32_t)p.ldq + quad * 16;
 
     // ---- metadata prefetch registers: one chunk (kGroupsPerChunk groups) ahead
-    v4i m_scale;     // scales: 4 groups x 128 B = 512 B per wave: lanes 0..31, 16 B each
-    v4i m_zp;        // zero-points: 4 groups x 64 B: lanes 0..15
+    v4i m_scale;     // scales: up to 4 groups x 128 B = 512 B per wave: lanes 0..31, 16 B each
+    v4i m_zp;        // zero-points: up to 4 groups x 64 B: lanes 0..15
     v4i m_rs[MB];    // row sums: lane -> (group lane >> 2, rows 4*(lane & 3) ..): lanes 0..15
     auto fetch_meta = [&](int gfirst) {  // groups gfirst .. gfirst + kGroupsPerChunk - 1, clamped to g1 - 1
         const size_t sgi = (size_t)min(gfirst + (lane >> 3), g1 - 1) * p.strips + strip;
@@ -97,103 +142,132 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
         if (ASYM)
             m_zp = *reinterpret_cast<const v4i*>(reinterpret_cast<const char*>(p.zp_r) +
                                                  ((size_t)gq * p.strips + strip) * 64 + (lane & 3) * 16);
-        const int32_t* rp = p.rowsum + (size_t)gq * p.ldr;
+        const int32_t* rp = rsp + (size_t)gq * p.ldr;
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-            m_rs[mb] = *reinterpret_cast<const v4i*>(rp + min(mb * 16 + (lane & 3) * 4, p.ldr - 4));
+            m_rs[mb] = *reinterpret_cast<const v4i*>(rp + min(mb * 16 + (lane & 3) * 4, ldr - 4));
     };
-    auto park_meta = [&]() {
-        if (lane < kDepth * 8)
-            *reinterpret_cast<v4i*>(reinterpret_cast<char*>(&sm.meta.scale[wave][0][0][0]) + lane * 16) = m_scale;
+    auto park_meta = [&](int gfirst) {  // the registers hold groups gfirst ..
+        // a group past the end of the range (ragged last chunk) gets zero scales: it then adds nothing
+        // (decided here, where the loaded registers are first needed anyway, not at the load)
+        if (gfirst + (lane >> 3) >= g1) m_scale = v4i{0, 0, 0, 0};
+        if (lane < kDepth * 8) *reinterpret_cast<v4i*>(reinterpret_cast<char*>(&meta.scale[0][0][0]) + lane * 16) = m_scale;
         if (lane < kDepth * 4) {
-            if (ASYM) *reinterpret_cast<v4i*>(reinterpret_cast<char*>(&sm.meta.zp[wave][0][0][0]) + lane * 16) = m_zp;
+            if (ASYM) *reinterpret_cast<v4i*>(reinterpret_cast<char*>(&meta.zp[0][0][0]) + lane * 16) = m_zp;
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
-                *reinterpret_cast<v4i*>(&sm.meta.rowsum[wave][lane >> 2][mb * 16 + (lane & 3) * 4]) = m_rs[mb];
+                *reinterpret_cast<v4i*>(&meta.rowsum[lane >> 2][mb * 16 + (lane & 3) * 4]) = m_rs[mb];
         }
     };
 
     // ---- weight / activation register ring
-    v4i wring[kDepth];
-    v4i aring[kDepth][MB];
+    v4u wring[kDepth];
+    v4u aring[kDepth][MB];
     auto issue = [&](int slot, int step) {  // step is wave-uniform
-        wring[slot] = *reinterpret_cast<const v4i*>(wb + (size_t)step * wstride + wlane);
+        wring[slot] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane, step * wstride + wbase, 0);
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-            aring[slot][mb] = *reinterpret_cast<const v4i*>(qb + (size_t)step * kStepK + aoff[mb]);
+            aring[slot][mb] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, aoff[mb], step * kStepK, 0);
     };
 
-    float t[MB][4][4];
+    // running sums, in units of 4^p (sub-block p < 3) resp. 64 (p = 3) times the result
+    v4f t[MB][4];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-        for (int pp = 0; pp < 4; ++pp)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) t[mb][pp][j] = 0.0f;
+        for (int pp = 0; pp < 4; ++pp) t[mb][pp] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // uniform zero-point in operand units, negated
+    const float czu[4] = {-(float)p.zp_const, -(float)(p.zp_const * 4), -(float)(p.zp_const * 16),
+                          -(float)((p.zp_const - 2) * 64)};
 
     if (s0 < s1) {
         // Same issue order as inside the loop (metadata first, then the ring), fenced, so that the
         // wait counts the compiler derives for the loop head hold on the entry path as well.
-        fetch_meta(s0 / GS);
+        fetch_meta(stepof(0) / GS);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < kDepth; ++i) issue(i, min(s0 + i, s_last));
+        for (int i = 0; i < kDepth; ++i) issue(i, stepof(i));
         __builtin_amdgcn_sched_barrier(0);
 
         v4i acc[MB][4];
-        v4i nrs[MB];
-        int zps[4];
-        float sc[4];
+        v4h sc;          // the group's four sub-block scales, kept in fp16: the drain's fma reads them as such
+        v4i nrs[MB];     // verification build only
+        int zps[4];      // verification build only
 
-        for (int cbase = s0; cbase < s1; cbase += kDepth) {
-            const int gchunk = cbase / GS;
-            park_meta();                              // this chunk's metadata: registers -> LDS
-            fetch_meta(gchunk + kGroupsPerChunk);     // next chunk's metadata: global -> registers
+        for (int it = 0; it < len; it += kDepth) {
+            const int gchunk = stepof(it) / GS;
+            park_meta(gchunk);                        // this chunk's metadata: registers -> LDS
+            fetch_meta(stepof(it + kDepth) / GS);     // next chunk's metadata: global -> registers
             __builtin_amdgcn_sched_barrier(0);
+
+            if (!DUMP) {
+                // zero-point term of the whole chunk: lane (col, quad) supplies token col / channel col of
+                // group `quad` of the chunk; lanes whose quad is past the chunk's groups supply zero
+                const int gi = quad % kGroupsPerChunk;
+                const bool on = quad < kGroupsPerChunk;
+                const v4h zs = *reinterpret_cast<const v4h*>(&meta.scale[gi][col][0]);
+                float zb[4];
+                if (ASYM) {
+                    const uint32_t zraw = *reinterpret_cast<const uint32_t*>(&meta.zp[gi][col][0]);
+                    zb[0] = -(float)(zraw & 0xffu) * (float)zs[0];
+                    zb[1] = -4.0f * (float)((zraw >> 8) & 0xffu) * (float)zs[1];
+                    zb[2] = -16.0f * (float)((zraw >> 16) & 0xffu) * (float)zs[2];
+                    zb[3] = (128.0f - 64.0f * (float)(zraw >> 24)) * (float)zs[3];
+                } else {
+#pragma unroll
+                    for (int pp = 0; pp < 4; ++pp) zb[pp] = czu[pp] * (float)zs[pp];
+                }
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    const int rsi = meta.rowsum[gi][mb * 16 + col];
+                    const float rsf = on ? (float)rsi : 0.0f;
+#pragma unroll
+                    for (int pp = 0; pp < 4; ++pp)
+                        if (ASYM || pp < 3 || p.zp_const != 2)  // uniform zero-point 2: field 3 is already centred
+                            t[mb][pp] = __builtin_amdgcn_mfma_f32_16x16x4f32(rsf, zb[pp], t[mb][pp], 0, 0, 0);
+                }
+            }
+
 #pragma unroll
             for (int i = 0; i < kDepth; ++i) {
-                const int step = cbase + i;
                 const int gi = i / GS;  // group within the chunk
                 if (i % GS == 0) {
-                    // a group past the end of K (ragged last chunk) is neutralised by a zero scale
-                    const float live = (gchunk + gi < g1) ? 1.0f : 0.0f;
-                    const uint2 sraw = *reinterpret_cast<const uint2*>(&sm.meta.scale[wave][gi][col][0]);
-                    sc[0] = half_bits_to_float((uint16_t)(sraw.x & 0xffffu)) * live;
-                    sc[1] = half_bits_to_float((uint16_t)(sraw.x >> 16)) * (0.25f * live);
-                    sc[2] = half_bits_to_float((uint16_t)(sraw.y & 0xffffu)) * (0.0625f * live);
-                    sc[3] = half_bits_to_float((uint16_t)(sraw.y >> 16)) * (0.015625f * live);
-                    // effective zero-points in operand units: zp * 4^p, (zp - 2) * 64 for the sign-bit field
-                    if (ASYM) {
-                        const uint32_t zraw = *reinterpret_cast<const uint32_t*>(&sm.meta.zp[wave][gi][col][0]);
-                        zps[0] = (int)(zraw & 0xffu);
-                        zps[1] = (int)((zraw >> 8) & 0xffu) * 4;
-                        zps[2] = (int)((zraw >> 16) & 0xffu) * 16;
-                        zps[3] = ((int)(zraw >> 24) - 2) * 64;
-                    } else {
-                        zps[0] = p.zp_const;
-                        zps[1] = p.zp_const * 4;
-                        zps[2] = p.zp_const * 16;
-                        zps[3] = (p.zp_const - 2) * 64;
-                    }
-                    // -rowsum of the lane's D rows: the zero-point term -zp * rowsum is folded in at the drain
+                    sc = *reinterpret_cast<const v4h*>(&meta.scale[gi][col][0]);
+                    if (DUMP) {
+                        // effective zero-points in operand units: zp * 4^p, (zp - 2) * 64 for the sign-bit field
+                        if (ASYM) {
+                            const uint32_t zraw = *reinterpret_cast<const uint32_t*>(&meta.zp[gi][col][0]);
+                            zps[0] = (int)(zraw & 0xffu);
+                            zps[1] = (int)((zraw >> 8) & 0xffu) * 4;
+                            zps[2] = (int)((zraw >> 16) & 0xffu) * 16;
+                            zps[3] = ((int)(zraw >> 24) - 2) * 64;
+                        } else {
+                            zps[0] = p.zp_const;
+                            zps[1] = p.zp_const * 4;
+                            zps[2] = p.zp_const * 16;
+                            zps[3] = (p.zp_const - 2) * 64;
+                        }
 #pragma unroll
-                    for (int mb = 0; mb < MB; ++mb)
-                        nrs[mb] = -*reinterpret_cast<const v4i*>(&sm.meta.rowsum[wave][gi][mb * 16 + quad * 4]);
+                        for (int mb = 0; mb < MB; ++mb)
+                            nrs[mb] = -*reinterpret_cast<const v4i*>(&meta.rowsum[gi][mb * 16 + quad * 4]);
+                    }
                 }
 
 #pragma unroll
                 for (int pp = 0; pp < 4; ++pp) {
-                    const v4i b = wring[i] & (int)(0x03030303u << (2 * pp));
+                    const v4i b = __builtin_bit_cast(v4i, wring[i] & (0x03030303u << (2 * pp)));
 #pragma unroll
                     for (int mb = 0; mb < MB; ++mb)  // the first step of a group starts from C = 0 (inline constant)
-                        acc[mb][pp] = mfma_i8_16x16x64(aring[i][mb], b, (i % GS == 0) ? v4i{0, 0, 0, 0} : acc[mb][pp]);
+                        acc[mb][pp] = mfma_i8_16x16x64(__builtin_bit_cast(v4i, aring[i][mb]), b,
+                                                       (i % GS == 0) ? v4i{0, 0, 0, 0} : acc[mb][pp]);
                 }
                 // Refill the slot only now that its old contents are dead, so the load can land in the
                 // same registers (no copies at the loop back-edge, and the wait before the next use is
                 // for exactly this load).  The fences stop the scheduler from sinking the four steps'
                 // loads to the end of the chunk, which would serialise load and compute.
                 __builtin_amdgcn_sched_barrier(0);
-                issue(i, min(step + kDepth, s_last));
+                issue(i, stepof(it + i + kDepth));
                 __builtin_amdgcn_sched_barrier(0);
 
                 if (i % GS == GS - 1) {
@@ -204,22 +278,17 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
                         for (int pp = 0; pp < 4; ++pp)
 #pragma unroll
                             for (int j = 0; j < J; ++j) {
-                                // true group sum (x 4^p) = raw - zp_eff * rowsum
-                                if (SYM2) {  // zero-point 2 everywhere: 2 * 4^p = 1 << (2p + 1); field 3 needs nothing
-                                    if (pp < 3) acc[mb][pp][j] += nrs[mb][j] << (2 * pp + 1);
-                                } else {
-                                    acc[mb][pp][j] += __mul24(nrs[mb][j], zps[pp]);
-                                }
-                                t[mb][pp][j] = __builtin_fmaf((float)acc[mb][pp][j], sc[pp], t[mb][pp][j]);
+                                if (DUMP) acc[mb][pp][j] += __mul24(nrs[mb][j], zps[pp]);  // true group sum x 4^p
+                                t[mb][pp][j] = __builtin_fmaf((float)acc[mb][pp][j], (float)sc[pp], t[mb][pp][j]);
                                 if (DUMP) {
                                     const int m = mb * 16 + quad * 4 + j;
                                     const int n = strip * kStripN + pp * 16 + col;
-                                    if (g < g1 && m < p.M && n < p.N) {
+                                    if (g < g1 && m < M && n < p.N) {
                                         const int v = acc[mb][pp][j] >> (2 * pp);  // exact: a multiple of 4^p
                                         if (p.dump_mode == 1)
-                                            p.acc_dump[((size_t)m * p.N + n) * p.G + g] = v;
+                                            p.acc_dump[((size_t)(m0 + m) * p.N + n) * p.G + g] = v;
                                         else
-                                            atomicAdd(p.acc_dump + (size_t)m * p.N + n, v);
+                                            atomicAdd(p.acc_dump + (size_t)(m0 + m) * p.N + n, v);
                                     }
                                 }
                             }
@@ -228,28 +297,44 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
         }
     }
 
+    constexpr float kUnscale[4] = {1.0f, 0.25f, 0.0625f, 0.015625f};  // 4^-p, exact
+
+    if (NWK == 1) {  // the wave owns the strip's whole K range: store the D fragments directly
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp)
+#pragma unroll
+                for (int j = 0; j < J; ++j) {
+                    const int m = mb * 16 + quad * 4 + j;
+                    const int n = strip * kStripN + pp * 16 + col;
+                    if (m < M && n < p.N)
+                        out[(size_t)m * p.ldo + n] = OutT::cast((t[mb][pp][j] * kUnscale[pp]) * sa[mb * J + j]);
+                }
+        return;
+    }
+
     // ---- meet the workgroup's waves in LDS (the metadata area is dead once every wave is here)
     __syncthreads();
-
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
         for (int pp = 0; pp < 4; ++pp)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) sm.red[wave][mb * 16 + quad * 4 + j][pp * 16 + col] = t[mb][pp][j];
+            for (int j = 0; j < J; ++j)
+                if (J > 1 || quad == 0) sm.red[pwave][mb * 16 + quad * 4 + j][pp * 16 + col] = t[mb][pp][j] * kUnscale[pp];
     __syncthreads();
 
-    uint16_t* out = reinterpret_cast<uint16_t*>(p.out);
     if (p.split == 1) {
 #pragma unroll
         for (int i = 0; i < kOutPerThread; ++i) {
             const int e = tid + kThreads * i;
             const int m = e >> 6, nl = e & 63;
             const int n = strip * kStripN + nl;
-            if (e < kTile && m < p.M && n < p.N) {
+            if (e < kLive && m < M && n < p.N) {
                 float v = sm.red[0][m][nl];
 #pragma unroll
-                for (int w = 1; w < NW; ++w) v += sm.red[w][m][nl];
+                for (int w = 1; w < NWP; ++w) v += sm.red[w][m][nl];
                 out[(size_t)m * p.ldo + n] = OutT::cast(v * sa[i]);
             }
         }
@@ -261,22 +346,22 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     // cache-bypassing loads on gfx950), so no L2 write-back / invalidate fence is needed: a fence
     // here costs about a microsecond per workgroup and serialises on each XCD's L2.
     // s_waitcnt vmcnt(0) makes every lane's stores complete before the arrival counter moves.
-    float* mine = p.ws_partial + ((size_t)split * p.strips + strip) * kTile;
+    float* mine = p.ws_partial + ((size_t)split * p.strips * mblocks + tile_id) * kTile;
 #pragma unroll
     for (int i = 0; i < kOutPerThread; ++i) {
         const int e = tid + kThreads * i;
-        if (e < kTile) {
+        if (e < kLive) {
             const int m = e >> 6, nl = e & 63;
             float v = sm.red[0][m][nl];
 #pragma unroll
-            for (int w = 1; w < NW; ++w) v += sm.red[w][m][nl];
+            for (int w = 1; w < NWP; ++w) v += sm.red[w][m][nl];
             __hip_atomic_store(mine + e, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) {
-        const unsigned prev = __hip_atomic_fetch_add(p.ws_counter + strip, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned prev = __hip_atomic_fetch_add(p.ws_counter + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         sm.last = (prev == (unsigned)(p.split - 1));
     }
     __syncthreads();
@@ -284,114 +369,397 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
 #pragma unroll
     for (int i = 0; i < kOutPerThread; ++i) {
         const int e = tid + kThreads * i;
-        if (e >= kTile) break;
+        if (e >= kLive) break;
         const int m = e >> 6, nl = e & 63;
         const int n = strip * kStripN + nl;
         float v = 0.0f;
         for (int sp = 0; sp < p.split; ++sp)
-            v += __hip_atomic_load(p.ws_partial + ((size_t)sp * p.strips + strip) * kTile + e, __ATOMIC_RELAXED,
+            v += __hip_atomic_load(p.ws_partial + ((size_t)sp * p.strips * mblocks + tile_id) * kTile + e, __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
-        if (m < p.M && n < p.N) out[(size_t)m * p.ldo + n] = OutT::cast(v * sa[i]);
+        if (m < M && n < p.N) out[(size_t)m * p.ldo + n] = OutT::cast(v * sa[i]);
     }
-    if (tid == 0) __hip_atomic_store(p.ws_counter + strip, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) __hip_atomic_store(p.ws_counter + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int MB, int J, int GS, int NW, int ZM, bool DUMP, typename OutT>
+template <int J, int GS, int NW, bool ASYM, bool DUMP, typename OutT>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const GemmParams p) {
-    __shared__ __attribute__((aligned(16))) SkinnySmem<MB, NW, 4> sm;
-    skinny_body<MB, J, GS, NW, ZM, DUMP, OutT, 4>(p, blockIdx.x, blockIdx.y, sm);
+    __shared__ __attribute__((aligned(16))) SkinnySmem<NW> sm;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keeps ranges and bases in SGPRs
+    skinny_body<J, GS, NW, NW, ASYM, DUMP, OutT>(p, blockIdx.x, blockIdx.y, blockIdx.z, wave, wave, sm);
 }
 
-// Several independent skinny GEMMs in one launch: workgroup ids are cut into runs, one run per
-// problem (one workgroup per strip, no split-K: together the problems fill the chip), and each
-// workgroup runs the single-problem body on its problem.  All problems share the group size,
-// the zero-point mode and the output type; M may differ (the three row-count variants live side
-// by side in the kernel).  The problem table travels in the kernel arguments.
-#ifndef SLIMK_GROUPED_WAVES_PER_SIMD
-#define SLIMK_GROUPED_WAVES_PER_SIMD 2
+// ---------------------------------------------------------------------------------------------
+// Grouped launch: several independent skinny GEMMs in one kernel.
+//
+// What bounds a decode GEMM on this chip is the per-CU vector memory path: every wave-wide load,
+// hit or miss, takes a slot in it, and the slots not taken by weight lines coming from HBM are
+// lost bandwidth.  With one activation load per weight load (the single-launch body above) half
+// the slots carry activations.  Here the eight waves of a workgroup work on neighbouring strips
+// of one problem over the same range of K and share its activations through LDS: per chunk of four
+// steps the chunk's four 1 KiB A fragments are fetched once per sharing set, one step per wave,
+// parked in a double-buffered LDS area, and read back by every wave of the set with ds_read_b128
+// (lane l of a fragment sits at 16*l: conflict-free).  One barrier per chunk keeps the set in step.
+//
+// Workgroup = NK k-parts x NS strips (NK * NS = 8 waves).  Short reductions use NK = 1 (nothing to
+// reduce, each wave stores its own D fragments); long ones split K over 2 or 4 parts that meet in
+// LDS, so that every wave of the launch streams a run of comparable length (48..96 steps) and its
+// start-up and wind-down cost is spread over enough steps.
+constexpr int kGroupedWaves = 8;
+#ifndef SLIMK_SHARE_ROWS
+#define SLIMK_SHARE_ROWS 8
 #endif
-template <int GS, int ZM, typename OutT>
-__global__ __launch_bounds__(256, SLIMK_GROUPED_WAVES_PER_SIMD) void skinny_grouped_kernel(const GroupedParams gp) {
-    __shared__ __attribute__((aligned(16))) union {
-        SkinnySmem<1, 4, 4> one;
-        SkinnySmem<2, 4, 4> two;
-    } sm;
+constexpr int kShareRows = SLIMK_SHARE_ROWS;  // token rows from which activations are shared through LDS
+
+// Per-group metadata is handled in blocks of kBlockGroups groups: one block's scales, zero-points
+// and activation row sums are fetched with three or four wave-wide loads (instead of a few small
+// loads every chunk), parked in a wave-private LDS area, and the block's whole zero-point term goes
+// through four fp32 MFMAs per sub-block at the block's start.
+constexpr int kBlockGroups = 16;
+
+struct GroupedMeta {
+    uint16_t scale[kBlockGroups][16][4];  // [group of the block][col][sub-block]   2 KiB
+    int32_t rowsum[kBlockGroups][16];     //                                        1 KiB
+    uint8_t zp[kBlockGroups][16][4];      //                                        1 KiB
+};
+
+struct GroupedSmem {
+    union {
+        GroupedMeta meta[kGroupedWaves];
+        float red[kGroupedWaves][16][kStripN + 1];
+    };
+    v4u abuf[4][2][kDepth][64];  // [k-part][parity][step of the chunk][lane]
+};
+
+template <int J, int GS, int NK, bool SHARE, bool ASYM, typename OutT>
+__device__ __forceinline__ void shared_body(const GemmParams& p, const int unit, const int mblk, const int wave,
+                                            GroupedSmem& sm) {
+    constexpr int NS = kGroupedWaves / NK;               // waves (strips) sharing one activation stream
+    constexpr int NL = NS >= kDepth ? 1 : kDepth / NS;   // A fragments a loading wave fetches per chunk
+    constexpr int kThreads = kGroupedWaves * 64;
+    constexpr int kGroupsPerChunk = kDepth / GS;         // GS = 4 is one group per chunk
+    constexpr int kChunksPerBlock = kBlockGroups / kGroupsPerChunk;
+    constexpr int kLive = (J == 1 ? 1 : 16) * kStripN;   // elements of a strip's tile that can hold real tokens
+    constexpr int kOutPerThread = (NS * kLive + kThreads - 1) / kThreads;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int col = lane & 15, quad = lane >> 4;
+    const int kpart = wave / NS, swave = wave % NS;
+    const int strip_raw = unit * NS + swave;
+    const bool active = strip_raw < p.strips;       // a padding wave streams a valid strip but stores nothing
+    const int strip = min(strip_raw, p.strips - 1);
+    GroupedMeta& meta = sm.meta[wave];
+
+    // this row block's view of the per-token operands
+    const int m0 = mblk * 16;
+    const int M = min(16, p.M - m0);
+    const int8_t* const qp = p.q + (size_t)m0 * p.ldq;
+    const float* const sap = p.s_a + m0;
+    const int32_t* const rsp = p.rowsum + m0;
+    const int ldr = p.ldr - m0;
+    uint16_t* const out = reinterpret_cast<uint16_t*>(p.out) + (size_t)m0 * p.ldo;
+
+    // token scales for the epilogue, fetched first
+    float sa[NK == 1 ? J : kOutPerThread];
+    if (NK == 1) {
+#pragma unroll
+        for (int j = 0; j < J; ++j) sa[j] = sap[min(quad * 4 + j, M - 1)];
+    } else {
+#pragma unroll
+        for (int i = 0; i < kOutPerThread; ++i) sa[i] = sap[min(((tid + kThreads * i) % kLive) >> 6, M - 1)];
+    }
+
+    // K range of this k-part in whole chunks; every part runs the same number of chunk iterations
+    // (the barrier count must agree), a shorter last part idles through the extra ones with zero scales.
+    const int chunks = (p.steps + kDepth - 1) / kDepth;
+    const int per_part = (chunks + NK - 1) / NK;
+    const int s0 = min(kpart * per_part * kDepth, p.steps);
+    const int s1 = min(s0 + per_part * kDepth, p.steps);
+    const int g0 = s0 / GS, g1 = s1 / GS;
+    const int len = s1 - s0;
+    auto stepof = [&](int it) { return s0 + max(min(it, len - 1), 0); };
+
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(p.w_r), 0, (int)((size_t)p.strips * p.steps * (kUnitDwords * 4)), 0x00020000);
+    const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int8_t*>(qp), 0, (int)((size_t)(M - 1) * p.ldq + p.K), 0x00020000);
+    const uint32_t wstride = (uint32_t)p.strips * (kUnitDwords * 4);
+    const uint32_t wbase = (uint32_t)strip * (kUnitDwords * 4);
+    const uint32_t wlane = lane * 16;
+    const uint32_t aoff = (uint32_t)min(col, M - 1) * (uint32_t)p.ldq + quad * 16;
+
+    // ---- metadata of one block of groups: global -> registers (a block ahead) -> LDS.
+    // Groups past the part's end are clamped onto its last group for the loads and get zero scales
+    // when parked, so they add nothing.
+    v4i m_scale[2], m_zp, m_rs;
+    auto fetch_meta = [&](int gfirst) {
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {  // scales: 16 groups x 128 B: lane -> group 8n + lane/8
+            const size_t sgi = (size_t)max(min(gfirst + n * 8 + (lane >> 3), g1 - 1), 0) * p.strips + strip;
+            m_scale[n] = *reinterpret_cast<const v4i*>(reinterpret_cast<const char*>(p.s_r) + sgi * 128 + (lane & 7) * 16);
+        }
+        const int gq = max(min(gfirst + (lane >> 2), g1 - 1), 0);  // row sums / zero-points: lane -> group lane/4
+        if (ASYM)
+            m_zp = *reinterpret_cast<const v4i*>(reinterpret_cast<const char*>(p.zp_r) +
+                                                 ((size_t)gq * p.strips + strip) * 64 + (lane & 3) * 16);
+        m_rs = *reinterpret_cast<const v4i*>(rsp + (size_t)gq * p.ldr + min((lane & 3) * 4, ldr - 4));
+    };
+    auto park_meta = [&](int gfirst) {
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            if (gfirst + n * 8 + (lane >> 3) >= g1) m_scale[n] = v4i{0, 0, 0, 0};
+            *reinterpret_cast<v4i*>(reinterpret_cast<char*>(&meta.scale[0][0][0]) + n * 1024 + lane * 16) = m_scale[n];
+        }
+        if (ASYM) *reinterpret_cast<v4i*>(reinterpret_cast<char*>(&meta.zp[0][0][0]) + lane * 16) = m_zp;
+        *reinterpret_cast<v4i*>(&meta.rowsum[lane >> 2][(lane & 3) * 4]) = m_rs;
+    };
+
+    // ---- weights: register ring.  Activations: with few token rows a fragment is only a line or two
+    // and each wave keeps its own register ring of them (SHARE = false: no LDS hand-over, no
+    // barrier); otherwise they are fetched once per sharing set and handed round through LDS.
+    v4u wring[kDepth];
+    auto issue_w = [&](int slot, int step) {
+        wring[slot] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane, step * wstride + wbase, 0);
+    };
+    v4u aring[kDepth];
+    auto issue_a = [&](int slot, int step) {
+        if (!SHARE) aring[slot] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, aoff, step * kStepK, 0);
+    };
+    const bool loader = SHARE && swave < kDepth;  // wave-uniform
+    v4u areg[NL];
+    auto fetch_a = [&](int it) {  // this wave's share of the chunk that starts at iteration `it`
+        if (loader) {
+#pragma unroll
+            for (int n = 0; n < NL; ++n) areg[n] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, aoff, stepof(it + swave + n * NS) * kStepK, 0);
+        }
+    };
+    auto park_a = [&](int parity) {
+        if (loader) {
+#pragma unroll
+            for (int n = 0; n < NL; ++n) sm.abuf[kpart][parity][swave + n * NS][lane] = areg[n];
+        }
+    };
+
+    // running sums, in units of 4^p (sub-block p < 3) resp. 64 (p = 3) times the result
+    v4f t[4];
+#pragma unroll
+    for (int pp = 0; pp < 4; ++pp) t[pp] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    const float czu[4] = {-(float)p.zp_const, -(float)(p.zp_const * 4), -(float)(p.zp_const * 16),
+                          -(float)((p.zp_const - 2) * 64)};
+
+    fetch_meta(g0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < kDepth; ++i) {
+        issue_w(i, stepof(i));
+        issue_a(i, stepof(i));
+    }
+    if (SHARE) {
+        fetch_a(0);
+        __builtin_amdgcn_sched_barrier(0);
+        park_a(0);
+        fetch_a(kDepth);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    v4i acc[4];
+    v4h sc;
+    const int blocks = (per_part + kChunksPerBlock - 1) / kChunksPerBlock;
+    for (int blk = 0; blk < blocks; ++blk) {
+        const int gblock = g0 + blk * kBlockGroups;
+        park_meta(gblock);                       // this block's metadata: registers -> LDS
+        fetch_meta(gblock + kBlockGroups);       // next block's: global -> registers
+        __builtin_amdgcn_sched_barrier(0);
+
+        // zero-point term of the whole block: lane (col, quad) supplies token col / channel col of
+        // group 4b + quad; -zpe * scale * rowsum summed over four groups per fp32 MFMA
+#pragma unroll
+        for (int b = 0; b < kBlockGroups / 4; ++b) {
+            const int gi = 4 * b + quad;
+            const v4h zs = *reinterpret_cast<const v4h*>(&meta.scale[gi][col][0]);
+            float zb[4];
+            if (ASYM) {
+                const uint32_t zraw = *reinterpret_cast<const uint32_t*>(&meta.zp[gi][col][0]);
+                zb[0] = -(float)(zraw & 0xffu) * (float)zs[0];
+                zb[1] = -4.0f * (float)((zraw >> 8) & 0xffu) * (float)zs[1];
+                zb[2] = -16.0f * (float)((zraw >> 16) & 0xffu) * (float)zs[2];
+                zb[3] = (128.0f - 64.0f * (float)(zraw >> 24)) * (float)zs[3];
+            } else {
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) zb[pp] = czu[pp] * (float)zs[pp];
+            }
+            const float rsf = (float)meta.rowsum[gi][col];
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp)
+                if (ASYM || pp < 3 || p.zp_const != 2)  // uniform zero-point 2: field 3 is already centred
+                    t[pp] = __builtin_amdgcn_mfma_f32_16x16x4f32(rsf, zb[pp], t[pp], 0, 0, 0);
+        }
+
+        const int c_end = min(per_part - blk * kChunksPerBlock, kChunksPerBlock);
+        for (int cc = 0; cc < c_end; ++cc) {
+            const int c = blk * kChunksPerBlock + cc;
+            const int it = c * kDepth;
+            if (SHARE) {
+                __syncthreads();             // chunk c's fragments are in place; chunk c-1's are no longer read
+                park_a((c + 1) & 1);         // chunk c+1's fragments: registers -> LDS
+                fetch_a(it + 2 * kDepth);    // chunk c+2's: global -> registers
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < kDepth; ++i) aring[i] = sm.abuf[kpart][c & 1][i][lane];
+            }
+            const uint16_t* const scp = &meta.scale[cc * kGroupsPerChunk][col][0];  // this chunk's groups
+#pragma unroll
+            for (int i = 0; i < kDepth; ++i) {
+                if (i % GS == 0) sc = *reinterpret_cast<const v4h*>(scp + (i / GS) * 64);
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) {
+                    const v4i b = __builtin_bit_cast(v4i, wring[i] & (0x03030303u << (2 * pp)));
+                    acc[pp] = mfma_i8_16x16x64(__builtin_bit_cast(v4i, aring[i]), b, (i % GS == 0) ? v4i{0, 0, 0, 0} : acc[pp]);
+                }
+                // refill the slot only now that its old contents are dead (see skinny_body)
+                __builtin_amdgcn_sched_barrier(0);
+                issue_w(i, stepof(it + i + kDepth));
+                issue_a(i, stepof(it + i + kDepth));
+                __builtin_amdgcn_sched_barrier(0);
+                if (i % GS == GS - 1) {
+#pragma unroll
+                    for (int pp = 0; pp < 4; ++pp)
+#pragma unroll
+                        for (int j = 0; j < J; ++j) t[pp][j] = __builtin_fmaf((float)acc[pp][j], (float)sc[pp], t[pp][j]);
+                }
+            }
+        }
+    }
+
+    constexpr float kUnscale[4] = {1.0f, 0.25f, 0.0625f, 0.015625f};  // 4^-p, exact
+    if (NK == 1) {
+        if (active) {
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp)
+#pragma unroll
+                for (int j = 0; j < J; ++j) {
+                    const int m = quad * 4 + j;
+                    const int n = strip * kStripN + pp * 16 + col;
+                    if (m < M && n < p.N) out[(size_t)m * p.ldo + n] = OutT::cast((t[pp][j] * kUnscale[pp]) * sa[j]);
+                }
+        }
+        return;
+    }
+
+    // ---- the k-parts of each strip meet in LDS (the metadata area is dead once every wave is here)
+    __syncthreads();
+#pragma unroll
+    for (int pp = 0; pp < 4; ++pp)
+#pragma unroll
+        for (int j = 0; j < J; ++j)
+            if (J > 1 || quad == 0) sm.red[wave][quad * 4 + j][pp * 16 + col] = t[pp][j] * kUnscale[pp];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kOutPerThread; ++i) {
+        const int e = tid + kThreads * i;
+        const int sidx = e / kLive, w = e % kLive;
+        const int m = w >> 6, nl = w & 63;
+        const int so = unit * NS + sidx;
+        const int n = so * kStripN + nl;
+        if (sidx < NS && so < p.strips && m < M && n < p.N) {
+            float v = sm.red[sidx][m][nl];
+#pragma unroll
+            for (int kp = 1; kp < NK; ++kp) v += sm.red[kp * NS + sidx][m][nl];
+            out[(size_t)m * p.ldo + n] = OutT::cast(v * sa[i]);
+        }
+    }
+}
+
+// Workgroup ids are cut into runs, one run per problem.  Within a problem, workgroups come in sets
+// of eight per row block: consecutive workgroup ids go to different XCDs, so the two row blocks of
+// a set of strips, eight ids apart, share an XCD and its L2.  All problems share the group size,
+// the zero-point mode and the output type.  The problem table travels in the kernel arguments.
+template <int GS, bool ASYM, typename OutT>
+__global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_grouped_kernel(const GroupedParams gp) {
+    __shared__ __attribute__((aligned(16))) GroupedSmem sm;
     const int wg = blockIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int i = 0;
     while (i + 1 < gp.count && wg >= gp.wg_begin[i + 1]) ++i;
     const GemmParams& p = gp.prob[i];
-    const int strip = wg - gp.wg_begin[i];
-    if (p.M == 1) skinny_body<1, 1, GS, 4, ZM, false, OutT, 4>(p, strip, 0, sm.one);
-    else if (p.M <= 16) skinny_body<1, 4, GS, 4, ZM, false, OutT, 4>(p, strip, 0, sm.one);
-    else skinny_body<2, 4, GS, 4, ZM, false, OutT, 4>(p, strip, 0, sm.two);
-}
-
-template <int MB, int J, int GS, int NW, int ZM, bool DUMP>
-static void launch_out(const GemmParams& p, bool out_bf16, hipStream_t stream) {
-    const dim3 grid(p.strips, p.split), block(NW * 64);
-    if (out_bf16)
-        skinny_kernel<MB, J, GS, NW, ZM, DUMP, OutBF16><<<grid, block, 0, stream>>>(p);
-    else
-        skinny_kernel<MB, J, GS, NW, ZM, DUMP, OutF16><<<grid, block, 0, stream>>>(p);
-}
-
-template <int MB, int J, int GS, int NW, bool DUMP>
-static void launch_zm(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
-    if (asym) launch_out<MB, J, GS, NW, 2, DUMP>(p, out_bf16, stream);
-    else if (p.zp_const == 2) launch_out<MB, J, GS, NW, 0, DUMP>(p, out_bf16, stream);
-    else launch_out<MB, J, GS, NW, 1, DUMP>(p, out_bf16, stream);
-}
-
-template <int MB, int GS, int NW>
-static void launch_flags(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
-    const bool dump = p.acc_dump != nullptr && p.dump_mode != 0;
-    if (dump) launch_zm<MB, 4, GS, 4, true>(p, asym, out_bf16, stream);  // verification: 4 waves, all rows
-    else if (MB == 1 && p.M == 1) launch_zm<MB, (MB == 1 ? 1 : 4), GS, NW, false>(p, asym, out_bf16, stream);
-    else launch_zm<MB, 4, GS, NW, false>(p, asym, out_bf16, stream);
-}
-
-template <int MB, int GS>
-static void launch_nw(const GemmParams& p, int waves, bool asym, bool out_bf16, hipStream_t stream) {
-    if (MB == 1) {
-        if (waves >= 16) launch_flags<MB, GS, (MB == 1 ? 16 : 8)>(p, asym, out_bf16, stream);
-        else launch_flags<MB, GS, 4>(p, asym, out_bf16, stream);
+    const int local = wg - gp.wg_begin[i];
+    const int mblocks = (p.M + 15) >> 4;
+    const int mblk = (local >> 3) % mblocks;
+    const int unit = (local / (8 * mblocks)) * 8 + (local & 7);  // set of strips
+    const int nk = gp.kparts[i];
+    if (unit * (kGroupedWaves / nk) >= p.strips) return;  // padding workgroup (uniform)
+    // activations go through LDS once a fragment spans enough cache lines to be worth a barrier
+    const int mrows = min(16, p.M - mblk * 16);
+    if (nk == 1) {
+        if (p.M == 1) shared_body<1, GS, 1, false, ASYM, OutT>(p, unit, mblk, wave, sm);
+        else if (mrows < kShareRows) shared_body<4, GS, 1, false, ASYM, OutT>(p, unit, mblk, wave, sm);
+        else shared_body<4, GS, 1, true, ASYM, OutT>(p, unit, mblk, wave, sm);
+    } else if (nk == 2) {
+        if (p.M == 1) shared_body<1, GS, 2, false, ASYM, OutT>(p, unit, mblk, wave, sm);
+        else if (mrows < kShareRows) shared_body<4, GS, 2, false, ASYM, OutT>(p, unit, mblk, wave, sm);
+        else shared_body<4, GS, 2, true, ASYM, OutT>(p, unit, mblk, wave, sm);
     } else {
-        if (waves >= 8) launch_flags<MB, GS, 8>(p, asym, out_bf16, stream);
-        else launch_flags<MB, GS, 4>(p, asym, out_bf16, stream);
+        if (p.M == 1) shared_body<1, GS, 4, false, ASYM, OutT>(p, unit, mblk, wave, sm);
+        else if (mrows < kShareRows) shared_body<4, GS, 4, false, ASYM, OutT>(p, unit, mblk, wave, sm);
+        else shared_body<4, GS, 4, true, ASYM, OutT>(p, unit, mblk, wave, sm);
     }
 }
 
-template <int MB>
-static void launch_gs(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, hipStream_t stream) {
-    if (gs == 1) launch_nw<MB, 1>(p, waves, asym, out_bf16, stream);
-    else if (gs == 2) launch_nw<MB, 2>(p, waves, asym, out_bf16, stream);
-    else launch_nw<MB, 4>(p, waves, asym, out_bf16, stream);
+template <int J, int GS, int NW, bool ASYM, bool DUMP>
+static void launch_out(const GemmParams& p, bool out_bf16, hipStream_t stream) {
+    const dim3 grid(p.strips, p.split, (p.M + 15) / 16), block(NW * 64);
+    if (out_bf16)
+        skinny_kernel<J, GS, NW, ASYM, DUMP, OutBF16><<<grid, block, 0, stream>>>(p);
+    else
+        skinny_kernel<J, GS, NW, ASYM, DUMP, OutF16><<<grid, block, 0, stream>>>(p);
 }
 
-template <int GS, int ZM>
-static void launch_grouped_out(const GroupedParams& gp, int total_wgs, bool out_bf16, hipStream_t stream) {
-    if (out_bf16) skinny_grouped_kernel<GS, ZM, OutBF16><<<dim3(total_wgs), dim3(256), 0, stream>>>(gp);
-    else skinny_grouped_kernel<GS, ZM, OutF16><<<dim3(total_wgs), dim3(256), 0, stream>>>(gp);
+template <int J, int GS, int NW, bool DUMP>
+static void launch_zm(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
+    if (asym) launch_out<J, GS, NW, true, DUMP>(p, out_bf16, stream);
+    else launch_out<J, GS, NW, false, DUMP>(p, out_bf16, stream);
 }
 
 template <int GS>
-static void launch_grouped_zm(const GroupedParams& gp, int total_wgs, int zm, bool out_bf16, hipStream_t stream) {
-    if (zm == 0) launch_grouped_out<GS, 0>(gp, total_wgs, out_bf16, stream);
-    else if (zm == 1) launch_grouped_out<GS, 1>(gp, total_wgs, out_bf16, stream);
-    else launch_grouped_out<GS, 2>(gp, total_wgs, out_bf16, stream);
+static void launch_nw(const GemmParams& p, int waves, bool asym, bool out_bf16, hipStream_t stream) {
+    const bool dump = p.acc_dump != nullptr && p.dump_mode != 0;
+    if (dump) launch_zm<4, GS, 4, true>(p, asym, out_bf16, stream);  // verification: 4 waves, all rows
+    else if (waves >= 16) {
+        if (p.M == 1) launch_zm<1, GS, 16, false>(p, asym, out_bf16, stream);
+        else launch_zm<4, GS, 16, false>(p, asym, out_bf16, stream);
+    } else if (waves >= 8) {
+        if (p.M == 1) launch_zm<1, GS, 8, false>(p, asym, out_bf16, stream);
+        else launch_zm<4, GS, 8, false>(p, asym, out_bf16, stream);
+    } else {
+        if (p.M == 1) launch_zm<1, GS, 4, false>(p, asym, out_bf16, stream);
+        else launch_zm<4, GS, 4, false>(p, asym, out_bf16, stream);
+    }
 }
 
-hipError_t launch_skinny_grouped(const GroupedParams& gp, int gs, int zm, bool out_bf16, hipStream_t stream) {
+template <int GS, bool ASYM>
+static void launch_grouped_out(const GroupedParams& gp, int total_wgs, bool out_bf16, hipStream_t stream) {
+    if (out_bf16) skinny_grouped_kernel<GS, ASYM, OutBF16><<<dim3(total_wgs), dim3(kGroupedWaves * 64), 0, stream>>>(gp);
+    else skinny_grouped_kernel<GS, ASYM, OutF16><<<dim3(total_wgs), dim3(kGroupedWaves * 64), 0, stream>>>(gp);
+}
+
+template <int GS>
+static void launch_grouped_zm(const GroupedParams& gp, int total_wgs, bool asym, bool out_bf16, hipStream_t stream) {
+    if (asym) launch_grouped_out<GS, true>(gp, total_wgs, out_bf16, stream);
+    else launch_grouped_out<GS, false>(gp, total_wgs, out_bf16, stream);
+}
+
+hipError_t launch_skinny_grouped(const GroupedParams& gp, int gs, bool asym, bool out_bf16, hipStream_t stream) {
     const int total_wgs = gp.wg_begin[gp.count];
-    if (gs == 1) launch_grouped_zm<1>(gp, total_wgs, zm, out_bf16, stream);
-    else if (gs == 2) launch_grouped_zm<2>(gp, total_wgs, zm, out_bf16, stream);
-    else launch_grouped_zm<4>(gp, total_wgs, zm, out_bf16, stream);
+    if (gs == 1) launch_grouped_zm<1>(gp, total_wgs, asym, out_bf16, stream);
+    else if (gs == 2) launch_grouped_zm<2>(gp, total_wgs, asym, out_bf16, stream);
+    else launch_grouped_zm<4>(gp, total_wgs, asym, out_bf16, stream);
     return hipGetLastError();
 }
 
 hipError_t launch_skinny(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, hipStream_t stream) {
-    if (p.M <= 16) launch_gs<1>(p, gs, waves, asym, out_bf16, stream);
-    else launch_gs<2>(p, gs, waves, asym, out_bf16, stream);
+    if (gs == 1) launch_nw<1>(p, waves, asym, out_bf16, stream);
+    else if (gs == 2) launch_nw<2>(p, waves, asym, out_bf16, stream);
+    else launch_nw<4>(p, waves, asym, out_bf16, stream);
     return hipGetLastError();
 }
 

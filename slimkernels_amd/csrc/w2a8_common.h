@@ -64,7 +64,8 @@ struct GemmParams {
 constexpr int kMaxGroup = 24;
 struct GroupedParams {
     GemmParams prob[kMaxGroup];
-    int wg_begin[kMaxGroup + 1];  // problem i owns workgroups wg_begin[i] .. wg_begin[i+1]-1 (one per strip)
+    int wg_begin[kMaxGroup + 1];  // problem i owns workgroups wg_begin[i] .. wg_begin[i+1]-1
+    int kparts[kMaxGroup];  // 1, 2 or 4: parts K is split into inside a workgroup of eight waves (8, 4 or 2 strips)
     int count;
 };
 

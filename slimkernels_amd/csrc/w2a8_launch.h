@@ -23,8 +23,8 @@ hipError_t launch_read_probe(const void* src, size_t bytes, uint32_t* sink, hipS
 // gs = 64-element steps per scale group (1, 2 or 4); waves = wavefronts per workgroup (4, 8, 16)
 hipError_t launch_skinny(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, hipStream_t stream);
 
-// zm: 0 uniform zero-point 2, 1 other uniform zero-point, 2 per-group zero-points
-hipError_t launch_skinny_grouped(const GroupedParams& gp, int gs, int zm, bool out_bf16, hipStream_t stream);
+// asym: every problem carries per-group zero-points (zp_r); otherwise each uses its uniform zp_const
+hipError_t launch_skinny_grouped(const GroupedParams& gp, int gs, bool asym, bool out_bf16, hipStream_t stream);
 
 // launch_tiled picks the fast kernel when it applies (uniform zero-point 2, group 64/128, K % 128 == 0,
 // no verification dump) and the generic one otherwise.

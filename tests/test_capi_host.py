@@ -57,7 +57,8 @@ def test_split_heuristic_and_workspace(L):
     assert s == 4
     ws = L.slimk_w2a8_gemm_workspace_bytes(16, 4096, 14336, 128, _lib.KERNEL_AUTO, 0)
     assert ws == 256 + s * 64 * (16 * 64) * 4     # counters + split x strips x (16 x 64 fp32 tile)
-    assert L.slimk_w2a8_gemm_workspace_bytes(32, 4096, 14336, 128, _lib.KERNEL_AUTO, 4) == 256 + 4 * 64 * (32 * 64) * 4
+    # 17..32 tokens run as two blocks of 16 rows: one counter and one tile per (strip, block)
+    assert L.slimk_w2a8_gemm_workspace_bytes(32, 4096, 14336, 128, _lib.KERNEL_AUTO, 4) == 512 + 4 * 64 * 2 * (16 * 64) * 4
     # the tiled kernel never splits
     assert L.slimk_w2a8_gemm_auto_split_k(512, 4096, 14336, 128, _lib.KERNEL_AUTO) == 1
     assert L.slimk_w2a8_gemm_auto_split_k(0, 4096, 4096, 128, 0) == 0
