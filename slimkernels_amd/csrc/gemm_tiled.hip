@@ -1,7 +1,7 @@
 // Fast tiled W2A8 GEMM for gfx950: the int8-MFMA-bound prefill regime, uniform zero-point 2
 // (the symmetric levels {-2..1}), group size 64 or 128, K a multiple of 128.
 //
-// Workgroup = 4 wavefronts side by side along the channels; workgroup tile 128 tokens x 256
+// Workgroup = 4 wavefronts side by side along the channels; workgroup tile 128 (or 64) tokens x 256
 // channels (four weight strips); wave tile 128 x 64 = 8 x 4 blocks of v_mfma_i32_16x16x64_i8.
 // A wide-in-N tile is the cheap one here: per reduction element a tile fetches BM bytes of
 // activations but only BN/4 bytes of 2-bit weights.
@@ -17,9 +17,12 @@
 //  * the unpacked weight operand of a wave (one strip) is reused by its eight token blocks;
 //  * activations sit in LDS in MFMA-operand order (1 KiB per 16-row x 64-k block, lane-major),
 //    so every fragment read is one conflict-free ds_read_b128 and the global->LDS transfer is a
-//    16-byte-per-lane copy; two LDS buffers, one barrier per 128-element stage;
-//  * a wave's weights are its own strip and nobody else's, so they never touch LDS: each wave
-//    loads its 2 KiB of packed codes per stage straight into registers one stage ahead.
+//    16-byte-per-lane LDS-direct copy that holds no registers while in flight;
+//  * a wave's weights are its own strip and nobody else's; they take the same LDS-direct road into a
+//    wave-private corner of the stage buffer;
+//  * three stage buffers: the loads of stage s+2 are in flight while stage s is consumed, one
+//    barrier per 128-element stage (with one workgroup on a CU there is no other wave to hide a
+//    stage's load latency behind).
 #include <stdlib.h>
 
 #include "w2a8_launch.h"
@@ -27,19 +30,26 @@
 namespace w2a8 {
 
 namespace fast {
-constexpr int kBM = 128, kBN = 256;
+constexpr int kBN = 256;
 constexpr int kStageSteps = 2;
-constexpr int kMB = kBM / 16;                              // 8 token blocks per wave
 constexpr int kStrips = kBN / kStripN;                     // 4 strips per workgroup, one per wave
-constexpr int kABlocks = kMB * kStageSteps;                // 16 activation blocks per stage
-constexpr int kStageDwords = kABlocks * 256;               // 16 KiB of activations per stage
 constexpr int kAQueue = 4;                                 // activation fragments kept in flight from LDS
 }  // namespace fast
 
-template <int GS, typename OutT>
-__global__ __launch_bounds__(256, 2) void tiled_kernel(const GemmParams p) {
+// BM = token rows of the workgroup tile: 128, or 64 when 128-row tiles would leave CUs idle
+// (fewer tiles than CUs, or a single workgroup per CU with nothing to hide its latencies behind).
+template <int BM, int GS, typename OutT>
+__device__ __forceinline__ void tiled_body(const GemmParams& p) {
     using namespace fast;
-    __shared__ __attribute__((aligned(16))) uint32_t lds[2][kStageDwords];
+    constexpr int kBM = BM;
+    constexpr int kMB = kBM / 16;                  // token blocks per wave (8 or 4)
+    constexpr int kABlocks = kMB * kStageSteps;    // activation blocks per stage (16 or 8)
+    constexpr int kStageDwords = kABlocks * 256;   // 16 or 8 KiB of activations per stage
+    constexpr int kALoads = kABlocks / 4;          // LDS-direct activation block loads per wave and stage
+    constexpr int kWDwords = kStrips * kStageSteps * 256;  // the four waves' weight units of a stage: 8 KiB
+    constexpr int kBufDwords = kStageDwords + kWDwords;
+    constexpr int kBufs = 3;                       // stage s+2 is in flight while stage s is consumed
+    __shared__ __attribute__((aligned(16))) uint32_t lds[kBufs][kBufDwords];
     constexpr int kGroupsPerStage = kStageSteps / GS;  // 2 (group 64) or 1 (group 128)
 
     const int tid = threadIdx.x;
@@ -75,38 +85,46 @@ __global__ __launch_bounds__(256, 2) void tiled_kernel(const GemmParams p) {
         const_cast<uint32_t*>(p.w_r), 0, (int)min((size_t)p.strips * p.steps * (kUnitDwords * 4), (size_t)0x7fffffff), 0x00020000);
     const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(p.s_r), 0, (int)min((size_t)p.strips * p.G * 128, (size_t)0x7fffffff), 0x00020000);
-    uint32_t a_off[4];
+    uint32_t a_off[kALoads];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int blk = wave + 4 * i;
-        a_off[i] = (uint32_t)(m_tile + (blk & 7) * 16 + col) * (uint32_t)p.ldq + (blk >> 3) * kStepK + quad * 16;
+    for (int i = 0; i < kALoads; ++i) {
+        const int blk = wave + 4 * i;  // block = step_in_stage * kMB + token block
+        a_off[i] = (uint32_t)(m_tile + (blk % kMB) * 16 + col) * (uint32_t)p.ldq + (blk / kMB) * kStepK + quad * 16;
     }
     const uint32_t b_step_stride = (uint32_t)p.strips * (kUnitDwords * 4);  // bytes between steps of a strip
     const uint32_t b_strip_off = (uint32_t)strip * (kUnitDwords * 4);
     const uint32_t s_lane_off = (uint32_t)(strip * 16 + col) * 8;
     const uint32_t s_group_stride = (uint32_t)p.strips * 128;               // bytes between groups of a strip
-    typedef unsigned v4u __attribute__((ext_vector_type(4)));
     typedef unsigned v2u __attribute__((ext_vector_type(2)));
-    v4u gb[kStageSteps];
     v2u sraw[kGroupsPerStage];
+    // Activations and this wave's weight units go straight from global memory into LDS (no registers
+    // held while in flight), two stages ahead; the scales, a few bytes, go to registers one stage ahead.
+    constexpr int kLdsLoads = kALoads + kStageSteps;  // LDS-direct loads a wave issues per stage
     auto fetch = [&](int stage, int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < kALoads; ++i)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
                 q_rsrc, (__attribute__((address_space(3))) void*)&lds[buf][(wave + 4 * i) * 256], 16, a_off[i],
                 stage * (kStageSteps * kStepK), 0, 0);
 #pragma unroll
         for (int s = 0; s < kStageSteps; ++s)
-            gb[s] = __builtin_amdgcn_raw_buffer_load_b128(
-                w_rsrc, lane * 16, (stage * kStageSteps + s) * b_step_stride + b_strip_off, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                w_rsrc, (__attribute__((address_space(3))) void*)&lds[buf][kStageDwords + (wave * kStageSteps + s) * 256], 16,
+                lane * 16, (stage * kStageSteps + s) * b_step_stride + b_strip_off, 0, 0);
+    };
+    auto fetch_scales = [&](int stage) {
 #pragma unroll
         for (int gi = 0; gi < kGroupsPerStage; ++gi)
             sraw[gi] = __builtin_amdgcn_raw_buffer_load_b64(
                 s_rsrc, s_lane_off, (stage * kGroupsPerStage + gi) * s_group_stride, 0);
     };
-    auto land = [&]() {  // every load of this wave has arrived (LDS-direct ones included), then meet the others
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+    // All but the newest stage's LDS-direct loads of this wave have arrived (loads complete in issue
+    // order; the newest kLdsLoads may still be in flight), then meet the other waves.
+    // (A bare s_barrier: __syncthreads() would add a fence that waits for every outstanding LDS-direct
+    // load.  LDS is only written by those loads and only read with ds_read here, and a wave's reads of
+    // a stage have all returned before it gets here, so nothing else needs ordering.)
+    auto land = [&]() {
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kLdsLoads) : "memory");
     };
 
     float t[kMB][4][4];
@@ -117,7 +135,9 @@ __global__ __launch_bounds__(256, 2) void tiled_kernel(const GemmParams p) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) t[mb][pp][j] = 0.0f;
 
+    fetch_scales(0);
     fetch(0, 0);
+    fetch(min(1, n_stages - 1), 1);
     land();
 
     // accumulator sets (two, alternating) and the scale of the unit carried over a stage boundary;
@@ -131,8 +151,8 @@ __global__ __launch_bounds__(256, 2) void tiled_kernel(const GemmParams p) {
         sc_prev[pp] = 0.0f;
     }
 
+    int buf = 0;
     for (int stage = 0; stage < n_stages; ++stage) {
-        const int buf = stage & 1;
         const uint32_t* la = &lds[buf][lane * 4];
         auto lds_a = [&](int r) {  // r-th fragment in consumption order: token block r / 2, step r % 2
             return *reinterpret_cast<const v4i*>(la + ((r % kStageSteps) * kMB + r / kStageSteps) * 256);
@@ -155,15 +175,18 @@ __global__ __launch_bounds__(256, 2) void tiled_kernel(const GemmParams p) {
         v4i b[kStageSteps][4];
 #pragma unroll
         for (int s = 0; s < kStageSteps; ++s) {
-            const v4i w = __builtin_bit_cast(v4i, gb[s]);
+            const v4i w = *reinterpret_cast<const v4i*>(la + kStageDwords + (wave * kStageSteps + s) * 256);
             const v4i wf = w ^ (int)0x2a2a2a2au;  // flip the high bit of fields 0..2: code -> two's complement of code - 2
 #pragma unroll
             for (int pp = 0; pp < 3; ++pp) b[s][pp] = (wf << (6 - 2 * pp)) & (int)0xc0c0c0c0u;
             b[s][3] = w & (int)0xc0c0c0c0u;  // field 3 is stored already flipped
         }
 
-        // next stage (the last iteration re-reads its own stage into the idle buffer: harmless)
-        fetch(min(stage + 1, n_stages - 1), buf ^ 1);
+        // the scales of the next stage first, then the stage after next into the buffer that stage - 1 used
+        // (every wave is past the barrier that ended stage - 1); the last iterations re-read the last
+        // stage into an idle buffer: harmless, and the number of loads in flight stays the same
+        fetch_scales(min(stage + 1, n_stages - 1));
+        fetch(min(stage + 2, n_stages - 1), buf == 0 ? 2 : buf - 1);
 
         // Work units in order: (token block, group of the stage).  The MFMAs of unit u go into
         // accumulator set u & 1 and are written before the drain of unit u - 1, so the matrix core
@@ -196,6 +219,7 @@ __global__ __launch_bounds__(256, 2) void tiled_kernel(const GemmParams p) {
         for (int pp = 0; pp < 4; ++pp) sc_prev[pp] = sc[kGroupsPerStage - 1][pp];
 
         land();
+        buf = buf == kBufs - 1 ? 0 : buf + 1;
     }
     // the last unit of the last stage
 #pragma unroll
@@ -222,6 +246,16 @@ __global__ __launch_bounds__(256, 2) void tiled_kernel(const GemmParams p) {
         }
 }
 
+// 128-row tiles: two workgroups (eight waves) per CU; 64-row tiles need fewer registers: three.
+template <int GS, typename OutT>
+__global__ __launch_bounds__(256, 2) void tiled_kernel(const GemmParams p) {
+    tiled_body<128, GS, OutT>(p);
+}
+template <int GS, typename OutT>
+__global__ __launch_bounds__(256, 3) void tiled_kernel_bm64(const GemmParams p) {
+    tiled_body<64, GS, OutT>(p);
+}
+
 bool tiled_fast_supported(const GemmParams& p, int gs, bool asym) {
     const bool dump = p.acc_dump != nullptr && p.dump_mode != 0;
     return !asym && !dump && p.zp_const == 2 && (gs == 1 || gs == 2) && p.steps % fast::kStageSteps == 0;
@@ -229,15 +263,29 @@ bool tiled_fast_supported(const GemmParams& p, int gs, bool asym) {
 
 hipError_t launch_tiled(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream) {
     if (!tiled_fast_supported(p, gs, asym)) return launch_tiled_generic(p, gs, asym, out_bf16, stream);
-    const int tiles = ((p.strips + fast::kStrips - 1) / fast::kStrips) * ((p.M + fast::kBM - 1) / fast::kBM);
+    const int tiles_n = (p.strips + fast::kStrips - 1) / fast::kStrips;
+    const int tiles128 = tiles_n * ((p.M + 127) / 128);
+    // two workgroups fit a CU: below about two 128-row tiles per CU, 64-row tiles fill the chip better
+    static const int forced_bm = [] { const char* e = getenv("SLIMK_W2A8_TILED_BM"); return e ? atoi(e) : 0; }();
+    const bool small = forced_bm ? forced_bm == 64 : tiles128 < 2 * 256;
+    const int tiles = small ? tiles_n * ((p.M + 63) / 64) : tiles128;
     const dim3 grid((tiles + 7) / 8 * 8), block(256);
-    static const int pad = [] { const char* e = getenv("SLIMK_W2A8_TILED_LDS_PAD"); return e ? atoi(e) : 0; }();
-    if (gs == 1) {
-        if (out_bf16) tiled_kernel<1, OutBF16><<<grid, block, pad, stream>>>(p);
-        else tiled_kernel<1, OutF16><<<grid, block, pad, stream>>>(p);
+    if (small) {
+        if (gs == 1) {
+            if (out_bf16) tiled_kernel_bm64<1, OutBF16><<<grid, block, 0, stream>>>(p);
+            else tiled_kernel_bm64<1, OutF16><<<grid, block, 0, stream>>>(p);
+        } else {
+            if (out_bf16) tiled_kernel_bm64<2, OutBF16><<<grid, block, 0, stream>>>(p);
+            else tiled_kernel_bm64<2, OutF16><<<grid, block, 0, stream>>>(p);
+        }
     } else {
-        if (out_bf16) tiled_kernel<2, OutBF16><<<grid, block, pad, stream>>>(p);
-        else tiled_kernel<2, OutF16><<<grid, block, pad, stream>>>(p);
+        if (gs == 1) {
+            if (out_bf16) tiled_kernel<1, OutBF16><<<grid, block, 0, stream>>>(p);
+            else tiled_kernel<1, OutF16><<<grid, block, 0, stream>>>(p);
+        } else {
+            if (out_bf16) tiled_kernel<2, OutBF16><<<grid, block, 0, stream>>>(p);
+            else tiled_kernel<2, OutF16><<<grid, block, 0, stream>>>(p);
+        }
     }
     return hipGetLastError();
 }
