@@ -276,9 +276,9 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
     w2a8::GroupedParams gp{};
     gp.count = count;
     int zm = -1, wgs = 0;
-    // A workgroup of eight waves covers 8 strips x all of K, 4 strips x 2 halves or 2 strips x 4 quarters:
-    // whichever keeps a wave's run at roughly 48..96 steps.
-    const auto kparts_of = [](int steps) { return steps > 192 ? 4 : (steps > 96 ? 2 : 1); };
+    // A workgroup of eight waves covers 8 strips x all of K, 4 strips x 2 halves or 2 strips x 4 quarters
+    // (measured on the Llama-8B decode shapes: runs of 32..64 steps per wave stream best).
+    const auto kparts_of = [](int steps) { return steps > 192 ? 4 : (steps > 32 ? 2 : 1); };
     for (int i = 0; i < count; ++i) {
         const slimk_w2a8_problem& pr = problems[order[i]];
         if (!pr.q || !pr.s_a || !pr.rowsum || !pr.w_r || !pr.s_r || !pr.out)
