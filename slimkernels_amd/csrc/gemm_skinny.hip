@@ -1,24 +1,24 @@
-// Skinny-M (M <= 32) split-K W2A8 GEMM for gfx950: the HBM-bound decode regime.
+// Skinny-M (M <= 32) W2A8 GEMMs for gfx950: the HBM-bound decode regime.  Two kernels.
 //
-// Grid (strips, split).  A workgroup of NW (4, 8 or 16) wavefronts owns one 64-channel strip
-// and a contiguous range of scale groups; its waves take contiguous sub-ranges, so
-// each wave streams a run of 1 KiB weight units (step-major layout) straight from global
-// memory into VGPRs (one global_load_dwordx4 per lane and unit, no LDS staging:
-// nothing in a unit is shared between waves).  The activation operand of a step is
-// loaded once per wave and reused by the strip's four 16-channel sub-blocks.
-//
-// The kernel is a latency problem before it is a bandwidth problem (a whole decode
-// GEMM is a few microseconds), so every load is issued as early as possible:
-//  * weights and activations run through a register ring kDepth steps deep (the
-//    load for step s + kDepth is issued when step s is consumed);
-//  * the per-group metadata (scales, zero-points, activation row sums) of the next
-//    16 steps is fetched into registers one chunk ahead and parked in a wave-private
-//    LDS area, from which each group reads it with short ds_read latency;
+// skinny_kernel: one GEMM per launch.  Grid (strips, split, 16-row token blocks).  A workgroup of
+// NW (4, 8 or 16) wavefronts owns one 64-channel strip and a contiguous range of scale groups; its
+// waves take contiguous sub-ranges, so each wave streams a run of 1 KiB weight units (step-major
+// layout) straight from global memory into VGPRs (one buffer_load_dwordx4 per lane and unit:
+// nothing in a unit is shared between waves).  A single decode GEMM is a latency problem before
+// it is a bandwidth problem (the whole thing is a few microseconds), so every load is issued as
+// early as possible:
+//  * weights and activations run through a register ring kDepth steps deep (the load for step
+//    s + kDepth is issued when step s is consumed), addressed through buffer descriptors with a
+//    per-lane offset fixed for the kernel and a scalar offset per step;
+//  * the per-group metadata (scales, zero-points, activation row sums) is fetched into registers
+//    one chunk ahead and parked in a wave-private LDS area;
 //  * the token scales s_a needed by the epilogue are fetched at kernel entry.
-// Per group the int32 accumulators are drained into fp32 running sums with the
-// group's scale; the workgroup's waves' sums meet in LDS, and for split > 1 the
-// workgroups' partial tiles meet in the workspace, summed in a fixed order by the
-// last workgroup to arrive (deterministic, no float atomics).
+// Per group the int32 accumulators are drained into fp32 running sums with the group's fp16 scale
+// (cvt + fma_mix); the workgroup's waves' sums meet in LDS, and for split > 1 the workgroups'
+// partial tiles meet in the workspace, summed in a fixed order by the last workgroup to arrive
+// (deterministic, no float atomics).
+//
+// skinny_grouped_kernel: several GEMMs per launch, built for throughput; see shared_body below.
 #include "w2a8_launch.h"
 
 namespace w2a8 {
@@ -405,10 +405,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const GemmParams p) {
 // LDS, so that every wave of the launch streams a run of comparable length (48..96 steps) and its
 // start-up and wind-down cost is spread over enough steps.
 constexpr int kGroupedWaves = 8;
-#ifndef SLIMK_SHARE_ROWS
-#define SLIMK_SHARE_ROWS 8
-#endif
-constexpr int kShareRows = SLIMK_SHARE_ROWS;  // token rows from which activations are shared through LDS
+constexpr int kShareRows = 8;  // token rows from which activations are shared through LDS
 
 // Per-group metadata is handled in blocks of kBlockGroups groups: one block's scales, zero-points
 // and activation row sums are fetched with three or four wave-wide loads (instead of a few small
@@ -671,9 +668,10 @@ __device__ __forceinline__ void shared_body(const GemmParams& p, const int unit,
 }
 
 // Workgroup ids are cut into runs, one run per problem.  Within a problem, workgroups come in sets
-// of eight per row block: consecutive workgroup ids go to different XCDs, so the two row blocks of
-// a set of strips, eight ids apart, share an XCD and its L2.  All problems share the group size,
-// the zero-point mode and the output type.  The problem table travels in the kernel arguments.
+// of eight per 16-row token block: consecutive workgroup ids go to different XCDs, so the two row
+// blocks of a set of strips, eight ids apart, share an XCD and its L2 (the second read of the
+// weights hits there).  All problems share the group size, the zero-point mode and the output
+// type.  The problem table travels in the kernel arguments.
 template <int GS, bool ASYM, typename OutT>
 __global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_grouped_kernel(const GroupedParams gp) {
     __shared__ __attribute__((aligned(16))) GroupedSmem sm;
