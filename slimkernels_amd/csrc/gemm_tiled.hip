@@ -29,6 +29,9 @@
 
 namespace w2a8 {
 
+#ifndef SLIMK_TILED_SETPRIO
+#define SLIMK_TILED_SETPRIO 0
+#endif
 namespace fast {
 constexpr int kBN = 256;
 constexpr int kStageSteps = 2;
@@ -58,14 +61,23 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
     const int col = lane & 15, quad = lane >> 4;
 
     // Tile order: consecutive workgroup ids land on different XCDs (id % 8), each with its own
-    // L2.  Give every XCD one contiguous run of tiles, channel tile fastest, so that the tiles
-    // an XCD works on at the same time share their activation rows in that L2.
+    // L2.  When the channel tiles divide by eight, every XCD owns one band of channel tiles for all
+    // token tiles: its share of the weights then stays in its L2 for the whole kernel and only the
+    // activations stream through (token tile major, so concurrent tiles share activation rows).
+    // Otherwise every XCD gets one contiguous run of tiles, channel tile fastest.
     const int tiles_n = (p.strips + kStrips - 1) / kStrips;
     const int tiles_m = (p.M + kBM - 1) / kBM;
     const int total = tiles_m * tiles_n;
     const int per_xcd = (total + 7) / 8;
-    const int tile = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
-    if (tile >= total) return;
+    const int xcd = (int)(blockIdx.x & 7), local = (int)(blockIdx.x >> 3);
+    int tile;
+    if (tiles_n % 8 == 0) {
+        const int band = tiles_n / 8;
+        tile = (local / band) * tiles_n + xcd * band + local % band;
+    } else {
+        tile = xcd * per_xcd + local;
+    }
+    if (local >= per_xcd || tile >= total) return;
     const int m_tile = (tile / tiles_n) * kBM;
     const int strip0 = (tile % tiles_n) * kStrips;
     const int strip = min(strip0 + wave, p.strips - 1);  // clamped: a surplus wave recomputes the last strip, stores nothing
@@ -196,6 +208,9 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
 #pragma unroll
         for (int u = 0; u < kUnits; ++u) {
             const int mb = u / kGroupsPerStage, gi = u % kGroupsPerStage;
+#if SLIMK_TILED_SETPRIO
+            __builtin_amdgcn_s_setprio(1);
+#endif
 #pragma unroll
             for (int s = 0; s < GS; ++s) {
                 const int r = mb * kStageSteps + gi * GS + s;  // fragment index in consumption order
@@ -205,6 +220,9 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
                                                       s == 0 ? v4i{0, 0, 0, 0} : acc[u & 1][pp]);
                 if (r + kAQueue < kABlocks) aq[r % kAQueue] = lds_a(r + kAQueue);
             }
+#if SLIMK_TILED_SETPRIO
+            __builtin_amdgcn_s_setprio(0);
+#endif
             // drain the previous unit (for u == 0: the last unit of the previous stage, scale sc_prev)
             const int pu = (u + kUnits - 1) % kUnits;
             const int pmb = pu / kGroupsPerStage, pgi = pu % kGroupsPerStage;
