@@ -522,18 +522,31 @@ __device__ __forceinline__ void shared_body(const GemmParams& p, const int unit,
     auto issue_a = [&](int slot, int step) {
         if (!SHARE) aring[slot] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, aoff, step * kStepK, 0);
     };
+    // Shared fragments are fetched two steps wide so that every load touches whole 128-byte lines of
+    // the row-major activations: fragment f of a chunk = (step pair f / 2, row half f % 2); lane l
+    // reads row 8 * half + l / 8, 16-byte piece l % 8 of the pair's 128 bytes, and parks it where the
+    // MFMA operand order wants it (step 2 * pair + piece / 4, lane (piece % 4) * 16 + row).
     const bool loader = SHARE && swave < kDepth;  // wave-uniform
     v4u areg[NL];
+    const int frow[2] = {lane >> 3, 8 + (lane >> 3)};
+    const uint32_t fpiece = lane & 7;
     auto fetch_a = [&](int it) {  // this wave's share of the chunk that starts at iteration `it`
         if (loader) {
 #pragma unroll
-            for (int n = 0; n < NL; ++n) areg[n] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, aoff, stepof(it + swave + n * NS) * kStepK, 0);
+            for (int n = 0; n < NL; ++n) {
+                const int f = swave + n * NS;
+                areg[n] = __builtin_amdgcn_raw_buffer_load_b128(
+                    q_rsrc, (uint32_t)min(frow[f & 1], M - 1) * (uint32_t)p.ldq + fpiece * 16, stepof(it + 2 * (f >> 1)) * kStepK, 0);
+            }
         }
     };
     auto park_a = [&](int parity) {
         if (loader) {
 #pragma unroll
-            for (int n = 0; n < NL; ++n) sm.abuf[kpart][parity][swave + n * NS][lane] = areg[n];
+            for (int n = 0; n < NL; ++n) {
+                const int f = swave + n * NS;
+                sm.abuf[kpart][parity][2 * (f >> 1) + (fpiece >> 2)][(fpiece & 3) * 16 + frow[f & 1]] = areg[n];
+            }
         }
     };
 

@@ -29,9 +29,6 @@
 
 namespace w2a8 {
 
-#ifndef SLIMK_TILED_SETPRIO
-#define SLIMK_TILED_SETPRIO 0
-#endif
 namespace fast {
 constexpr int kBN = 256;
 constexpr int kStageSteps = 2;
@@ -208,9 +205,6 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
 #pragma unroll
         for (int u = 0; u < kUnits; ++u) {
             const int mb = u / kGroupsPerStage, gi = u % kGroupsPerStage;
-#if SLIMK_TILED_SETPRIO
-            __builtin_amdgcn_s_setprio(1);
-#endif
 #pragma unroll
             for (int s = 0; s < GS; ++s) {
                 const int r = mb * kStageSteps + gi * GS + s;  // fragment index in consumption order
@@ -220,9 +214,6 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
                                                       s == 0 ? v4i{0, 0, 0, 0} : acc[u & 1][pp]);
                 if (r + kAQueue < kABlocks) aq[r % kAQueue] = lds_a(r + kAQueue);
             }
-#if SLIMK_TILED_SETPRIO
-            __builtin_amdgcn_s_setprio(0);
-#endif
             // drain the previous unit (for u == 0: the last unit of the previous stage, scale sc_prev)
             const int pu = (u + kUnits - 1) % kUnits;
             const int pmb = pu / kGroupsPerStage, pgi = pu % kGroupsPerStage;
