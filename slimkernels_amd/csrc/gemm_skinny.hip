@@ -690,8 +690,11 @@ __global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_grouped_kernel(c
     __shared__ __attribute__((aligned(16))) GroupedSmem sm;
     const int wg = blockIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    int i = 0;
-    while (i + 1 < gp.count && wg >= gp.wg_begin[i + 1]) ++i;
+    // problem index = number of run boundaries at or below this workgroup id: one lane per boundary,
+    // one ballot (a serial walk of the table costs a scalar load latency per problem)
+    const int bl = min((int)(threadIdx.x & 63), kMaxGroup - 1);
+    const bool past = bl + 1 < gp.count && wg >= gp.wg_begin[bl + 1];
+    const int i = __builtin_amdgcn_readfirstlane(__builtin_popcountll(__ballot(past)));
     const GemmParams& p = gp.prob[i];
     const int local = wg - gp.wg_begin[i];
     const int mblocks = (p.M + 15) >> 4;
