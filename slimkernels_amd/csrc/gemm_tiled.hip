@@ -205,24 +205,30 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
 #pragma unroll
         for (int u = 0; u < kUnits; ++u) {
             const int mb = u / kGroupsPerStage, gi = u % kGroupsPerStage;
+            // The drain of the previous unit (for u == 0: the last unit of the previous stage, scale
+            // sc_prev) is dealt out evenly between this unit's MFMAs, with fences so that the
+            // scheduler keeps the weave: the matrix core then always has the next MFMA queued behind
+            // a few vector instructions instead of behind a whole drain.
+            const int pu = (u + kUnits - 1) % kUnits;
+            const int pmb = pu / kGroupsPerStage, pgi = pu % kGroupsPerStage;
+            constexpr int kDrainPerMfma = 16 / (GS * 4);  // elements of the previous unit per MFMA of this one
 #pragma unroll
             for (int s = 0; s < GS; ++s) {
                 const int r = mb * kStageSteps + gi * GS + s;  // fragment index in consumption order
 #pragma unroll
-                for (int pp = 0; pp < 4; ++pp)
+                for (int pp = 0; pp < 4; ++pp) {
                     acc[u & 1][pp] = mfma_i8_16x16x64(aq[r % kAQueue], b[gi * GS + s][pp],
                                                       s == 0 ? v4i{0, 0, 0, 0} : acc[u & 1][pp]);
-                if (r + kAQueue < kABlocks) aq[r % kAQueue] = lds_a(r + kAQueue);
+#pragma unroll
+                    for (int d = 0; d < kDrainPerMfma; ++d) {
+                        const int e = (s * 4 + pp) * kDrainPerMfma + d;  // 0..15: sub-block e / 4, row e % 4
+                        t[pmb][e / 4][e % 4] = __builtin_fmaf((float)acc[(u & 1) ^ 1][e / 4][e % 4],
+                                                              u == 0 ? sc_prev[e / 4] : sc[pgi][e / 4], t[pmb][e / 4][e % 4]);
+                    }
+                    if (pp == 3 && r + kAQueue < kABlocks) aq[r % kAQueue] = lds_a(r + kAQueue);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
-            // drain the previous unit (for u == 0: the last unit of the previous stage, scale sc_prev)
-            const int pu = (u + kUnits - 1) % kUnits;
-            const int pmb = pu / kGroupsPerStage, pgi = pu % kGroupsPerStage;
-#pragma unroll
-            for (int pp = 0; pp < 4; ++pp)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    t[pmb][pp][j] = __builtin_fmaf((float)acc[(u & 1) ^ 1][pp][j], u == 0 ? sc_prev[pp] : sc[pgi][pp],
-                                                   t[pmb][pp][j]);
         }
 #pragma unroll
         for (int pp = 0; pp < 4; ++pp) sc_prev[pp] = sc[kGroupsPerStage - 1][pp];
