@@ -101,18 +101,11 @@ int auto_split(int M, int N, int K, int group_size, int kernel) {
     return (G + gps - 1) / gps;
 }
 
-// Wavefronts per workgroup of the skinny kernel (the in-workgroup split of K).
-// SLIMK_W2A8_SKINNY_WAVES overrides the choice (read once; a tuning aid, not an interface).
+// Wavefronts per workgroup of the skinny kernel (the in-workgroup split of K): split runs are the
+// long-K ones, more waves per workgroup keep more loads in flight per CU.
 int skinny_waves(int M, int split) {
-    static const int forced = [] {
-        const char* e = getenv("SLIMK_W2A8_SKINNY_WAVES");
-        return e ? atoi(e) : 0;
-    }();
-    if (forced) return forced;
-    // split runs are the long-K ones: more waves per workgroup keep more loads in flight per CU
     (void)M;
-    if (split > 1) return 16;
-    return 4;
+    return split > 1 ? 16 : 4;
 }
 
 }  // namespace

@@ -23,6 +23,9 @@
 
 namespace w2a8 {
 
+// cache policy of the weight loads when every byte is used exactly once (the nt bit of the buffer
+// instruction); with two 16-row blocks the second block's read is meant to hit in L2 instead
+constexpr int kStreamOnce = 2;
 constexpr int kDepth = 4;  // ring depth in steps = steps per metadata chunk = granule of the K partition
 
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -63,7 +66,7 @@ struct SkinnySmem {
 // product over the groups (16 tokens x 16 channels x up to 4 groups of a chunk) and goes through
 // one v_mfma_f32_16x16x4_f32 per chunk and sub-block, accumulating straight into the fp32 running
 // sums (same D layout as the int8 MFMA).  The verification build folds it in integers instead.
-template <int J, int GS, int NWK, int NWP, bool ASYM, bool DUMP, typename OutT>
+template <int J, int GS, int NWK, int NWP, bool ASYM, bool DUMP, bool NT, typename OutT>
 __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip, const int split, const int mblk,
                                             const int kwave, const int pwave, SkinnySmem<NWP>& sm) {
     constexpr int MB = 1;
@@ -164,7 +167,7 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     v4u wring[kDepth];
     v4u aring[kDepth][MB];
     auto issue = [&](int slot, int step) {  // step is wave-uniform
-        wring[slot] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane, step * wstride + wbase, 0);
+        wring[slot] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane, step * wstride + wbase, NT ? kStreamOnce : 0);
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
             aring[slot][mb] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, aoff[mb], step * kStepK, 0);
@@ -381,11 +384,11 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     if (tid == 0) __hip_atomic_store(p.ws_counter + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int J, int GS, int NW, bool ASYM, bool DUMP, typename OutT>
+template <int J, int GS, int NW, bool ASYM, bool DUMP, bool NT, typename OutT>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const GemmParams p) {
     __shared__ __attribute__((aligned(16))) SkinnySmem<NW> sm;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keeps ranges and bases in SGPRs
-    skinny_body<J, GS, NW, NW, ASYM, DUMP, OutT>(p, blockIdx.x, blockIdx.y, blockIdx.z, wave, wave, sm);
+    skinny_body<J, GS, NW, NW, ASYM, DUMP, NT, OutT>(p, blockIdx.x, blockIdx.y, blockIdx.z, wave, wave, sm);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -427,7 +430,7 @@ struct GroupedSmem {
     v4u abuf[4][2][kDepth][64];  // [k-part][parity][step of the chunk][lane]
 };
 
-template <int J, int GS, int NK, bool SHARE, bool ASYM, typename OutT>
+template <int J, int GS, int NK, bool SHARE, bool ASYM, bool NT, typename OutT>
 __device__ __forceinline__ void shared_body(const GemmParams& p, const int unit, const int mblk, const int wave,
                                             GroupedSmem& sm) {
     constexpr int NS = kGroupedWaves / NK;               // waves (strips) sharing one activation stream
@@ -516,7 +519,7 @@ __device__ __forceinline__ void shared_body(const GemmParams& p, const int unit,
     // barrier); otherwise they are fetched once per sharing set and handed round through LDS.
     v4u wring[kDepth];
     auto issue_w = [&](int slot, int step) {
-        wring[slot] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane, step * wstride + wbase, 0);
+        wring[slot] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane, step * wstride + wbase, NT ? kStreamOnce : 0);
     };
     v4u aring[kDepth];
     auto issue_a = [&](int slot, int step) {
@@ -705,49 +708,51 @@ __global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_grouped_kernel(c
     // activations go through LDS once a fragment spans enough cache lines to be worth a barrier
     const int mrows = min(16, p.M - mblk * 16);
     if (nk == 1) {
-        if (p.M == 1) shared_body<1, GS, 1, false, ASYM, OutT>(p, unit, mblk, wave, sm);
-        else if (mrows < kShareRows) shared_body<4, GS, 1, false, ASYM, OutT>(p, unit, mblk, wave, sm);
-        else shared_body<4, GS, 1, true, ASYM, OutT>(p, unit, mblk, wave, sm);
+        if (p.M == 1) shared_body<1, GS, 1, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
+        else if (mrows < kShareRows) shared_body<4, GS, 1, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
+        else if (mblocks == 1) shared_body<4, GS, 1, true, ASYM, true, OutT>(p, unit, mblk, wave, sm);
+        else shared_body<4, GS, 1, true, ASYM, false, OutT>(p, unit, mblk, wave, sm);
     } else if (nk == 2) {
-        if (p.M == 1) shared_body<1, GS, 2, false, ASYM, OutT>(p, unit, mblk, wave, sm);
-        else if (mrows < kShareRows) shared_body<4, GS, 2, false, ASYM, OutT>(p, unit, mblk, wave, sm);
-        else shared_body<4, GS, 2, true, ASYM, OutT>(p, unit, mblk, wave, sm);
+        if (p.M == 1) shared_body<1, GS, 2, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
+        else if (mrows < kShareRows) shared_body<4, GS, 2, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
+        else if (mblocks == 1) shared_body<4, GS, 2, true, ASYM, true, OutT>(p, unit, mblk, wave, sm);
+        else shared_body<4, GS, 2, true, ASYM, false, OutT>(p, unit, mblk, wave, sm);
     } else {
-        if (p.M == 1) shared_body<1, GS, 4, false, ASYM, OutT>(p, unit, mblk, wave, sm);
-        else if (mrows < kShareRows) shared_body<4, GS, 4, false, ASYM, OutT>(p, unit, mblk, wave, sm);
-        else shared_body<4, GS, 4, true, ASYM, OutT>(p, unit, mblk, wave, sm);
+        if (p.M == 1) shared_body<1, GS, 4, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
+        else if (mrows < kShareRows) shared_body<4, GS, 4, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
+        else if (mblocks == 1) shared_body<4, GS, 4, true, ASYM, true, OutT>(p, unit, mblk, wave, sm);
+        else shared_body<4, GS, 4, true, ASYM, false, OutT>(p, unit, mblk, wave, sm);
     }
 }
 
-template <int J, int GS, int NW, bool ASYM, bool DUMP>
+template <int J, int GS, int NW, bool ASYM, bool DUMP, bool NT>
 static void launch_out(const GemmParams& p, bool out_bf16, hipStream_t stream) {
     const dim3 grid(p.strips, p.split, (p.M + 15) / 16), block(NW * 64);
     if (out_bf16)
-        skinny_kernel<J, GS, NW, ASYM, DUMP, OutBF16><<<grid, block, 0, stream>>>(p);
+        skinny_kernel<J, GS, NW, ASYM, DUMP, NT, OutBF16><<<grid, block, 0, stream>>>(p);
     else
-        skinny_kernel<J, GS, NW, ASYM, DUMP, OutF16><<<grid, block, 0, stream>>>(p);
+        skinny_kernel<J, GS, NW, ASYM, DUMP, NT, OutF16><<<grid, block, 0, stream>>>(p);
 }
 
-template <int J, int GS, int NW, bool DUMP>
+template <int J, int GS, int NW, bool DUMP, bool NT>
 static void launch_zm(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
-    if (asym) launch_out<J, GS, NW, true, DUMP>(p, out_bf16, stream);
-    else launch_out<J, GS, NW, false, DUMP>(p, out_bf16, stream);
+    if (asym) launch_out<J, GS, NW, true, DUMP, NT>(p, out_bf16, stream);
+    else launch_out<J, GS, NW, false, DUMP, NT>(p, out_bf16, stream);
+}
+
+template <int GS, int NW>
+static void launch_rows(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
+    if (p.M == 1) launch_zm<1, GS, NW, false, true>(p, asym, out_bf16, stream);
+    else if (p.M <= 16) launch_zm<4, GS, NW, false, true>(p, asym, out_bf16, stream);
+    else launch_zm<4, GS, NW, false, false>(p, asym, out_bf16, stream);  // two row blocks share the weights in L2
 }
 
 template <int GS>
 static void launch_nw(const GemmParams& p, int waves, bool asym, bool out_bf16, hipStream_t stream) {
     const bool dump = p.acc_dump != nullptr && p.dump_mode != 0;
-    if (dump) launch_zm<4, GS, 4, true>(p, asym, out_bf16, stream);  // verification: 4 waves, all rows
-    else if (waves >= 16) {
-        if (p.M == 1) launch_zm<1, GS, 16, false>(p, asym, out_bf16, stream);
-        else launch_zm<4, GS, 16, false>(p, asym, out_bf16, stream);
-    } else if (waves >= 8) {
-        if (p.M == 1) launch_zm<1, GS, 8, false>(p, asym, out_bf16, stream);
-        else launch_zm<4, GS, 8, false>(p, asym, out_bf16, stream);
-    } else {
-        if (p.M == 1) launch_zm<1, GS, 4, false>(p, asym, out_bf16, stream);
-        else launch_zm<4, GS, 4, false>(p, asym, out_bf16, stream);
-    }
+    if (dump) launch_zm<4, GS, 4, true, false>(p, asym, out_bf16, stream);  // verification: 4 waves, all rows
+    else if (waves >= 16) launch_rows<GS, 16>(p, asym, out_bf16, stream);
+    else launch_rows<GS, 4>(p, asym, out_bf16, stream);
 }
 
 template <int GS, bool ASYM>
