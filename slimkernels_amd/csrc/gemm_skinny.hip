@@ -496,7 +496,8 @@ __device__ __forceinline__ void shared_body(const GemmParams& p, const int unit,
 #pragma unroll
         for (int n = 0; n < 2; ++n) {  // scales: 16 groups x 128 B: lane -> group 8n + lane/8
             const size_t sgi = (size_t)max(min(gfirst + n * 8 + (lane >> 3), g1 - 1), 0) * p.strips + strip;
-            m_scale[n] = *reinterpret_cast<const v4i*>(reinterpret_cast<const char*>(p.s_r) + sgi * 128 + (lane & 7) * 16);
+            const v4i* sp = reinterpret_cast<const v4i*>(reinterpret_cast<const char*>(p.s_r) + sgi * 128 + (lane & 7) * 16);
+            m_scale[n] = NT ? __builtin_nontemporal_load(sp) : *sp;
         }
         const int gq = max(min(gfirst + (lane >> 2), g1 - 1), 0);  // row sums / zero-points: lane -> group lane/4
         if (ASYM)
