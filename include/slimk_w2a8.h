@@ -135,7 +135,9 @@ int slimk_w2a8_act_quant(const void* x, int ldx, int x_dtype, int M, int K, int 
  *   workspace                : required when the effective split_k > 1
  *                              (slimk_w2a8_gemm_workspace_bytes), else may be NULL
  *   kernel, split_k          : SLIMK_KERNEL_* and the split-K factor; 0 = choose.  split_k is an upper
- *                              bound: a split owns whole 256-element chunks of K, so fewer may be used */
+ *                              bound: a split owns whole 256-element chunks of K, so fewer may be used
+ * Repacked weights and activations are addressed with 32-bit offsets: more than 2 GiB of either
+ * is SLIMK_ERR_UNSUPPORTED. */
 int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,
                     const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
                     int M, int N, int K, int group_size,
@@ -162,12 +164,14 @@ typedef struct slimk_w2a8_problem {
 
 /* Several independent skinny (M <= 32) GEMMs in ONE kernel launch.  A decode step issues many
  * small GEMMs whose individual run time is a few microseconds of mostly launch and memory
- * latency; run together they fill the chip and stream from HBM at full rate.
+ * latency; run together they fill the chip and stream from HBM at several times the rate
+ * (the throughput-oriented kernel: eight-wave workgroups, activations shared through LDS).
  * `problems` is a HOST array of `count` (1..SLIMK_W2A8_MAX_GROUP) entries, copied into the
  * kernel arguments (so the call is graph-capturable and the array may be reused at once).
- * All problems share group_size, out_dtype and the zero-point mode (all zp_r NULL with
- * zp_const == 2, all zp_r NULL with other constants, or all zp_r non-NULL); M, N, K may
- * differ.  No split-K, no workspace.  No upstream counterpart. */
+ * All problems share group_size and out_dtype, and either all carry per-group zero-points
+ * (zp_r non-NULL) or none does (each then uses its own zp_const); M, N, K may differ.
+ * No split-K, no workspace.  For a single problem slimk_w2a8_gemm is the faster call.
+ * No upstream counterpart. */
 int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int group_size, int out_dtype,
                             void* stream);
 

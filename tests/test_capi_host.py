@@ -98,6 +98,8 @@ def test_gemm_argument_validation(L):
     assert _gemm(L, K=14336, ldq=14336) == 5 and b"workspace" in L.slimk_w2a8_last_error()
     assert _gemm(L, K=14336, ldq=14336, ws=FAKE, wsb=1024) == 5
     assert _gemm(L, split=64) == 2                                     # more splits than groups
+    # 32-bit buffer offsets: more than 2 GiB of repacked weights is refused, not mis-addressed
+    assert _gemm(L, N=1 << 19, ldo=1 << 19, K=1 << 16, ldq=1 << 16) == 7 and b"2 GiB" in L.slimk_w2a8_last_error()
 
 
 def test_repack_and_act_quant_validation(L):
