@@ -61,7 +61,7 @@ enum slimk_dtype { SLIMK_F16 = 0, SLIMK_BF16 = 1 };
 enum slimk_kernel {
     SLIMK_KERNEL_AUTO = 0,   /* skinny split-K for M <= 32, tiled otherwise */
     SLIMK_KERNEL_SKINNY = 1, /* weight-streaming split-K kernel, M <= 32 */
-    SLIMK_KERNEL_TILED = 2   /* LDS double-buffered MFMA tile kernel, any M */
+    SLIMK_KERNEL_TILED = 2   /* LDS-pipelined MFMA tile kernel, any M */
 };
 
 /* what the optional int32 verification buffer receives */
@@ -85,7 +85,10 @@ size_t slimk_w2a8_repacked_scale_bytes(int N, int K, int group_size);
 size_t slimk_w2a8_repacked_zp_bytes(int N, int K, int group_size);
 
 /* Split-K factor slimk_w2a8_gemm would choose for this problem (1 = no workspace needed),
- * and the workspace bytes a given split needs (0 when split_k <= 1).
+ * and the workspace bytes a given split needs (0 when split_k <= 1).  Both kernels can split K:
+ * the skinny one when few strips leave CUs idle, the tiled one when it has fewer 64-row tiles
+ * than CUs and K is long.  Split results are deterministic (partials are added in split order)
+ * but their fp32 summation order differs from the unsplit one.
  * No upstream counterpart: upstream has no split-K launcher (the idea appears only in
  * slimkernels/triton/gemm_splitk.ipynb cell 0). */
 int slimk_w2a8_gemm_auto_split_k(int M, int N, int K, int group_size, int kernel);

@@ -86,8 +86,11 @@ int groups_per_split(int G, int group_size, int split) {
 // costs about 3 us.  Only a large matrix with few strips (small N, long K) is split, up to about
 // 256 workgroups, because a quarter of the CUs cannot pull full HBM bandwidth.
 int auto_split(int M, int N, int K, int group_size, int kernel) {
-    (void)M;
-    if (kernel != SLIMK_KERNEL_SKINNY) return 1;
+    if (kernel != SLIMK_KERNEL_SKINNY) {
+        // the fast tiled kernel splits K when its tiles would leave CUs idle (group 64 / 128 only)
+        if (group_size > 128) return 1;
+        return w2a8::tiled_fast_auto_split(M, strips_of(N), K / w2a8::kStepK);
+    }
     const int strips = strips_of(N);
     const int G = K / group_size;
     const int chunks = (K / 64 + 3) / 4;
@@ -140,8 +143,12 @@ size_t slimk_w2a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int 
     if (M <= 0 || N <= 0 || !shape_ok(K, group_size)) return 0;
     const int kern = resolve_kernel(M, kernel);
     if (split_k <= 0) split_k = auto_split(M, N, K, group_size, kern);
-    if (split_k <= 1 || kern != SLIMK_KERNEL_SKINNY) return 0;
+    if (split_k <= 1) return 0;
     const int strips = strips_of(N);
+    if (kern != SLIMK_KERNEL_SKINNY) {  // one arrival counter and `split_k` fp32 tiles of 64 x 256 per 64-row tile
+        const size_t tiles = w2a8::tiled_fast_workspace_tiles(M, strips);
+        return counter_bytes((int)tiles) + (size_t)split_k * tiles * 64 * 256 * sizeof(float);
+    }
     const int mblocks = (M + 15) / 16;  // one tile and one arrival counter per (strip, block of 16 rows)
     const size_t tile = (size_t)16 * w2a8::kStripN;
     return counter_bytes(strips * mblocks) + (size_t)split_k * strips * mblocks * tile * sizeof(float);
@@ -213,12 +220,31 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
     if (kern == SLIMK_KERNEL_SKINNY && M > 32)
         return fail(SLIMK_ERR_UNSUPPORTED, "the skinny kernel handles M <= 32 (M=%d)", M);
     const int G = K / group_size;
+    const bool split_chosen_here = split_k <= 0;
     if (split_k <= 0) split_k = auto_split(M, N, K, group_size, kern);
-    if (kern == SLIMK_KERNEL_TILED && split_k != 1)
-        return fail(SLIMK_ERR_UNSUPPORTED, "the tiled kernel has no split-K (split_k=%d)", split_k);
     if (split_k > G) return fail(SLIMK_ERR_BAD_SHAPE, "split_k=%d exceeds the number of groups %d", split_k, G);
-    const int gps = groups_per_split(G, group_size, split_k);
-    split_k = (G + gps - 1) / gps;  // effective split: the request is an upper bound (whole chunks per split)
+    int gps;
+    if (kern == SLIMK_KERNEL_TILED) {
+        // only the fast kernel (uniform zero-point 2, no dump, group 64 / 128) with 64-row tiles splits K
+        w2a8::GemmParams probe{};
+        probe.acc_dump = dump_mode != SLIMK_DUMP_NONE ? acc_dump : nullptr; probe.dump_mode = dump_mode;
+        probe.zp_const = zp_const; probe.steps = K / w2a8::kStepK;
+        const bool can = w2a8::tiled_fast_supported(probe, group_size / w2a8::kStepK, zp_r != nullptr) &&
+                         w2a8::tiled_fast_max_split(M, strips_of(N), K / w2a8::kStepK) > 1 &&
+                         (size_t)split_k * w2a8::tiled_fast_workspace_tiles(M, strips_of(N)) * 64 * 256 * 4 < 0x7fffffffu;
+        if (split_k > 1 && !can) {
+            if (!split_chosen_here)
+                return fail(SLIMK_ERR_UNSUPPORTED, "this tiled GEMM cannot split K (split_k=%d)", split_k);
+            split_k = 1;
+        }
+        const int stages = K / (2 * w2a8::kStepK);
+        const int sps = split_k > 1 ? (stages + split_k - 1) / split_k : stages;
+        if (split_k > 1) split_k = (stages + sps - 1) / sps;  // effective split: whole 128-element stages per split
+        gps = split_k > 1 ? sps * (128 / group_size) : G;
+    } else {
+        gps = groups_per_split(G, group_size, split_k);
+        split_k = (G + gps - 1) / gps;  // effective split: the request is an upper bound (whole chunks per split)
+    }
 
     w2a8::GemmParams p{};
     p.q = q; p.s_a = s_a; p.rowsum = rowsum; p.w_r = w_r; p.s_r = s_r; p.zp_r = zp_r;
@@ -235,7 +261,9 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
             return fail(SLIMK_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, need);
         if (!aligned16(workspace)) return fail(SLIMK_ERR_MISALIGNED, "workspace must be 16-byte aligned");
         p.ws_counter = reinterpret_cast<unsigned*>(workspace);
-        p.ws_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counter_bytes(p.strips * ((M + 15) / 16)));
+        const int counters = kern == SLIMK_KERNEL_SKINNY ? p.strips * ((M + 15) / 16)
+                                                         : (int)w2a8::tiled_fast_workspace_tiles(M, p.strips);
+        p.ws_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counter_bytes(counters));
     }
 
     hipStream_t st = (hipStream_t)stream;

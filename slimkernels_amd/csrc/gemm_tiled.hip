@@ -38,7 +38,7 @@ constexpr int kAQueue = 4;                                 // activation fragmen
 
 // BM = token rows of the workgroup tile: 128, or 64 when 128-row tiles would leave CUs idle
 // (fewer tiles than CUs, or a single workgroup per CU with nothing to hide its latencies behind).
-template <int BM, int GS, typename OutT>
+template <int BM, int GS, bool SPLIT, bool ZP, typename OutT>
 __device__ __forceinline__ void tiled_body(const GemmParams& p) {
     using namespace fast;
     constexpr int kBM = BM;
@@ -79,7 +79,11 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
     const int strip0 = (tile % tiles_n) * kStrips;
     const int strip = min(strip0 + wave, p.strips - 1);  // clamped: a surplus wave recomputes the last strip, stores nothing
     const bool strip_ok = strip0 + wave < p.strips;
-    const int n_stages = p.steps / kStageSteps;
+    // this workgroup's share of K in stages (all of it unless K is split over blockIdx.y)
+    const int all_stages = p.steps / kStageSteps;
+    const int stages_per_split = SPLIT ? p.groups_per_split / (kStageSteps / GS) : all_stages;
+    const int stage0 = SPLIT ? (int)blockIdx.y * stages_per_split : 0;
+    const int n_stages = min(stages_per_split, all_stages - stage0);
 
     // ---- loads, one stage ahead, all through buffer instructions: a wave-uniform descriptor plus a
     // scalar offset that advances per stage, so no vector ALU work goes into addresses, and rows
@@ -105,6 +109,7 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
     const uint32_t s_lane_off = (uint32_t)(strip * 16 + col) * 8;
     const uint32_t s_group_stride = (uint32_t)p.strips * 128;               // bytes between groups of a strip
     typedef unsigned v2u __attribute__((ext_vector_type(2)));
+    typedef unsigned v4u_t __attribute__((ext_vector_type(4)));
     v2u sraw[kGroupsPerStage];
     // Activations and this wave's weight units go straight from global memory into LDS (no registers
     // held while in flight), two stages ahead; the scales, a few bytes, go to registers one stage ahead.
@@ -114,18 +119,18 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
         for (int i = 0; i < kALoads; ++i)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
                 q_rsrc, (__attribute__((address_space(3))) void*)&lds[buf][(wave + 4 * i) * 256], 16, a_off[i],
-                stage * (kStageSteps * kStepK), 0, 0);
+                (stage0 + stage) * (kStageSteps * kStepK), 0, 0);
 #pragma unroll
         for (int s = 0; s < kStageSteps; ++s)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
                 w_rsrc, (__attribute__((address_space(3))) void*)&lds[buf][kStageDwords + (wave * kStageSteps + s) * 256], 16,
-                lane * 16, (stage * kStageSteps + s) * b_step_stride + b_strip_off, 0, 0);
+                lane * 16, ((stage0 + stage) * kStageSteps + s) * b_step_stride + b_strip_off, 0, 0);
     };
     auto fetch_scales = [&](int stage) {
 #pragma unroll
         for (int gi = 0; gi < kGroupsPerStage; ++gi)
             sraw[gi] = __builtin_amdgcn_raw_buffer_load_b64(
-                s_rsrc, s_lane_off, (stage * kGroupsPerStage + gi) * s_group_stride, 0);
+                s_rsrc, s_lane_off, ((stage0 + stage) * kGroupsPerStage + gi) * s_group_stride, 0);
     };
     // All but the newest stage's LDS-direct loads of this wave have arrived (loads complete in issue
     // order; the newest kLdsLoads may still be in flight), then meet the other waves.
@@ -147,6 +152,55 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
     fetch_scales(0);
     fetch(0, 0);
     fetch(min(1, n_stages - 1), 1);
+
+    if (ZP) {
+        // Zero-points other than the 2 the operand bytes are centred on: the missing term
+        // -(zp - 2) * scale * rowsum of this workgroup's groups goes into the running sums first, as a
+        // small matrix product over the groups through v_mfma_f32_16x16x4_f32 (lane (col, quad) supplies
+        // token col / channel col of group 4b + quad; same D layout as the int8 MFMA), four blocks of
+        // four groups per round so that a round's loads are in flight together.
+        typedef float v4f __attribute__((ext_vector_type(4)));
+        typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+        constexpr int kRound = 4;
+        const int g_lo = stage0 * kGroupsPerStage, g_cnt = n_stages * kGroupsPerStage;
+        const uint32_t* zp32 = reinterpret_cast<const uint32_t*>(p.zp_r);
+        int rrow[kMB];
+#pragma unroll
+        for (int mb = 0; mb < kMB; ++mb) rrow[mb] = min(m_tile + mb * 16 + col, p.M - 1);
+        for (int gb = 0; gb < g_cnt; gb += 4 * kRound) {
+            v2u zs[kRound];
+            uint32_t zz[kRound];
+            int rs[kRound][kMB];
+#pragma unroll
+            for (int b = 0; b < kRound; ++b) {
+                const int g = g_lo + min(gb + 4 * b + quad, g_cnt - 1);  // clamped; masked below
+                zs[b] = __builtin_amdgcn_raw_buffer_load_b64(s_rsrc, s_lane_off, g * s_group_stride, 0);
+                zz[b] = p.zp_r ? zp32[((size_t)g * p.strips + strip) * 16 + col] : (uint32_t)p.zp_const * 0x01010101u;
+#pragma unroll
+                for (int mb = 0; mb < kMB; ++mb) rs[b][mb] = p.rowsum[(size_t)g * p.ldr + rrow[mb]];
+            }
+#pragma unroll
+            for (int b = 0; b < kRound; ++b) {
+                const bool on = gb + 4 * b + quad < g_cnt;
+                const v4h sh = __builtin_bit_cast(v4h, zs[b]);
+                float zb[4];
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp)
+                    zb[pp] = on ? (2.0f - (float)((zz[b] >> (8 * pp)) & 0xffu)) * (float)sh[pp] : 0.0f;
+#pragma unroll
+                for (int mb = 0; mb < kMB; ++mb) {
+                    const float rsf = (float)rs[b][mb];
+#pragma unroll
+                    for (int pp = 0; pp < 4; ++pp) {
+                        v4f c = {t[mb][pp][0], t[mb][pp][1], t[mb][pp][2], t[mb][pp][3]};
+                        c = __builtin_amdgcn_mfma_f32_16x16x4f32(rsf, zb[pp], c, 0, 0, 0);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) t[mb][pp][j] = c[j];
+                    }
+                }
+            }
+        }
+    }
     land();
 
     // accumulator sets (two, alternating) and the scale of the unit carried over a stage boundary;
@@ -243,9 +297,56 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
         for (int j = 0; j < 4; ++j)
             t[kMB - 1][pp][j] = __builtin_fmaf((float)acc[1][pp][j], sc_prev[pp], t[kMB - 1][pp][j]);
 
+    uint16_t* out = reinterpret_cast<uint16_t*>(p.out);
+    if (SPLIT) {
+        // ---- split-K: every workgroup of the tile publishes its fp32 partial sums (fragment order:
+        // the wave that reduces them has the same lane layout, so no transposition), the last to
+        // arrive adds them up in split order (deterministic) and finishes.  Agent-scope relaxed
+        // atomics: write-through stores and cache-bypassing loads, no L2 fence needed.
+        // Partials move as 16-byte buffer stores / loads at system-coherent cache policy (write-through,
+        // read around the L2 of whichever XCD the reducing workgroup runs on): plain memory
+        // instructions, so the reduction's loads are all in flight together.
+        constexpr int kTileBytes = kBM * kBN * 4;
+        constexpr int kCoherent = 17;  // sc0 | sc1
+        typedef float v4f __attribute__((ext_vector_type(4)));
+        const int n_split = (int)gridDim.y;
+        const __amdgpu_buffer_rsrc_t ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            p.ws_partial, 0, (int)((size_t)n_split * total * kTileBytes), 0x00020000);
+        const uint32_t ws_lane = (uint32_t)wave * (kMB * 16 * 64 * 4) + lane * 16;   // this wave's fragments, this lane's 16 bytes
+        const uint32_t ws_tile = (uint32_t)tile * kTileBytes;
+        const uint32_t ws_split_pitch = (uint32_t)total * kTileBytes;
+#pragma unroll
+        for (int mb = 0; mb < kMB; ++mb)
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp) {
+                const v4f v = {t[mb][pp][0], t[mb][pp][1], t[mb][pp][2], t[mb][pp][3]};
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_t, v), ws_rsrc, ws_lane + (mb * 4 + pp) * 1024,
+                                                       blockIdx.y * ws_split_pitch + ws_tile, kCoherent);
+            }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned prev = __hip_atomic_fetch_add(p.ws_counter + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            lds[0][0] = (prev == (unsigned)(n_split - 1));
+        }
+        __syncthreads();
+        if (lds[0][0] == 0) return;
+#pragma unroll
+        for (int mb = 0; mb < kMB; ++mb)
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp) {
+                v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+                for (int sp = 0; sp < n_split; ++sp)
+                    v += __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
+                             ws_rsrc, ws_lane + (mb * 4 + pp) * 1024, sp * ws_split_pitch + ws_tile, kCoherent));
+#pragma unroll
+                for (int j = 0; j < 4; ++j) t[mb][pp][j] = v[j];
+            }
+        if (tid == 0) __hip_atomic_store(p.ws_counter + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
     // ---- epilogue: out = cast(t * s_a[m])
     if (!strip_ok) return;
-    uint16_t* out = reinterpret_cast<uint16_t*>(p.out);
 #pragma unroll
     for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
@@ -262,46 +363,90 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
 }
 
 // 128-row tiles: two workgroups (eight waves) per CU; 64-row tiles need fewer registers: three.
-template <int GS, typename OutT>
+template <int GS, bool ZP, typename OutT>
 __global__ __launch_bounds__(256, 2) void tiled_kernel(const GemmParams p) {
-    tiled_body<128, GS, OutT>(p);
+    tiled_body<128, GS, false, ZP, OutT>(p);
 }
-template <int GS, typename OutT>
+template <int GS, bool SPLIT, bool ZP, typename OutT>
 __global__ __launch_bounds__(256, 3) void tiled_kernel_bm64(const GemmParams p) {
-    tiled_body<64, GS, OutT>(p);
+    tiled_body<64, GS, SPLIT, ZP, OutT>(p);
 }
 
 bool tiled_fast_supported(const GemmParams& p, int gs, bool asym) {
+    (void)asym;
     const bool dump = p.acc_dump != nullptr && p.dump_mode != 0;
-    return !asym && !dump && p.zp_const == 2 && (gs == 1 || gs == 2) && p.steps % fast::kStageSteps == 0;
+    return !dump && (gs == 1 || gs == 2) && p.steps % fast::kStageSteps == 0;
+}
+
+// Tile height and tile count of the fast kernel for a problem: two workgroups fit a CU, so below
+// about two 128-row tiles per CU, 64-row tiles fill the chip better.
+static void tiled_fast_tiles(int M, int strips, int* bm, int* tiles) {
+    const int tiles_n = (strips + fast::kStrips - 1) / fast::kStrips;
+    const int tiles128 = tiles_n * ((M + 127) / 128);
+    static const int forced_bm = [] { const char* e = getenv("SLIMK_W2A8_TILED_BM"); return e ? atoi(e) : 0; }();
+    const bool small = forced_bm ? forced_bm == 64 : tiles128 < 2 * 256;
+    *bm = small ? 64 : 128;
+    *tiles = small ? tiles_n * ((M + 63) / 64) : tiles128;
+}
+
+int tiled_fast_max_split(int M, int strips, int steps) {
+    int bm, tiles;
+    tiled_fast_tiles(M, strips, &bm, &tiles);
+    if (bm != 64 || steps % fast::kStageSteps != 0) return 1;
+    return steps / fast::kStageSteps;
+}
+
+// With fewer 64-row tiles than CUs and a long reduction, K is split over up to four workgroups per
+// tile so that about two workgroups per CU exist.  Measured: a lone workgroup on a CU spends about a
+// microsecond per 128-element stage whatever it does, so splitting pays once a split still runs 28
+// stages or more (K >= 7168); below that the exchange of partial tiles costs more than it saves.
+int tiled_fast_auto_split(int M, int strips, int steps) {
+    int bm, tiles;
+    tiled_fast_tiles(M, strips, &bm, &tiles);
+    if (bm != 64 || steps % fast::kStageSteps != 0 || tiles >= 256) return 1;
+    const int stages = steps / fast::kStageSteps;
+    int split = (512 + tiles - 1) / tiles;
+    if (split > 4) split = 4;
+    if (split > stages / 28) split = stages / 28;
+    if (split < 1) split = 1;
+    const int sps = (stages + split - 1) / split;
+    return (stages + sps - 1) / sps;
+}
+
+size_t tiled_fast_workspace_tiles(int M, int strips) {
+    int bm, tiles;
+    tiled_fast_tiles(M, strips, &bm, &tiles);
+    return (size_t)tiles;
 }
 
 hipError_t launch_tiled(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream) {
     if (!tiled_fast_supported(p, gs, asym)) return launch_tiled_generic(p, gs, asym, out_bf16, stream);
-    const int tiles_n = (p.strips + fast::kStrips - 1) / fast::kStrips;
-    const int tiles128 = tiles_n * ((p.M + 127) / 128);
-    // two workgroups fit a CU: below about two 128-row tiles per CU, 64-row tiles fill the chip better
-    static const int forced_bm = [] { const char* e = getenv("SLIMK_W2A8_TILED_BM"); return e ? atoi(e) : 0; }();
-    const bool small = forced_bm ? forced_bm == 64 : tiles128 < 2 * 256;
-    const int tiles = small ? tiles_n * ((p.M + 63) / 64) : tiles128;
-    const dim3 grid((tiles + 7) / 8 * 8), block(256);
-    if (small) {
-        if (gs == 1) {
-            if (out_bf16) tiled_kernel_bm64<1, OutBF16><<<grid, block, 0, stream>>>(p);
-            else tiled_kernel_bm64<1, OutF16><<<grid, block, 0, stream>>>(p);
-        } else {
-            if (out_bf16) tiled_kernel_bm64<2, OutBF16><<<grid, block, 0, stream>>>(p);
-            else tiled_kernel_bm64<2, OutF16><<<grid, block, 0, stream>>>(p);
-        }
+    int bm, tiles;
+    tiled_fast_tiles(p.M, p.strips, &bm, &tiles);
+    const dim3 grid((tiles + 7) / 8 * 8, p.split > 1 ? p.split : 1), block(256);
+    const bool zp = asym || p.zp_const != 2;
+    const bool split = bm == 64 && p.split > 1;
+#define SLIMK_TILED_LAUNCH(GSV, ZPV)                                                                          \
+    do {                                                                                                      \
+        if (bm == 128) {                                                                                      \
+            if (out_bf16) tiled_kernel<GSV, ZPV, OutBF16><<<grid, block, 0, stream>>>(p);                     \
+            else tiled_kernel<GSV, ZPV, OutF16><<<grid, block, 0, stream>>>(p);                               \
+        } else if (split) {                                                                                   \
+            if (out_bf16) tiled_kernel_bm64<GSV, true, ZPV, OutBF16><<<grid, block, 0, stream>>>(p);          \
+            else tiled_kernel_bm64<GSV, true, ZPV, OutF16><<<grid, block, 0, stream>>>(p);                    \
+        } else {                                                                                              \
+            if (out_bf16) tiled_kernel_bm64<GSV, false, ZPV, OutBF16><<<grid, block, 0, stream>>>(p);         \
+            else tiled_kernel_bm64<GSV, false, ZPV, OutF16><<<grid, block, 0, stream>>>(p);                   \
+        }                                                                                                     \
+    } while (0)
+    if (gs == 1) {
+        if (zp) SLIMK_TILED_LAUNCH(1, true);
+        else SLIMK_TILED_LAUNCH(1, false);
     } else {
-        if (gs == 1) {
-            if (out_bf16) tiled_kernel<1, OutBF16><<<grid, block, 0, stream>>>(p);
-            else tiled_kernel<1, OutF16><<<grid, block, 0, stream>>>(p);
-        } else {
-            if (out_bf16) tiled_kernel<2, OutBF16><<<grid, block, 0, stream>>>(p);
-            else tiled_kernel<2, OutF16><<<grid, block, 0, stream>>>(p);
-        }
+        if (zp) SLIMK_TILED_LAUNCH(2, true);
+        else SLIMK_TILED_LAUNCH(2, false);
     }
+#undef SLIMK_TILED_LAUNCH
     return hipGetLastError();
 }
 

@@ -29,6 +29,12 @@ hipError_t launch_skinny_grouped(const GroupedParams& gp, int gs, bool asym, boo
 // launch_tiled picks the fast kernel when it applies (uniform zero-point 2, group 64/128, K % 128 == 0,
 // no verification dump) and the generic one otherwise.
 hipError_t launch_tiled(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
+// Split-K of the fast tiled kernel (64-row tiles only): the factor it would choose, the largest it
+// accepts, and the number of tiles a split workspace must hold (64 x 256 fp32 each, per split).
+bool tiled_fast_supported(const GemmParams& p, int gs, bool asym);
+int tiled_fast_auto_split(int M, int strips, int steps);
+int tiled_fast_max_split(int M, int strips, int steps);
+size_t tiled_fast_workspace_tiles(int M, int strips);
 hipError_t launch_tiled_generic(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
 
 }  // namespace w2a8

@@ -59,8 +59,11 @@ def test_split_heuristic_and_workspace(L):
     assert ws == 256 + s * 64 * (16 * 64) * 4     # counters + split x strips x (16 x 64 fp32 tile)
     # 17..32 tokens run as two blocks of 16 rows: one counter and one tile per (strip, block)
     assert L.slimk_w2a8_gemm_workspace_bytes(32, 4096, 14336, 128, _lib.KERNEL_AUTO, 4) == 512 + 4 * 64 * 2 * (16 * 64) * 4
-    # the tiled kernel never splits
-    assert L.slimk_w2a8_gemm_auto_split_k(512, 4096, 14336, 128, _lib.KERNEL_AUTO) == 1
+    # the tiled kernel splits K only when its 64-row tiles would leave CUs idle
+    assert L.slimk_w2a8_gemm_auto_split_k(4096, 14336, 4096, 128, _lib.KERNEL_AUTO) == 1
+    s = L.slimk_w2a8_gemm_auto_split_k(512, 4096, 14336, 128, _lib.KERNEL_AUTO)      # 16 x 8 tiles, 112 stages
+    assert s == 4
+    assert L.slimk_w2a8_gemm_workspace_bytes(512, 4096, 14336, 128, _lib.KERNEL_AUTO, 0) == 512 + s * 128 * (64 * 256) * 4
     assert L.slimk_w2a8_gemm_auto_split_k(0, 4096, 4096, 128, 0) == 0
 
 
@@ -93,7 +96,8 @@ def test_gemm_argument_validation(L):
     assert _gemm(L, dump=3) == 4
     assert _gemm(L, dump=1, acc=None) == 1
     assert _gemm(L, M=64, ldr=64, kernel=_lib.KERNEL_SKINNY) == 7
-    assert _gemm(L, M=64, ldr=64, kernel=_lib.KERNEL_TILED, split=2) == 7
+    assert _gemm(L, M=64, ldr=64, kernel=_lib.KERNEL_TILED, split=2) == 5       # valid, but needs a workspace
+    assert _gemm(L, M=64, ldr=64, kernel=_lib.KERNEL_TILED, split=2, dump=2, acc=FAKE) == 7   # the verification kernel cannot split
     # split-K without / with too small a workspace (N = 4096, K = 14336 wants split 4)
     assert _gemm(L, K=14336, ldq=14336) == 5 and b"workspace" in L.slimk_w2a8_last_error()
     assert _gemm(L, K=14336, ldq=14336, ws=FAKE, wsb=1024) == 5

@@ -41,6 +41,7 @@ def _check_case(gpu_ops, oracle, case, sample_rows, seed=0):
     qa = gpu_ops.quantize_act_int8(xd, case.group_size)
     odt = pu.torch_dtype(case)
     out = gpu_ops.w2a8_gemm(qa, w, odt)
+    out_unsplit = gpu_ops.w2a8_gemm(qa, w, odt, split_k=1) if M > 32 else None
     _, acc_sum = gpu_ops.w2a8_gemm(qa, w, odt, dump="sum")
     torch.cuda.synchronize()
 
@@ -63,9 +64,10 @@ def _check_case(gpu_ops, oracle, case, sample_rows, seed=0):
     rows_t = torch.from_numpy(rows).cuda()
     np.testing.assert_array_equal(acc_sum[rows_t].cpu().numpy(), ref_sum)
     got_bits = pu.out_tensor_bits(out[rows_t])
-    if M > 32:      # tiled kernel: same summation order as the oracle
-        np.testing.assert_array_equal(got_bits, ref_bits)
-    else:           # skinny split-K: the output criterion (1 ULP or rtol 1e-3, plus fp32 re-association noise)
+    if M > 32:      # tiled kernel, K unsplit: same summation order as the oracle
+        np.testing.assert_array_equal(pu.out_tensor_bits(out_unsplit[rows_t]), ref_bits)
+    if True:        # the library's own choice (skinny, or tiled with K possibly split): the output criterion
+                    # (1 ULP or rtol 1e-3, plus fp32 re-association noise)
         g, r = pu.bits_to_f32(got_bits, bf16), pu.bits_to_f32(ref_bits, bf16)
         # bound the re-association noise by G * 2^-24 * s_a * sum_g |acc_g| * scale <= G * 2^-24 * s_a * K * 127 * 3 * max scale
         smax = float(scales.astype(np.float32).max())

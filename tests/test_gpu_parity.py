@@ -116,8 +116,31 @@ def test_skinny_small(gpu_ops, oracle, M, N, K, g, mode, out):
 ])
 def test_tiled_small(gpu_ops, oracle, M, N, K, g, mode, out):
     case = pu.small_case(M, N, K, g, mode, seed=M + N + 1, out_dtype=out)
-    _run_case(gpu_ops, oracle, case, "tiled", dump="groups", exact_out=True)
-    _run_case(gpu_ops, oracle, case, "tiled", dump="sum", exact_out=True)
+    # unsplit and with the zero-point the operand bytes are centred on (the symmetric levels), the tiled
+    # kernels sum the groups in the oracle's order: bit-identical outputs.  Other zero-points add their
+    # term through fp32 MFMAs first: the output criterion.
+    exact = mode == "sym"
+    _run_case(gpu_ops, oracle, case, "tiled", split_k=1, dump="groups", exact_out=exact)
+    _run_case(gpu_ops, oracle, case, "tiled", split_k=1, dump="sum", exact_out=exact)
+    # whatever split the library picks by itself (K may be split when tiles are few): the output criterion
+    _run_case(gpu_ops, oracle, case, "tiled", split_k=0, dump="sum")
+
+
+@pytest.mark.parametrize("M,N,K,g,out,split", [(64, 256, 2048, 128, "float16", 2), (77, 300, 4096, 64, "bfloat16", 4),
+                                                 (130, 64, 3072, 128, "float16", 3), (40, 512, 8192, 128, "float16", 8)])
+def test_tiled_split_k(gpu_ops, oracle, M, N, K, g, out, split):
+    """Split-K of the fast tiled kernel: the output criterion, and run-to-run identical bits."""
+    case = pu.small_case(M, N, K, g, "sym", seed=M + K, out_dtype=out)
+    packed, scales, zero = pu.quantized_weight(case)
+    x = workloads.make_activation(case)
+    bf16 = out == "bfloat16"
+    w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, x)
+    qa = gpu_ops.quantize_act_int8(xd, g)
+    outs = [pu.out_tensor_bits(gpu_ops.w2a8_gemm(qa, w, pu.torch_dtype(case), kernel="tiled", split_k=split)) for _ in range(4)]
+    for o in outs[1:]:
+        np.testing.assert_array_equal(o, outs[0])
+    ref = oracle.reference_forward(x, packed, scales, zero, g, out_bf16=bf16)
+    pu.assert_out_close(outs[0], ref["out_bits"], bf16, pu.reorder_bound(ref["acc"], scales, ref["s_a"]), f"tiled split {split}")
 
 
 def test_split_k_is_deterministic_and_workspace_reusable(gpu_ops, oracle):
@@ -150,7 +173,7 @@ def test_config_c2_decode(gpu_ops, oracle, shape, M):
 
 def test_config_c5_asym_ragged(gpu_ops, oracle):
     a, b = workloads.config_cases("c5")
-    _run_case(gpu_ops, oracle, a, "auto", exact_out=True)  # M = 77 -> tiled
+    _run_case(gpu_ops, oracle, a, "auto")                  # M = 77 -> tiled, per-group zero-points
     _run_case(gpu_ops, oracle, b, "auto")                  # M = 1  -> skinny split-K
 
 
