@@ -327,7 +327,7 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
         gp.wg_begin[i] = wgs;
         gp.kparts[i] = kparts_of(g.steps);
         // units (sets of 8, 4 or 2 strips) in whole sets of eight, times the row blocks of 16 tokens
-        const int per_unit = 8 / gp.kparts[i];
+        const int per_unit = w2a8::kGroupedWavesPerWg / gp.kparts[i];
         const int units = (g.strips + per_unit - 1) / per_unit;
         wgs += (units + 7) / 8 * 8 * ((pr.M + 15) / 16);
     }

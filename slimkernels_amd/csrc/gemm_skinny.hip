@@ -407,7 +407,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const GemmParams p) {
 // reduce, each wave stores its own D fragments); long ones split K over 2 or 4 parts that meet in
 // LDS, so that every wave of the launch streams a run of comparable length (48..96 steps) and its
 // start-up and wind-down cost is spread over enough steps.
-constexpr int kGroupedWaves = 8;
+constexpr int kGroupedWaves = kGroupedWavesPerWg;  // w2a8_common.h: the host sizes the grid with it
 constexpr int kShareRows = 8;  // token rows from which activations are shared through LDS
 
 // Per-group metadata is handled in blocks of kBlockGroups groups: one block's scales, zero-points
