@@ -23,8 +23,6 @@
 //  * three stage buffers: the loads of stage s+2 are in flight while stage s is consumed, one
 //    barrier per 128-element stage (with one workgroup on a CU there is no other wave to hide a
 //    stage's load latency behind).
-#include <stdlib.h>
-
 #include "w2a8_launch.h"
 
 namespace w2a8 {
@@ -383,8 +381,7 @@ bool tiled_fast_supported(const GemmParams& p, int gs, bool asym) {
 static void tiled_fast_tiles(int M, int strips, int* bm, int* tiles) {
     const int tiles_n = (strips + fast::kStrips - 1) / fast::kStrips;
     const int tiles128 = tiles_n * ((M + 127) / 128);
-    static const int forced_bm = [] { const char* e = getenv("SLIMK_W2A8_TILED_BM"); return e ? atoi(e) : 0; }();
-    const bool small = forced_bm ? forced_bm == 64 : tiles128 < 2 * 256;
+    const bool small = tiles128 < 2 * 256;
     *bm = small ? 64 : 128;
     *tiles = small ? tiles_n * ((M + 63) / 64) : tiles128;
 }
