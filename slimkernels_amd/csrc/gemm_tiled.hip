@@ -329,21 +329,81 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
         }
         __syncthreads();
         if (lds[0][0] == 0) return;
+        // one split at a time, all of its fragments in flight together (one memory latency per split)
 #pragma unroll
         for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
-            for (int pp = 0; pp < 4; ++pp) {
-                v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-                for (int sp = 0; sp < n_split; ++sp)
-                    v += __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
-                             ws_rsrc, ws_lane + (mb * 4 + pp) * 1024, sp * ws_split_pitch + ws_tile, kCoherent));
+            for (int pp = 0; pp < 4; ++pp)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) t[mb][pp][j] = v[j];
-            }
+                for (int j = 0; j < 4; ++j) t[mb][pp][j] = 0.0f;
+        for (int sp = 0; sp < n_split; ++sp) {
+            v4f v[kMB][4];
+#pragma unroll
+            for (int mb = 0; mb < kMB; ++mb)
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp)
+                    v[mb][pp] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
+                        ws_rsrc, ws_lane + (mb * 4 + pp) * 1024, sp * ws_split_pitch + ws_tile, kCoherent));
+#pragma unroll
+            for (int mb = 0; mb < kMB; ++mb)
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) t[mb][pp][j] += v[mb][pp][j];
+        }
         if (tid == 0) __hip_atomic_store(p.ws_counter + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // ---- epilogue: out = cast(t * s_a[m])
+    // the token scales first, all loads in flight together (a load inside the store loop would not
+    // move above the stores before it and would cost one memory latency per row)
+    float sa_row[kMB][4];
+#pragma unroll
+    for (int mb = 0; mb < kMB; ++mb)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sa_row[mb][j] = p.s_a[min(m_tile + mb * 16 + quad * 4 + j, p.M - 1)];
+
+    if ((p.N & 7) == 0 && (p.ldo & 7) == 0) {
+        // Rows of 8 channels x 2 bytes = one 16-byte store per lane, eight lanes per 128-byte line of an
+        // output row.  The accumulator layout has a lane's values in different rows, so they turn
+        // through LDS: each wave owns a corner of the (now idle) stage buffers, writes 32 token rows
+        // x 64 channels of scaled fp32 sums (row pitch 68 floats: the four row groups of a write fall
+        // into different banks), and reads them back as 8 consecutive channels per lane.
+        // Every wave's LDS-direct loads must have landed and every wave must be out of the main
+        // loop before the buffers change their use.
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+        if (!strip_ok) return;
+        constexpr int kPitch = 68;
+        static_assert(32 * kPitch * 4 * kStrips <= (int)sizeof(lds), "output staging exceeds the stage buffers");
+        float* stage_out = reinterpret_cast<float*>(&lds[0][0]) + wave * (32 * kPitch);
+        typedef float v4f_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int rd = 0; rd < kMB / 2; ++rd) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        stage_out[(h * 16 + quad * 4 + j) * kPitch + pp * 16 + col] = t[rd * 2 + h][pp][j] * sa_row[rd * 2 + h][j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = i * 8 + (lane >> 3), cg = lane & 7;
+                const v4f_t lo = *reinterpret_cast<const v4f_t*>(stage_out + row * kPitch + cg * 8);
+                const v4f_t hi = *reinterpret_cast<const v4f_t*>(stage_out + row * kPitch + cg * 8 + 4);
+                v4u_t v;
+                v.x = (uint32_t)OutT::cast(lo.x) | ((uint32_t)OutT::cast(lo.y) << 16);
+                v.y = (uint32_t)OutT::cast(lo.z) | ((uint32_t)OutT::cast(lo.w) << 16);
+                v.z = (uint32_t)OutT::cast(hi.x) | ((uint32_t)OutT::cast(hi.y) << 16);
+                v.w = (uint32_t)OutT::cast(hi.z) | ((uint32_t)OutT::cast(hi.w) << 16);
+                const int m = m_tile + rd * 32 + row, n = strip * kStripN + cg * 8;
+                if (m < p.M && n < p.N) *reinterpret_cast<v4u_t*>(out + (size_t)m * p.ldo + n) = v;
+            }
+        }
+        return;
+    }
+
+    // any N and row pitch: one 2-byte store per value
     if (!strip_ok) return;
 #pragma unroll
     for (int mb = 0; mb < kMB; ++mb)
@@ -351,7 +411,7 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
         for (int j = 0; j < 4; ++j) {
             const int m = m_tile + mb * 16 + quad * 4 + j;
             if (m >= p.M) continue;
-            const float sa = p.s_a[m];
+            const float sa = sa_row[mb][j];
 #pragma unroll
             for (int pp = 0; pp < 4; ++pp) {
                 const int n = strip * kStripN + pp * 16 + col;
@@ -393,18 +453,19 @@ int tiled_fast_max_split(int M, int strips, int steps) {
     return steps / fast::kStageSteps;
 }
 
-// With fewer 64-row tiles than CUs and a long reduction, K is split over up to four workgroups per
-// tile so that about two workgroups per CU exist.  Measured: a lone workgroup on a CU spends about a
-// microsecond per 128-element stage whatever it does, so splitting pays once a split still runs 28
-// stages or more (K >= 7168); below that the exchange of partial tiles costs more than it saves.
+// With at most half as many 64-row tiles as CUs, K is split over several workgroups per tile so that
+// about two workgroups per CU exist.  Measured: a workgroup alone on a CU spends about 0.7 us per
+// 128-element stage and two on a CU about 1.25 us for both; a split costs the reducing workgroup
+// about a microsecond plus 0.8 us per partial tile it reads.  Hence up to eight splits, each at
+// least eight stages (K >= 1024 per split) long; with more tiles than that a split gains nothing.
 int tiled_fast_auto_split(int M, int strips, int steps) {
     int bm, tiles;
     tiled_fast_tiles(M, strips, &bm, &tiles);
-    if (bm != 64 || steps % fast::kStageSteps != 0 || tiles >= 256) return 1;
+    if (bm != 64 || steps % fast::kStageSteps != 0 || tiles > 128) return 1;
     const int stages = steps / fast::kStageSteps;
-    int split = (512 + tiles - 1) / tiles;
-    if (split > 4) split = 4;
-    if (split > stages / 28) split = stages / 28;
+    int split = 512 / tiles;
+    if (split > 8) split = 8;
+    if (split > stages / 8) split = stages / 8;
     if (split < 1) split = 1;
     const int sps = (stages + split - 1) / split;
     return (stages + sps - 1) / sps;
