@@ -297,6 +297,7 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
     w2a8::GroupedParams gp{};
     gp.count = count;
     int zm = -1, wgs = 0;
+    long long xcd_load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     // A workgroup of eight waves covers 8 strips x all of K, 4 strips x 2 halves or 2 strips x 4 quarters
     // (measured on the Llama-8B decode shapes: runs of 32..64 steps per wave stream best).
     const auto kparts_of = [](int steps) { return steps > 192 ? 4 : (steps > 32 ? 2 : 1); };
@@ -329,7 +330,23 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
         // units (sets of 8, 4 or 2 strips) in whole sets of eight, times the row blocks of 16 tokens
         const int per_unit = w2a8::kGroupedWavesPerWg / gp.kparts[i];
         const int units = (g.strips + per_unit - 1) / per_unit;
-        wgs += (units + 7) / 8 * 8 * ((pr.M + 15) / 16);
+        const int mblocks = (pr.M + 15) / 16;
+        wgs += (units + 7) / 8 * 8 * mblocks;
+        // The workgroup with id % 8 == x runs on XCD x.  The units of the last, partial set go to the
+        // XCDs that have the least work so far (work = steps a workgroup streams).
+        int by_load[8];
+        for (int x = 0; x < 8; ++x) by_load[x] = x;
+        for (int a = 1; a < 8; ++a)
+            for (int b = a; b > 0 && xcd_load[by_load[b]] < xcd_load[by_load[b - 1]]; --b) {
+                const int t = by_load[b]; by_load[b] = by_load[b - 1]; by_load[b - 1] = t;
+            }
+        uint32_t slots = 0;
+        const long long unit_work = (long long)mblocks * (g.steps / gp.kparts[i] + 16);
+        for (int slot = 0; slot < 8; ++slot) {
+            slots |= (uint32_t)slot << (3 * by_load[slot]);
+            if (slot < units % 8) xcd_load[by_load[slot]] += unit_work;
+        }
+        gp.xcd_slots[i] = slots;
     }
     gp.wg_begin[count] = wgs;
     return hip_result(w2a8::launch_skinny_grouped(gp, group_size / w2a8::kStepK, zm == 1, out_dtype == SLIMK_BF16,

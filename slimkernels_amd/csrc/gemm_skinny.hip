@@ -687,7 +687,9 @@ __device__ __forceinline__ void shared_body(const GemmParams& p, const int unit,
 // Workgroup ids are cut into runs, one run per problem.  Within a problem, workgroups come in sets
 // of eight per 16-row token block: consecutive workgroup ids go to different XCDs, so the two row
 // blocks of a set of strips, eight ids apart, share an XCD and its L2 (the second read of the
-// weights hits there).  All problems share the group size, the zero-point mode and the output
+// weights hits there).  Which unit of a set an XCD takes is the host's choice per problem
+// (xcd_slots): the last, partial set of every problem leaves some XCDs without work, and the host
+// deals those gaps out evenly, because an XCD's 32 CUs can only stream so much.  All problems share the group size, the zero-point mode and the output
 // type.  The problem table travels in the kernel arguments.
 template <int GS, bool ASYM, typename OutT>
 __global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_grouped_kernel(const GroupedParams gp) {
@@ -703,7 +705,7 @@ __global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_grouped_kernel(c
     const int local = wg - gp.wg_begin[i];
     const int mblocks = (p.M + 15) >> 4;
     const int mblk = (local >> 3) % mblocks;
-    const int unit = (local / (8 * mblocks)) * 8 + (local & 7);  // set of strips
+    const int unit = (local / (8 * mblocks)) * 8 + (int)((gp.xcd_slots[i] >> (3 * (local & 7))) & 7u);  // set of strips
     const int nk = gp.kparts[i];
     if (unit * (kGroupedWaves / nk) >= p.strips) return;  // padding workgroup (uniform)
     // activations go through LDS once a fragment spans enough cache lines to be worth a barrier
