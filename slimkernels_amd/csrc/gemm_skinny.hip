@@ -40,12 +40,13 @@ struct SkinnyMeta {
     int32_t rowsum[kDepth][16];
 };
 
-template <int NWP>
+template <int NWP, bool WIDE>
 struct SkinnySmem {
     union {
         SkinnyMeta meta[NWP];
         float red[NWP][16][kStripN + 1];
     };
+    v4u atile[WIDE ? NWP : 1][kDepth][64];  // WIDE: a wave's activation fragments of one chunk, in MFMA operand order
     int last;
 };
 
@@ -59,6 +60,9 @@ struct SkinnySmem {
 //         stores its results itself; NWP: all the workgroup's waves, meeting in LDS)
 //   ASYM  per-(group, channel) zero-points from zp_r instead of the uniform zp_const
 //   DUMP  verification build: exact int32 group sums are written out
+//   WIDE  activations are fetched two steps wide (whole 128-byte lines of the row-major tokens: half
+//         the cache lines of a step-by-step fetch once there are eight rows or more) and turned into
+//         MFMA operand order through a wave-private LDS tile; no barrier, the wave only meets itself
 //
 // Zero-points.  The MFMA operand of field p is code * 4^p (p < 3) or 64 * (code - 2) (p = 3), so
 // a group's true sum is raw - zpe * rowsum with zpe = zp * 4^p resp. (zp - 2) * 64.  The timed
@@ -66,9 +70,10 @@ struct SkinnySmem {
 // product over the groups (16 tokens x 16 channels x up to 4 groups of a chunk) and goes through
 // one v_mfma_f32_16x16x4_f32 per chunk and sub-block, accumulating straight into the fp32 running
 // sums (same D layout as the int8 MFMA).  The verification build folds it in integers instead.
-template <int J, int GS, int NWK, int NWP, bool ASYM, bool DUMP, bool NT, typename OutT>
+template <int J, int GS, int NWK, int NWP, bool ASYM, bool DUMP, bool NT, bool WIDE, typename OutT>
 __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip, const int split, const int mblk,
-                                            const int kwave, const int pwave, SkinnySmem<NWP>& sm) {
+                                            const int kwave, const int pwave, SkinnySmem<NWP, WIDE>& sm) {
+    static_assert(!(WIDE && DUMP), "the verification build fetches step by step");
     constexpr int MB = 1;
     static_assert(NWK == 1 || NWK == NWP, "K is split over one wave or over the whole workgroup");
     constexpr int kThreads = NWP * 64;
@@ -168,9 +173,32 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     v4u aring[kDepth][MB];
     auto issue = [&](int slot, int step) {  // step is wave-uniform
         wring[slot] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane, step * wstride + wbase, NT ? kStreamOnce : 0);
+        if (!WIDE) {
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-            aring[slot][mb] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, aoff[mb], step * kStepK, 0);
+            for (int mb = 0; mb < MB; ++mb)
+                aring[slot][mb] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, aoff[mb], step * kStepK, 0);
+        }
+    };
+    // WIDE: fragment (pair q, row half h) of a chunk: lane l reads row 8h + l/8, 16-byte piece l%8 of the
+    // 128 bytes the pair's two steps cover, and parks it at step 2q + piece/4, lane (piece%4)*16 + row.
+    // (A pair that starts on the range's last step reads 64 bytes past it: the bytes of the next
+    // step or, past K, zeros or the next row; that step carries a zero scale.)
+    v4u awide[kDepth];
+    const uint32_t wpiece = lane & 7;
+    const int wrow[2] = {lane >> 3, 8 + (lane >> 3)};
+    auto fetch_wide = [&](int it) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                awide[2 * q + h] = __builtin_amdgcn_raw_buffer_load_b128(
+                    q_rsrc, (uint32_t)min(wrow[h], M - 1) * (uint32_t)p.ldq + wpiece * 16, stepof(it + 2 * q) * kStepK, 0);
+    };
+    auto park_wide = [&]() {
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) sm.atile[WIDE ? pwave : 0][2 * q + (wpiece >> 2)][(wpiece & 3) * 16 + wrow[h]] = awide[2 * q + h];
     };
 
     // running sums, in units of 4^p (sub-block p < 3) resp. 64 (p = 3) times the result
@@ -191,6 +219,7 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < kDepth; ++i) issue(i, stepof(i));
+        if (WIDE) fetch_wide(0);
         __builtin_amdgcn_sched_barrier(0);
 
         v4i acc[MB][4];
@@ -230,6 +259,14 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
                         if (ASYM || pp < 3 || p.zp_const != 2)  // uniform zero-point 2: field 3 is already centred
                             t[mb][pp] = __builtin_amdgcn_mfma_f32_16x16x4f32(rsf, zb[pp], t[mb][pp], 0, 0, 0);
                 }
+            }
+
+            if (WIDE) {
+                park_wide();                  // this chunk's fragments: registers -> LDS tile
+                fetch_wide(it + kDepth);      // next chunk's: global -> registers
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < kDepth; ++i) aring[i][0] = sm.atile[WIDE ? pwave : 0][i][lane];
             }
 
 #pragma unroll
@@ -384,11 +421,11 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     if (tid == 0) __hip_atomic_store(p.ws_counter + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int J, int GS, int NW, bool ASYM, bool DUMP, bool NT, typename OutT>
+template <int J, int GS, int NW, bool ASYM, bool DUMP, bool NT, bool WIDE, typename OutT>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const GemmParams p) {
-    __shared__ __attribute__((aligned(16))) SkinnySmem<NW> sm;
+    __shared__ __attribute__((aligned(16))) SkinnySmem<NW, WIDE> sm;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keeps ranges and bases in SGPRs
-    skinny_body<J, GS, NW, NW, ASYM, DUMP, NT, OutT>(p, blockIdx.x, blockIdx.y, blockIdx.z, wave, wave, sm);
+    skinny_body<J, GS, NW, NW, ASYM, DUMP, NT, WIDE, OutT>(p, blockIdx.x, blockIdx.y, blockIdx.z, wave, wave, sm);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -728,32 +765,41 @@ __global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_grouped_kernel(c
     }
 }
 
-template <int J, int GS, int NW, bool ASYM, bool DUMP, bool NT>
+template <int J, int GS, int NW, bool ASYM, bool DUMP, bool NT, bool WIDE>
 static void launch_out(const GemmParams& p, bool out_bf16, hipStream_t stream) {
     const dim3 grid(p.strips, p.split, (p.M + 15) / 16), block(NW * 64);
     if (out_bf16)
-        skinny_kernel<J, GS, NW, ASYM, DUMP, NT, OutBF16><<<grid, block, 0, stream>>>(p);
+        skinny_kernel<J, GS, NW, ASYM, DUMP, NT, WIDE, OutBF16><<<grid, block, 0, stream>>>(p);
     else
-        skinny_kernel<J, GS, NW, ASYM, DUMP, NT, OutF16><<<grid, block, 0, stream>>>(p);
+        skinny_kernel<J, GS, NW, ASYM, DUMP, NT, WIDE, OutF16><<<grid, block, 0, stream>>>(p);
 }
 
-template <int J, int GS, int NW, bool DUMP, bool NT>
+template <int J, int GS, int NW, bool DUMP, bool NT, bool WIDE>
 static void launch_zm(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
-    if (asym) launch_out<J, GS, NW, true, DUMP, NT>(p, out_bf16, stream);
-    else launch_out<J, GS, NW, false, DUMP, NT>(p, out_bf16, stream);
+    if (asym) launch_out<J, GS, NW, true, DUMP, NT, WIDE>(p, out_bf16, stream);
+    else launch_out<J, GS, NW, false, DUMP, NT, WIDE>(p, out_bf16, stream);
 }
+
+// Two-steps-wide activation fetch pays from 16 token rows on when the reduction is long (measured:
+// 5..15 % faster at K >= 8192, M = 16..32; the LDS turn costs a short problem more than the saved
+// cache-line slots bring).
+constexpr int kWideRows = 16, kWideK = 8192;
 
 template <int GS, int NW>
 static void launch_rows(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
-    if (p.M == 1) launch_zm<1, GS, NW, false, true>(p, asym, out_bf16, stream);
-    else if (p.M <= 16) launch_zm<4, GS, NW, false, true>(p, asym, out_bf16, stream);
-    else launch_zm<4, GS, NW, false, false>(p, asym, out_bf16, stream);  // two row blocks share the weights in L2
+    const bool wide = p.M >= kWideRows && p.K >= kWideK;
+    if (p.M == 1) launch_zm<1, GS, NW, false, true, false>(p, asym, out_bf16, stream);
+    else if (p.M <= 16 && !wide) launch_zm<4, GS, NW, false, true, false>(p, asym, out_bf16, stream);
+    else if (p.M <= 16) launch_zm<4, GS, NW, false, true, true>(p, asym, out_bf16, stream);
+    // two row blocks share the weights in L2
+    else if (!wide) launch_zm<4, GS, NW, false, false, false>(p, asym, out_bf16, stream);
+    else launch_zm<4, GS, NW, false, false, true>(p, asym, out_bf16, stream);
 }
 
 template <int GS>
 static void launch_nw(const GemmParams& p, int waves, bool asym, bool out_bf16, hipStream_t stream) {
     const bool dump = p.acc_dump != nullptr && p.dump_mode != 0;
-    if (dump) launch_zm<4, GS, 4, true, false>(p, asym, out_bf16, stream);  // verification: 4 waves, all rows
+    if (dump) launch_zm<4, GS, 4, true, false, false>(p, asym, out_bf16, stream);  // verification: 4 waves, all rows
     else if (waves >= 16) launch_rows<GS, 16>(p, asym, out_bf16, stream);
     else launch_rows<GS, 4>(p, asym, out_bf16, stream);
 }

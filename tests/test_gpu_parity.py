@@ -109,6 +109,21 @@ def test_skinny_small(gpu_ops, oracle, M, N, K, g, mode, out):
         _run_case(gpu_ops, oracle, case, "skinny", split_k=2)
 
 
+@pytest.mark.parametrize("M,N,K,g,mode,out,split", [
+    (16, 64, 8192, 128, "sym", "float16", 1),
+    (16, 130, 8256, 64, "asym", "bfloat16", 1),   # 129 steps: the last pair of steps is half past the end
+    (29, 70, 8320, 64, "sym", "float16", 1),      # two row blocks, the second ragged
+    (32, 64, 9216, 256, "asym", "float16", 2),
+    (20, 128, 8192, 128, "sym", "bfloat16", 3),
+])
+def test_skinny_wide_activation_fetch(gpu_ops, oracle, M, N, K, g, mode, out, split):
+    """From 16 token rows and K >= 8192 on the skinny kernel fetches activations two steps wide and
+    turns them through LDS: same results as the step-by-step fetch (int32 sums exact)."""
+    case = pu.small_case(M, N, K, g, mode, seed=M + K, out_dtype=out)
+    _run_case(gpu_ops, oracle, case, "skinny", split_k=split)
+    _run_case(gpu_ops, oracle, case, "skinny", split_k=0, dump="sum")
+
+
 @pytest.mark.parametrize("M,N,K,g,mode,out", SMALL + [
     (77, 200, 512, 128, "asym", "float16"),
     (129, 130, 320, 64, "sym", "float16"),
