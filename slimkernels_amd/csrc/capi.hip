@@ -301,6 +301,31 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
     // A workgroup of eight waves covers 8 strips x all of K, 4 strips x 2 halves or 2 strips x 4 quarters
     // (measured on the Llama-8B decode shapes: runs of 32..64 steps per wave stream best).
     const auto kparts_of = [](int steps) { return steps > 192 ? 4 : (steps > 32 ? 2 : 1); };
+    // K-parts per problem.  A launch that would not even put one workgroup on every CU is bound by
+    // latency, not bandwidth: there the problem whose waves run longest is split further (down to runs
+    // of four chunks) until the CUs are covered.
+    int kparts[SLIMK_W2A8_MAX_GROUP];
+    {
+        const auto wgs_of = [&](int i, int parts) {
+            const int per_unit = w2a8::kGroupedWavesPerWg / parts;
+            return (strips_of(problems[i].N) + per_unit - 1) / per_unit * ((problems[i].M + 15) / 16);
+        };
+        int total = 0;
+        for (int i = 0; i < count; ++i) {
+            kparts[i] = problems[i].K >= 64 ? kparts_of(problems[i].K / w2a8::kStepK) : 1;
+            total += problems[i].N > 0 && problems[i].M > 0 ? wgs_of(i, kparts[i]) : 0;
+        }
+        while (total < 256) {
+            int pick = -1, run = 0;
+            for (int i = 0; i < count; ++i) {
+                const int r = (problems[i].K / w2a8::kStepK + 3) / 4 / kparts[i];  // chunks per part
+                if (kparts[i] < 8 && r >= 8 && r > run && problems[i].N > 0 && problems[i].M > 0) { pick = i; run = r; }
+            }
+            if (pick < 0) break;
+            total += wgs_of(pick, kparts[pick] * 2) - wgs_of(pick, kparts[pick]);
+            kparts[pick] *= 2;
+        }
+    }
     for (int i = 0; i < count; ++i) {
         const slimk_w2a8_problem& pr = problems[order[i]];
         if (!pr.q || !pr.s_a || !pr.rowsum || !pr.w_r || !pr.s_r || !pr.out)
@@ -326,7 +351,7 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
         g.strips = strips_of(pr.N); g.zp_const = pr.zp_const;
         g.split = 1; g.groups_per_split = groups_per_split(g.G, group_size, 1);
         gp.wg_begin[i] = wgs;
-        gp.kparts[i] = kparts_of(g.steps);
+        gp.kparts[i] = kparts[order[i]];
         // units (sets of 8, 4 or 2 strips) in whole sets of eight, times the row blocks of 16 tokens
         const int per_unit = w2a8::kGroupedWavesPerWg / gp.kparts[i];
         const int units = (g.strips + per_unit - 1) / per_unit;

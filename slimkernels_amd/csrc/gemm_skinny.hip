@@ -757,11 +757,15 @@ __global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_grouped_kernel(c
         else if (mrows < kShareRows) shared_body<4, GS, 2, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
         else if (mblocks == 1) shared_body<4, GS, 2, true, ASYM, true, OutT>(p, unit, mblk, wave, sm);
         else shared_body<4, GS, 2, true, ASYM, false, OutT>(p, unit, mblk, wave, sm);
-    } else {
+    } else if (nk == 4) {
         if (p.M == 1) shared_body<1, GS, 4, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
         else if (mrows < kShareRows) shared_body<4, GS, 4, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
         else if (mblocks == 1) shared_body<4, GS, 4, true, ASYM, true, OutT>(p, unit, mblk, wave, sm);
         else shared_body<4, GS, 4, true, ASYM, false, OutT>(p, unit, mblk, wave, sm);
+    } else {  // eight k-parts of one strip (small launches of long reductions): nobody to share activations with
+        if (p.M == 1) shared_body<1, GS, 8, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
+        else if (mblocks == 1) shared_body<4, GS, 8, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
+        else shared_body<4, GS, 8, false, ASYM, false, OutT>(p, unit, mblk, wave, sm);
     }
 }
 

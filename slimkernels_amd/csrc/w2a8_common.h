@@ -66,7 +66,7 @@ constexpr int kMaxGroup = 24;
 struct GroupedParams {
     GemmParams prob[kMaxGroup];
     int wg_begin[kMaxGroup + 1];  // problem i owns workgroups wg_begin[i] .. wg_begin[i+1]-1
-    int kparts[kMaxGroup];  // 1, 2 or 4: parts K is split into inside a workgroup of eight waves (8, 4 or 2 strips)
+    int kparts[kMaxGroup];  // 1, 2, 4 or 8: parts K is split into inside a workgroup of eight waves (8, 4, 2 or 1 strips)
     uint32_t xcd_slots[kMaxGroup];  // 3 bits per XCD x: which unit of a set of eight the workgroup with id % 8 == x takes
     int count;
 };
