@@ -173,7 +173,9 @@ typedef struct slimk_w2a8_problem {
  * kernel arguments (so the call is graph-capturable and the array may be reused at once).
  * All problems share group_size and out_dtype, and either all carry per-group zero-points
  * (zp_r non-NULL) or none does (each then uses its own zp_const); M, N, K may differ.
- * No split-K, no workspace.  For a single problem slimk_w2a8_gemm is the faster call.
+ * No split-K, no workspace.  A launch too small to cover the chip splits its longest reductions
+ * further inside the workgroups; a lone problem that slimk_w2a8_gemm would run unsplit is handed
+ * to that kernel (faster for one problem).
  * No upstream counterpart. */
 int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int group_size, int out_dtype,
                             void* stream);

@@ -374,6 +374,14 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
         gp.xcd_slots[i] = slots;
     }
     gp.wg_begin[count] = wgs;
+    // A single problem that the one-problem kernel runs unsplit is faster there (measured 5 us
+    // against 7.6 us at 4096 x 4096, M = 1: one strip per workgroup puts more waves on the chip).
+    if (count == 1 && auto_split(problems[0].M, problems[0].N, problems[0].K, group_size, SLIMK_KERNEL_SKINNY) == 1) {
+        const slimk_w2a8_problem& pr = problems[0];
+        return slimk_w2a8_gemm(pr.q, pr.ldq, pr.s_a, pr.rowsum, pr.ldr, pr.w_r, pr.s_r, pr.zp_r, pr.zp_const, pr.M, pr.N, pr.K,
+                               group_size, pr.out, pr.ldo, out_dtype, nullptr, SLIMK_DUMP_NONE, nullptr, 0,
+                               SLIMK_KERNEL_SKINNY, 1, stream);
+    }
     return hip_result(w2a8::launch_skinny_grouped(gp, group_size / w2a8::kStepK, zm == 1, out_dtype == SLIMK_BF16,
                                                   (hipStream_t)stream),
                       "grouped skinny gemm");
