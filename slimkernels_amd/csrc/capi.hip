@@ -80,6 +80,28 @@ int groups_per_split(int G, int group_size, int split) {
     return (gps + cg - 1) / cg * cg;
 }
 
+// One problem with 17..32 token rows on a matrix big enough to be bound by bandwidth goes through
+// the shared-activation workgroups (eight waves = two k-parts x four strips whose waves fetch the
+// activations once): 8..27 % faster there than one strip per workgroup (at 16 rows and below the
+// one-strip kernel is as fast or faster).  K is split across workgroups until about 256 exist, as
+// long as a wave keeps at least six chunks of four steps.
+constexpr size_t kSharedMinWeightBytes = (size_t)24 << 20;
+constexpr int kSharedParts = w2a8::kSharedParts;
+bool skinny_shared_applies(int M, int N, int K) {
+    return M > 16 && M <= 32 && (size_t)strips_of(N) * 64 * (K / 4) >= kSharedMinWeightBytes;
+}
+int skinny_shared_split(int M, int N, int K, int group_size) {
+    const int per_unit = w2a8::kGroupedWavesPerWg / kSharedParts;
+    const int units = (strips_of(N) + per_unit - 1) / per_unit * ((M + 15) / 16);
+    const int chunks = (K / 64 + 3) / 4;
+    int split = (256 + units / 2) / units;
+    if (split > chunks / (kSharedParts * 6)) split = chunks / (kSharedParts * 6);
+    if (split < 1) split = 1;
+    const int G = K / group_size;
+    const int gps = groups_per_split(G, group_size, split);
+    return (G + gps - 1) / gps;
+}
+
 // Split-K heuristic of the skinny kernel (measured on MI355X, cold weights).  One workgroup per
 // 64-channel strip already covers the chip when there are >= 192 strips, and a matrix of a few
 // MiB is latency-bound whatever is done, so both run unsplit: the cross-workgroup reduction
@@ -91,6 +113,7 @@ int auto_split(int M, int N, int K, int group_size, int kernel) {
         if (group_size > 128) return 1;
         return w2a8::tiled_fast_auto_split(M, strips_of(N), K / w2a8::kStepK);
     }
+    if (skinny_shared_applies(M, N, K)) return skinny_shared_split(M, N, K, group_size);
     const int strips = strips_of(N);
     const int G = K / group_size;
     const int chunks = (K / 64 + 3) / 4;
@@ -273,6 +296,8 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
     const int gs = group_size / w2a8::kStepK;
     const bool asym = zp_r != nullptr;
     const bool out_bf16 = out_dtype == SLIMK_BF16;
+    if (kern == SLIMK_KERNEL_SKINNY && p.acc_dump == nullptr && skinny_shared_applies(M, N, K))
+        return hip_result(w2a8::launch_skinny_shared(p, gs, asym, out_bf16, st), "shared skinny gemm");
     if (kern == SLIMK_KERNEL_SKINNY)
         return hip_result(w2a8::launch_skinny(p, gs, skinny_waves(M, split_k), asym, out_bf16, st), "skinny gemm");
     return hip_result(w2a8::launch_tiled(p, gs, asym, out_bf16, st), "tiled gemm");

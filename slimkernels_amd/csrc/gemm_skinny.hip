@@ -465,11 +465,15 @@ struct GroupedSmem {
         float red[kGroupedWaves][16][kStripN + 1];
     };
     v4u abuf[4][2][kDepth][64];  // [k-part][parity][step of the chunk][lane]
+    int last;                    // split-K: this workgroup was the last of its unit to arrive
 };
 
-template <int J, int GS, int NK, bool SHARE, bool ASYM, bool NT, typename OutT>
+// SPLIT: the workgroup owns only the steps of K-split `split` (one-problem launches: grid.y splits,
+// partial tiles meet in the caller's workspace, the last workgroup of a unit to arrive adds them
+// up in split order and stores).
+template <int J, int GS, int NK, bool SHARE, bool ASYM, bool NT, bool SPLIT, typename OutT>
 __device__ __forceinline__ void shared_body(const GemmParams& p, const int unit, const int mblk, const int wave,
-                                            GroupedSmem& sm) {
+                                            GroupedSmem& sm, const int split = 0) {
     constexpr int NS = kGroupedWaves / NK;               // waves (strips) sharing one activation stream
     constexpr int NL = NS >= kDepth ? 1 : kDepth / NS;   // A fragments a loading wave fetches per chunk
     constexpr int kThreads = kGroupedWaves * 64;
@@ -497,8 +501,8 @@ __device__ __forceinline__ void shared_body(const GemmParams& p, const int unit,
     uint16_t* const out = reinterpret_cast<uint16_t*>(p.out) + (size_t)m0 * p.ldo;
 
     // token scales for the epilogue, fetched first
-    float sa[NK == 1 ? J : kOutPerThread];
-    if (NK == 1) {
+    float sa[NK == 1 && !SPLIT ? J : kOutPerThread];
+    if (NK == 1 && !SPLIT) {
 #pragma unroll
         for (int j = 0; j < J; ++j) sa[j] = sap[min(quad * 4 + j, M - 1)];
     } else {
@@ -508,10 +512,12 @@ __device__ __forceinline__ void shared_body(const GemmParams& p, const int unit,
 
     // K range of this k-part in whole chunks; every part runs the same number of chunk iterations
     // (the barrier count must agree), a shorter last part idles through the extra ones with zero scales.
-    const int chunks = (p.steps + kDepth - 1) / kDepth;
+    const int wg_s0 = SPLIT ? min(split * p.groups_per_split, p.G) * GS : 0;
+    const int wg_s1 = SPLIT ? min((split + 1) * p.groups_per_split, p.G) * GS : p.steps;
+    const int chunks = (wg_s1 - wg_s0 + kDepth - 1) / kDepth;
     const int per_part = (chunks + NK - 1) / NK;
-    const int s0 = min(kpart * per_part * kDepth, p.steps);
-    const int s1 = min(s0 + per_part * kDepth, p.steps);
+    const int s0 = min(wg_s0 + kpart * per_part * kDepth, wg_s1);
+    const int s1 = min(s0 + per_part * kDepth, wg_s1);
     const int g0 = s0 / GS, g1 = s1 / GS;
     const int len = s1 - s0;
     auto stepof = [&](int it) { return s0 + max(min(it, len - 1), 0); };
@@ -683,7 +689,7 @@ __device__ __forceinline__ void shared_body(const GemmParams& p, const int unit,
     }
 
     constexpr float kUnscale[4] = {1.0f, 0.25f, 0.0625f, 0.015625f};  // 4^-p, exact
-    if (NK == 1) {
+    if (NK == 1 && !SPLIT) {
         if (active) {
 #pragma unroll
             for (int pp = 0; pp < 4; ++pp)
@@ -705,20 +711,84 @@ __device__ __forceinline__ void shared_body(const GemmParams& p, const int unit,
         for (int j = 0; j < J; ++j)
             if (J > 1 || quad == 0) sm.red[wave][quad * 4 + j][pp * 16 + col] = t[pp][j] * kUnscale[pp];
     __syncthreads();
+    if (!SPLIT) {
+#pragma unroll
+        for (int i = 0; i < kOutPerThread; ++i) {
+            const int e = tid + kThreads * i;
+            const int sidx = e / kLive, w = e % kLive;
+            const int m = w >> 6, nl = w & 63;
+            const int so = unit * NS + sidx;
+            const int n = so * kStripN + nl;
+            if (sidx < NS && so < p.strips && m < M && n < p.N) {
+                float v = sm.red[sidx][m][nl];
+#pragma unroll
+                for (int kp = 1; kp < NK; ++kp) v += sm.red[kp * NS + sidx][m][nl];
+                out[(size_t)m * p.ldo + n] = OutT::cast(v * sa[i]);
+            }
+        }
+        return;
+    }
+
+    // ---- split-K: publish this workgroup's partial tiles (one 16 x 64 fp32 tile per strip and row
+    // block, the one-problem kernel's workspace layout), count arrivals per unit, the last one reduces
+    // in split order.  Partials move at system-coherent cache policy (write-through stores, loads
+    // around the reader's L2), a split's loads all in flight together.
+    constexpr int kCoherent = 17;  // sc0 | sc1
+    constexpr int kTile = 16 * kStripN;
+    const int mblocks = (p.M + 15) >> 4;
+    const int n_split = p.split;
+    const size_t tiles = (size_t)p.strips * mblocks;
+    const __amdgpu_buffer_rsrc_t ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        p.ws_partial, 0, (int)min((size_t)n_split * tiles * kTile * 4, (size_t)0x7fffffff), 0x00020000);
+    const uint32_t split_pitch = (uint32_t)(tiles * kTile * 4);
+    uint32_t eoff[kOutPerThread];
+    bool eon[kOutPerThread];
+#pragma unroll
+    for (int i = 0; i < kOutPerThread; ++i) {
+        const int e = tid + kThreads * i;
+        const int sidx = e / kLive, w = e % kLive;
+        const int so = unit * NS + sidx;
+        eon[i] = sidx < NS && so < p.strips;
+        eoff[i] = (uint32_t)(((size_t)min(so, p.strips - 1) * mblocks + mblk) * kTile + w) * 4;
+    }
+#pragma unroll
+    for (int i = 0; i < kOutPerThread; ++i) {
+        const int e = tid + kThreads * i;
+        const int sidx = min(e / kLive, NS - 1), w = e % kLive;
+        float v = sm.red[sidx][w >> 6][w & 63];
+#pragma unroll
+        for (int kp = 1; kp < NK; ++kp) v += sm.red[kp * NS + sidx][w >> 6][w & 63];
+        if (eon[i]) __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), ws_rsrc, eoff[i], split * split_pitch, kCoherent);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const int counter_id = (unit * NS) * mblocks + mblk;  // the unit's first strip stands for the unit
+    if (tid == 0) {
+        const unsigned prev = __hip_atomic_fetch_add(p.ws_counter + counter_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        sm.last = (prev == (unsigned)(n_split - 1));
+    }
+    __syncthreads();
+    if (!sm.last) return;
+    float v[kOutPerThread];
+#pragma unroll
+    for (int i = 0; i < kOutPerThread; ++i) v[i] = 0.0f;
+    for (int sp = 0; sp < n_split; ++sp) {
+        float part[kOutPerThread];
+#pragma unroll
+        for (int i = 0; i < kOutPerThread; ++i)
+            part[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ws_rsrc, eoff[i], sp * split_pitch, kCoherent));
+#pragma unroll
+        for (int i = 0; i < kOutPerThread; ++i) v[i] += part[i];
+    }
 #pragma unroll
     for (int i = 0; i < kOutPerThread; ++i) {
         const int e = tid + kThreads * i;
         const int sidx = e / kLive, w = e % kLive;
         const int m = w >> 6, nl = w & 63;
-        const int so = unit * NS + sidx;
-        const int n = so * kStripN + nl;
-        if (sidx < NS && so < p.strips && m < M && n < p.N) {
-            float v = sm.red[sidx][m][nl];
-#pragma unroll
-            for (int kp = 1; kp < NK; ++kp) v += sm.red[kp * NS + sidx][m][nl];
-            out[(size_t)m * p.ldo + n] = OutT::cast(v * sa[i]);
-        }
+        const int n = (unit * NS + sidx) * kStripN + nl;
+        if (eon[i] && m < M && n < p.N) out[(size_t)m * p.ldo + n] = OutT::cast(v[i] * sa[i]);
     }
+    if (tid == 0) __hip_atomic_store(p.ws_counter + counter_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Workgroup ids are cut into runs, one run per problem.  Within a problem, workgroups come in sets
@@ -748,25 +818,64 @@ __global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_grouped_kernel(c
     // activations go through LDS once a fragment spans enough cache lines to be worth a barrier
     const int mrows = min(16, p.M - mblk * 16);
     if (nk == 1) {
-        if (p.M == 1) shared_body<1, GS, 1, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
-        else if (mrows < kShareRows) shared_body<4, GS, 1, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
-        else if (mblocks == 1) shared_body<4, GS, 1, true, ASYM, true, OutT>(p, unit, mblk, wave, sm);
-        else shared_body<4, GS, 1, true, ASYM, false, OutT>(p, unit, mblk, wave, sm);
+        if (p.M == 1) shared_body<1, GS, 1, false, ASYM, true, false, OutT>(p, unit, mblk, wave, sm);
+        else if (mrows < kShareRows) shared_body<4, GS, 1, false, ASYM, true, false, OutT>(p, unit, mblk, wave, sm);
+        else if (mblocks == 1) shared_body<4, GS, 1, true, ASYM, true, false, OutT>(p, unit, mblk, wave, sm);
+        else shared_body<4, GS, 1, true, ASYM, false, false, OutT>(p, unit, mblk, wave, sm);
     } else if (nk == 2) {
-        if (p.M == 1) shared_body<1, GS, 2, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
-        else if (mrows < kShareRows) shared_body<4, GS, 2, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
-        else if (mblocks == 1) shared_body<4, GS, 2, true, ASYM, true, OutT>(p, unit, mblk, wave, sm);
-        else shared_body<4, GS, 2, true, ASYM, false, OutT>(p, unit, mblk, wave, sm);
+        if (p.M == 1) shared_body<1, GS, 2, false, ASYM, true, false, OutT>(p, unit, mblk, wave, sm);
+        else if (mrows < kShareRows) shared_body<4, GS, 2, false, ASYM, true, false, OutT>(p, unit, mblk, wave, sm);
+        else if (mblocks == 1) shared_body<4, GS, 2, true, ASYM, true, false, OutT>(p, unit, mblk, wave, sm);
+        else shared_body<4, GS, 2, true, ASYM, false, false, OutT>(p, unit, mblk, wave, sm);
     } else if (nk == 4) {
-        if (p.M == 1) shared_body<1, GS, 4, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
-        else if (mrows < kShareRows) shared_body<4, GS, 4, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
-        else if (mblocks == 1) shared_body<4, GS, 4, true, ASYM, true, OutT>(p, unit, mblk, wave, sm);
-        else shared_body<4, GS, 4, true, ASYM, false, OutT>(p, unit, mblk, wave, sm);
+        if (p.M == 1) shared_body<1, GS, 4, false, ASYM, true, false, OutT>(p, unit, mblk, wave, sm);
+        else if (mrows < kShareRows) shared_body<4, GS, 4, false, ASYM, true, false, OutT>(p, unit, mblk, wave, sm);
+        else if (mblocks == 1) shared_body<4, GS, 4, true, ASYM, true, false, OutT>(p, unit, mblk, wave, sm);
+        else shared_body<4, GS, 4, true, ASYM, false, false, OutT>(p, unit, mblk, wave, sm);
     } else {  // eight k-parts of one strip (small launches of long reductions): nobody to share activations with
-        if (p.M == 1) shared_body<1, GS, 8, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
-        else if (mblocks == 1) shared_body<4, GS, 8, false, ASYM, true, OutT>(p, unit, mblk, wave, sm);
-        else shared_body<4, GS, 8, false, ASYM, false, OutT>(p, unit, mblk, wave, sm);
+        if (p.M == 1) shared_body<1, GS, 8, false, ASYM, true, false, OutT>(p, unit, mblk, wave, sm);
+        else if (mblocks == 1) shared_body<4, GS, 8, false, ASYM, true, false, OutT>(p, unit, mblk, wave, sm);
+        else shared_body<4, GS, 8, false, ASYM, false, false, OutT>(p, unit, mblk, wave, sm);
     }
+}
+
+// One problem through the shared-activation body: grid.x = sets of strips (in whole sets of eight per
+// row block, as in the grouped kernel), grid.y = K splits.  For 17..32 token rows on matrices big
+// enough to be bound by bandwidth (measured 8..27 % faster than one strip per workgroup there; at
+// 16 rows and below the one-strip kernel is as fast or faster).
+template <int GS, int NK, bool ASYM, typename OutT>
+__global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_shared_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(16))) GroupedSmem sm;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int local = blockIdx.x;
+    const int mblocks = (p.M + 15) >> 4;
+    const int mblk = (local >> 3) % mblocks;
+    const int unit = (local / (8 * mblocks)) * 8 + (local & 7);
+    if (unit * (kGroupedWaves / NK) >= p.strips) return;  // padding workgroup (uniform)
+    // two row blocks (the host sends 17..32 token rows here): the second read of the weights comes from L2
+    if (p.split > 1) shared_body<4, GS, NK, true, ASYM, false, true, OutT>(p, unit, mblk, wave, sm, blockIdx.y);
+    else shared_body<4, GS, NK, true, ASYM, false, false, OutT>(p, unit, mblk, wave, sm);
+}
+
+template <int GS, int NK>
+static void launch_shared_nk(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
+    const int per_unit = kGroupedWaves / NK;
+    const int units = (p.strips + per_unit - 1) / per_unit;
+    const dim3 grid((units + 7) / 8 * 8 * ((p.M + 15) / 16), p.split > 1 ? p.split : 1), block(kGroupedWaves * 64);
+    if (asym) {
+        if (out_bf16) skinny_shared_kernel<GS, NK, true, OutBF16><<<grid, block, 0, stream>>>(p);
+        else skinny_shared_kernel<GS, NK, true, OutF16><<<grid, block, 0, stream>>>(p);
+    } else {
+        if (out_bf16) skinny_shared_kernel<GS, NK, false, OutBF16><<<grid, block, 0, stream>>>(p);
+        else skinny_shared_kernel<GS, NK, false, OutF16><<<grid, block, 0, stream>>>(p);
+    }
+}
+
+hipError_t launch_skinny_shared(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream) {
+    if (gs == 1) launch_shared_nk<1, kSharedParts>(p, asym, out_bf16, stream);
+    else if (gs == 2) launch_shared_nk<2, kSharedParts>(p, asym, out_bf16, stream);
+    else launch_shared_nk<4, kSharedParts>(p, asym, out_bf16, stream);
+    return hipGetLastError();
 }
 
 template <int J, int GS, int NW, bool ASYM, bool DUMP, bool NT, bool WIDE>

@@ -62,6 +62,7 @@ struct GemmParams {
 
 // Problem table of a grouped skinny launch; passed by value in the kernel arguments (< 4 KiB).
 constexpr int kGroupedWavesPerWg = 8;  // wavefronts per workgroup of the grouped skinny kernel
+constexpr int kSharedParts = 2;  // k-parts per workgroup when one problem runs through the shared-activation workgroups
 constexpr int kMaxGroup = 24;
 struct GroupedParams {
     GemmParams prob[kMaxGroup];

@@ -23,6 +23,10 @@ hipError_t launch_read_probe(const void* src, size_t bytes, uint32_t* sink, hipS
 // gs = 64-element steps per scale group (1, 2 or 4); waves = wavefronts per workgroup (4 or 16)
 hipError_t launch_skinny(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, hipStream_t stream);
 
+// one problem of 17..32 token rows through the shared-activation workgroups (kSharedParts k-parts x
+// 8 / kSharedParts strips per workgroup, p.split K splits across workgroups)
+hipError_t launch_skinny_shared(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
+
 // asym: every problem carries per-group zero-points (zp_r); otherwise each uses its uniform zp_const
 hipError_t launch_skinny_grouped(const GroupedParams& gp, int gs, bool asym, bool out_bf16, hipStream_t stream);
 
