@@ -382,11 +382,18 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     }
 
     // ---- split-K: publish this workgroup's partial tile, last arrival reduces all of them.
-    // The partials are written and read with agent-scope relaxed atomics (write-through stores,
-    // cache-bypassing loads on gfx950), so no L2 write-back / invalidate fence is needed: a fence
-    // here costs about a microsecond per workgroup and serialises on each XCD's L2.
-    // s_waitcnt vmcnt(0) makes every lane's stores complete before the arrival counter moves.
-    float* mine = p.ws_partial + ((size_t)split * p.strips * mblocks + tile_id) * kTile;
+    // The partials move at system-coherent cache policy (write-through stores, loads around the
+    // reader's L2), so no L2 write-back / invalidate fence is needed: a fence here costs about a
+    // microsecond per workgroup and serialises on each XCD's L2.  They are plain memory instructions,
+    // so the reduction keeps four splits' loads in flight at a time (one memory latency per four
+    // splits instead of one per split).  s_waitcnt vmcnt(0) makes every lane's stores complete
+    // before the arrival counter moves.
+    constexpr int kCoherent = 17;  // sc0 | sc1
+    const size_t tiles = (size_t)p.strips * mblocks;
+    const __amdgpu_buffer_rsrc_t ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        p.ws_partial, 0, (int)min((size_t)p.split * tiles * kTile * 4, (size_t)0x7fffffff), 0x00020000);
+    const uint32_t split_pitch = (uint32_t)(tiles * kTile * 4);
+    const uint32_t tile_off = (uint32_t)tile_id * (kTile * 4);
 #pragma unroll
     for (int i = 0; i < kOutPerThread; ++i) {
         const int e = tid + kThreads * i;
@@ -395,7 +402,7 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
             float v = sm.red[0][m][nl];
 #pragma unroll
             for (int w = 1; w < NWP; ++w) v += sm.red[w][m][nl];
-            __hip_atomic_store(mine + e, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), ws_rsrc, tile_off + e * 4, split * split_pitch, kCoherent);
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -413,9 +420,16 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
         const int m = e >> 6, nl = e & 63;
         const int n = strip * kStripN + nl;
         float v = 0.0f;
-        for (int sp = 0; sp < p.split; ++sp)
-            v += __hip_atomic_load(p.ws_partial + ((size_t)sp * p.strips * mblocks + tile_id) * kTile + e, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
+        for (int sp0 = 0; sp0 < p.split; sp0 += 4) {
+            float part[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)  // past the last split: the last one again, not added
+                part[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                              ws_rsrc, tile_off + e * 4, min(sp0 + u, p.split - 1) * split_pitch, kCoherent));
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (sp0 + u < p.split) v += part[u];
+        }
         if (m < M && n < p.N) out[(size_t)m * p.ldo + n] = OutT::cast(v * sa[i]);
     }
     if (tid == 0) __hip_atomic_store(p.ws_counter + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
