@@ -363,7 +363,7 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) sa_row[mb][j] = p.s_a[min(m_tile + mb * 16 + quad * 4 + j, p.M - 1)];
 
-    if ((p.N & 7) == 0 && (p.ldo & 7) == 0) {
+    if ((p.N & 7) == 0 && (p.ldo & 7) == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0) {
         // Rows of 8 channels x 2 bytes = one 16-byte store per lane, eight lanes per 128-byte line of an
         // output row.  The accumulator layout has a lane's values in different rows, so they turn
         // through LDS: each wave owns a corner of the (now idle) stage buffers, writes 32 token rows
@@ -403,7 +403,7 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
         return;
     }
 
-    // any N and row pitch: one 2-byte store per value
+    // any N, row pitch and alignment of out: one 2-byte store per value
     if (!strip_ok) return;
 #pragma unroll
     for (int mb = 0; mb < kMB; ++mb)

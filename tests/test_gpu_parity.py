@@ -156,6 +156,32 @@ def test_tiled_small(gpu_ops, oracle, M, N, K, g, mode, out):
     _run_case(gpu_ops, oracle, case, "tiled", split_k=0, dump="sum")
 
 
+@pytest.mark.parametrize("M,N,K,g,out", [(70, 256, 512, 128, "float16"), (130, 320, 768, 64, "bfloat16")])
+def test_tiled_output_views(gpu_ops, oracle, M, N, K, g, out):
+    """The tiled kernel stores 16 bytes per lane when N, the row pitch and the address of out allow
+    it and 2 bytes per value otherwise: a contiguous output, one that starts two bytes off a
+    16-byte boundary and one with an odd row pitch hold the same bits."""
+    _say("tiled output views", M, N, K, g, out)
+    case = pu.small_case(M, N, K, g, "sym", seed=M + N + K, out_dtype=out)
+    packed, scales, zero = pu.quantized_weight(case)
+    x = workloads.make_activation(case)
+    ref = oracle.reference_forward(x, packed, scales, zero, g, out_bf16=(out == "bfloat16"))
+    w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, x)
+    qa = gpu_ops.quantize_act_int8(xd, g)
+    odt = pu.torch_dtype(case)
+    plain = gpu_ops.w2a8_gemm(qa, w, odt, kernel="tiled", split_k=1)
+    wide = torch.zeros(M, N + 8, dtype=odt, device="cuda")
+    odd = torch.zeros(M, N + 3, dtype=odt, device="cuda")
+    shifted = gpu_ops.w2a8_gemm(qa, w, odt, kernel="tiled", split_k=1, out=wide[:, 1:1 + N])
+    pitched = gpu_ops.w2a8_gemm(qa, w, odt, kernel="tiled", split_k=1, out=odd[:, :N])
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(pu.out_tensor_bits(plain), ref["out_bits"])
+    np.testing.assert_array_equal(pu.out_tensor_bits(shifted.contiguous()), ref["out_bits"])
+    np.testing.assert_array_equal(pu.out_tensor_bits(pitched.contiguous()), ref["out_bits"])
+    assert float(wide[:, 0].abs().max()) == 0.0 and float(wide[:, 1 + N:].abs().max()) == 0.0
+    assert float(odd[:, N:].abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("M,N,K,g,out,split", [(64, 256, 2048, 128, "float16", 2), (77, 300, 4096, 64, "bfloat16", 4),
                                                  (130, 64, 3072, 128, "float16", 3), (40, 512, 8192, 128, "float16", 8)])
 def test_tiled_split_k(gpu_ops, oracle, M, N, K, g, out, split):
