@@ -350,6 +350,17 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
             total += wgs_of(pick, kparts[pick] * 2) - wgs_of(pick, kparts[pick]);
             kparts[pick] *= 2;
         }
+        // 512 workgroups run at once (two per CU); those beyond start as the first ones end, into a
+        // chip that is emptying.  The problems that start there (in launch order) get twice the
+        // k-parts: a second round of about twice the workgroups, each half as long.
+        int before = 0;
+        for (int oi = 0; oi < count; ++oi) {
+            const int i = order[oi];
+            if (problems[i].N <= 0 || problems[i].M <= 0) continue;
+            const int r = (problems[i].K / w2a8::kStepK + 3) / 4 / kparts[i];
+            if (before >= 512 && kparts[i] < 4 && r >= 8) kparts[i] *= 2;
+            before += wgs_of(i, kparts[i]);
+        }
     }
     for (int i = 0; i < count; ++i) {
         const slimk_w2a8_problem& pr = problems[order[i]];
