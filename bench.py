@@ -41,7 +41,7 @@ COLD_FOOTPRINT = 640 << 20    # bytes of distinct weight copies between two uses
 # `python3 bench.py --skip-detail` (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same
 # counter reads for this file's 256 MiB calibration read (read_probe_kernel: 131080 -> x2.0) and
 # calibration fill (fill_zero_kernel: 262144 -> x1.0):  (115515 * 2.0 + 2898 * 1.0) KiB.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = int((115494 * 2.0 + 2898 * 1.0) * 1024)
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = int((115929 * 2.0 + 2898 * 1.0) * 1024)
 
 
 def main():
