@@ -128,10 +128,14 @@ int auto_split(int M, int N, int K, int group_size, int kernel) {
 }
 
 // Wavefronts per workgroup of the skinny kernel (the in-workgroup split of K): split runs are the
-// long-K ones, more waves per workgroup keep more loads in flight per CU.
-int skinny_waves(int M, int split) {
-    (void)M;
-    return split > 1 ? 16 : 4;
+// long-K ones, more waves per workgroup keep more loads in flight per CU.  An unsplit matrix of
+// up to 16 MiB with at most four token rows is bound by latency: eight waves per strip instead of
+// four shorten each wave's run (measured 5.09 -> 4.72 us at 4096 x 4096, M = 1; larger matrices
+// and more rows lose).
+int skinny_waves(int M, int N, int K, int split) {
+    if (split > 1) return 16;
+    const size_t weight_bytes = (size_t)strips_of(N) * 64 * (K / 4);
+    return M <= 4 && weight_bytes <= ((size_t)16 << 20) && K >= 2048 ? 8 : 4;
 }
 
 }  // namespace
@@ -299,7 +303,7 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
     if (kern == SLIMK_KERNEL_SKINNY && p.acc_dump == nullptr && skinny_shared_applies(M, N, K))
         return hip_result(w2a8::launch_skinny_shared(p, gs, asym, out_bf16, st), "shared skinny gemm");
     if (kern == SLIMK_KERNEL_SKINNY)
-        return hip_result(w2a8::launch_skinny(p, gs, skinny_waves(M, split_k), asym, out_bf16, st), "skinny gemm");
+        return hip_result(w2a8::launch_skinny(p, gs, skinny_waves(M, N, K, split_k), asym, out_bf16, st), "skinny gemm");
     return hip_result(w2a8::launch_tiled(p, gs, asym, out_bf16, st), "tiled gemm");
 }
 

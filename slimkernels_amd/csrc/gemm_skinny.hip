@@ -928,6 +928,7 @@ static void launch_nw(const GemmParams& p, int waves, bool asym, bool out_bf16, 
     const bool dump = p.acc_dump != nullptr && p.dump_mode != 0;
     if (dump) launch_zm<4, GS, 4, true, false, false>(p, asym, out_bf16, stream);  // verification: 4 waves, all rows
     else if (waves >= 16) launch_rows<GS, 16>(p, asym, out_bf16, stream);
+    else if (waves >= 8) launch_rows<GS, 8>(p, asym, out_bf16, stream);
     else launch_rows<GS, 4>(p, asym, out_bf16, stream);
 }
 

@@ -20,7 +20,7 @@ hipError_t launch_fill_zero(void* p, size_t bytes, hipStream_t stream);
 
 hipError_t launch_read_probe(const void* src, size_t bytes, uint32_t* sink, hipStream_t stream);
 
-// gs = 64-element steps per scale group (1, 2 or 4); waves = wavefronts per workgroup (4 or 16)
+// gs = 64-element steps per scale group (1, 2 or 4); waves = wavefronts per workgroup (4, 8 or 16)
 hipError_t launch_skinny(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, hipStream_t stream);
 
 // one problem of 17..32 token rows through the shared-activation workgroups (kSharedParts k-parts x
