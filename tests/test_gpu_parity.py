@@ -280,9 +280,38 @@ def test_grouped_launch_matches_single_launches(gpu_ops, oracle):
     pu.assert_out_close(pu.out_tensor_bits(o), ref["out_bits"], True, pu.reorder_bound(ref["acc"], scales, ref["s_a"]), "grouped asym")
 
 
-# every shape class of the grouped kernel: k-parts 1 / 2 / 4 (by K), one-row / few-row / shared-activation
-# bodies (by M), two row blocks (M > 16), group sizes 64 / 128 / 256, per-group zero-points, a K range
-# whose last chunk is ragged, k-parts of unequal length
+def test_grouped_launch_that_fills_the_chip(gpu_ops, oracle):
+    """A launch of more than 512 workgroups keeps the default k-parts (1 / 2 / 4 by K: the shared-
+    activation bodies with 8, 4 and 2 strips per workgroup) for the problems of its first round and
+    doubles them for the problems that start later; a small launch raises them all.  Three weights,
+    each used by problems of several M, every output against the oracle."""
+    weights = {}
+    for name, (N, K) in {"a": (8192, 4096), "b": (8192, 2048), "c": (4096, 14336)}.items():
+        case = pu.small_case(1, N, K, 128, "sym", seed=900 + K)
+        packed, scales, zero = pu.quantized_weight(case)
+        w, _ = pu.device_inputs(gpu_ops, case, packed, scales, zero, workloads.make_activation(case))
+        weights[name] = (N, K, packed, scales, zero, w)
+    plan = [("c", 1), ("c", 16), ("c", 32)] + [("a", m) for m in (1, 3, 8, 16, 32, 2, 4, 12, 24)] + \
+           [("b", m) for m in (1, 3, 8, 16, 32)]
+    probs, refs = [], []
+    for i, (name, M) in enumerate(plan):
+        N, K, packed, scales, zero, w = weights[name]
+        case = pu.small_case(M, N, K, 128, "sym", seed=950 + i)
+        x = workloads.make_activation(case)
+        xd = torch.from_numpy(x).cuda()
+        probs.append((gpu_ops.quantize_act_int8(xd, 128), w))
+        refs.append((oracle.reference_forward(x, packed, scales, zero, 128), scales))
+    _say("grouped launch of", len(probs), "problems")
+    outs = gpu_ops.w2a8_gemm_grouped(probs)
+    torch.cuda.synchronize()
+    for (name, M), o, (ref, scales) in zip(plan, outs, refs):
+        pu.assert_out_close(pu.out_tensor_bits(o), ref["out_bits"], False,
+                            pu.reorder_bound(ref["acc"], scales, ref["s_a"]), f"grouped big launch {name} M={M}")
+
+
+# shape classes of the grouped kernel in small launches (k-parts raised to 4 / 8 where K allows): one-row /
+# few-row / shared-activation bodies (by M), two row blocks (M > 16), group sizes 64 / 128 / 256, per-group
+# zero-points, a K range whose last chunk is ragged, k-parts of unequal length
 GROUPED_SETS = [
     (128, "sym", [(1, 192, 8192), (9, 192, 8192), (32, 130, 14336), (4, 64, 14336), (16, 300, 4096), (17, 64, 4096)]),
     (64, "sym", [(1, 128, 8192), (12, 128, 2368), (32, 100, 6208)]),
