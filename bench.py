@@ -299,6 +299,44 @@ def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, d
             pre.append({"shape": f"{N}x{K}", "M": M, "us": round(us, 1), "TOPS": round(tops, 1),
                         "frac_int8_mfma": round(tops / INT8_PEAK_TOPS, 4)})
     detail["prefill"] = pre
+
+    # ---- the other configurations (c4: Llama-70B-class linears, group 64, bf16 out; c5: ragged shapes
+    # with per-group zero-points), timing only, on random codes and scales in the streaming layout
+    # (their parity is what the GPU tests check on quantised data).  M <= 16 cold (five weight copies
+    # in rotation, more than the 256 MiB last-level cache), larger M warm.
+    def random_weight(N, K, g, asym):
+        strips = -(-N // 64)
+        w_r = torch.randint(-2**31, 2**31 - 1, (strips * (K // 64) * 256,), dtype=torch.int32, device=dev)
+        s_r = (torch.rand(strips * (K // g) * 64, device=dev) * 0.02 + 0.005).half()
+        zp_r = torch.randint(0, 4, (strips * (K // g) * 64,), dtype=torch.uint8, device=dev) if asym else None
+        return ops.W2A8Weight(w_r, s_r, zp_r, 0 if asym else 2, N, K, g)
+
+    others = []
+    plan = [("c4", N, K, 64, "sym", torch.bfloat16, M) for (N, K) in ((28672, 8192), (8192, 28672)) for M in (1, 16, 128, 2048)]
+    plan += [("c5", 11008, 4096, 128, "asym", torch.float16, 77), ("c5", 5120, 13824, 128, "asym", torch.float16, 1)]
+    cache = {}
+    for (cfg, N, K, g, mode, odt, M) in plan:
+        cold = M <= 16
+        key = (N, K, g, mode)
+        if key not in cache:
+            cache.clear()
+            torch.cuda.empty_cache()
+            cache[key] = [random_weight(N, K, g, mode == "asym") for _ in range(5)]
+        ws = cache[key] if cold else cache[key][:1] * 4
+        c = workloads.Case(cfg, M, N, K, group_size=g, mode=mode, out_dtype="bfloat16" if odt == torch.bfloat16 else "float16")
+        x = torch.randn(M, K, device=dev, dtype=torch.float16)
+        qa = ops.quantize_act_int8(x, g)
+        out = torch.empty((M, N), dtype=odt, device=dev)
+        for w in (ws if cold else ws[:1]):  # also allocates each copy's split-K workspace outside the capture
+            ops.w2a8_gemm(qa, w, odt, out=out)
+        us = time_graph(torch, lambda: [ops.w2a8_gemm(qa, w, odt, out=out) for w in ws], len(ws), replays=4)
+        nb, nops = workloads.algorithmic_bytes(c), workloads.algorithmic_ops(c)
+        others.append({"config": cfg, "shape": f"{N}x{K}", "M": M, "group": g, "mode": mode, "weights": "cold" if cold else "warm",
+                       "split_k": L.slimk_w2a8_gemm_auto_split_k(M, N, K, g, 0), "us": round(us, 2),
+                       "GBps": round(nb / (us * 1e-6) / 1e9, 1), "frac_hbm": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                       "TOPS": round(nops / (us * 1e-6) / 1e12, 1), "frac_int8_mfma": round(nops / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4)})
+    cache.clear()
+    detail["other_configs"] = others
     return detail
 
 
