@@ -103,10 +103,12 @@ int skinny_shared_split(int M, int N, int K, int group_size) {
 }
 
 // Split-K heuristic of the skinny kernel (measured on MI355X, cold weights).  One workgroup per
-// 64-channel strip already covers the chip when there are >= 192 strips, and a matrix of a few
+// 64-channel strip covers at least half the CUs when there are more than 128 strips, and a matrix of a few
 // MiB is latency-bound whatever is done, so both run unsplit: the cross-workgroup reduction
 // costs about 3 us.  Only a large matrix with few strips (small N, long K) is split, up to about
-// 256 workgroups, because a quarter of the CUs cannot pull full HBM bandwidth.
+// 256 workgroups, because a quarter of the CUs cannot pull full HBM bandwidth - and never beyond:
+// with more workgroups than CUs some CUs carry two (5120 x 13824, 80 strips: 8.2 us at split 3,
+// 11.6 us at split 4).
 int auto_split(int M, int N, int K, int group_size, int kernel) {
     if (kernel != SLIMK_KERNEL_SKINNY) {
         // the fast tiled kernel splits K when its tiles would leave CUs idle (group 64 / 128 only)
@@ -119,7 +121,7 @@ int auto_split(int M, int N, int K, int group_size, int kernel) {
     const int chunks = (K / 64 + 3) / 4;
     const size_t weight_bytes = (size_t)strips * 64 * (K / 4);
     int split = 1;
-    if (strips < 192 && weight_bytes > (size_t)6 << 20) split = (256 + strips - 1) / strips;
+    if (strips <= 128 && weight_bytes > (size_t)6 << 20) split = 256 / strips;  // never more workgroups than CUs
     const int max_split = chunks / 4 > 0 ? chunks / 4 : 1;
     if (split > max_split) split = max_split;
     if (split > 32) split = 32;
