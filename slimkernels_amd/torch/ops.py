@@ -106,6 +106,15 @@ def repack_w2(packed, scales, zp=None, group_size: int = 128, zp_const: int = 2,
     return W2A8Weight(w_r, s_r, zp_r, int(zp_const), N, K, group_size)
 
 
+def load_w2_weight(path, device="cuda", mmap=True) -> W2A8Weight:
+    """Read a weight file written by ``slimkernels_amd.packed_format.save_w2`` (the interchange
+    layout) and re-lay it for the GPU: the streaming layout exists only in device memory."""
+    from ..packed_format import load_w2
+    f = load_w2(path, mmap=mmap)
+    return repack_w2(np.ascontiguousarray(f["packed"]), np.ascontiguousarray(f["scales"]), f["zp"], f["group_size"],
+                     zp_const=f["zp_const"] if f["zp_const"] is not None else 0, device=device)
+
+
 def quantize_act_int8(x: torch.Tensor, group_size: int = 128) -> QuantizedActivation:
     """Per-token symmetric int8 quantisation: x [M, K] fp16/bf16 -> q, s_a, per-group row sums."""
     L = _lib.lib()
@@ -241,6 +250,11 @@ class W2A8Linear(torch.nn.Module):
         w = repack_w2(packed, scales, None if uniform is not None else zero, group_size,
                       zp_const=uniform if uniform is not None else 0, device=device)
         return cls(w, bias, out_dtype)
+
+    @classmethod
+    def from_file(cls, path, bias=None, out_dtype=torch.float16, device="cuda"):
+        """A layer from a packed weight file (slimkernels_amd.packed_format)."""
+        return cls(load_w2_weight(path, device), bias, out_dtype)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         lead = x.shape[:-1]
