@@ -116,6 +116,26 @@ int slimk_w2a8_repack(const uint8_t* w_packed, int ldw, const uint16_t* scales, 
                       int N, int K, int group_size,
                       uint32_t* w_r, uint16_t* s_r, uint8_t* zp_r, void* stream);
 
+/* which level set slimk_w2a8_quantize_weight produces */
+enum slimk_quant_mode {
+    SLIMK_QUANT_REF = 0,  /* upstream quantize_to_uint2: zero-point 1, scale = absmax / 1.5 (quantization.py:29-46) */
+    SLIMK_QUANT_SYM = 1,  /* levels -2..1: zero-point 2, scale = absmax / 2 */
+    SLIMK_QUANT_ASYM = 2  /* scale = (max - min) / 3, zero-point = clip(rne(-min / scale), 0, 3) per group */
+};
+
+/* Group-wise 2-bit weight quantisation on the GPU: the work of upstream quantize_to_uint2
+ * (quantization.py:17-53) followed by pack_matrix (matrix_packer.py:14-34), for a weight in the
+ * nn.Linear orientation, with the same numbers as the host-side functions of this package
+ * (binary32 arithmetic, IEEE division, round-half-even, the scale rounded to fp16 once).
+ *   w      [N][ldw] fp16 or bf16 (w_dtype), groups of group_size consecutive elements along K
+ *   packed [N][ldp] uint8 : four codes per byte along K, first code in bits 7:6; ldp >= K/4
+ *   scales [G][N]   fp16
+ *   zp     [G][N]   uint8 : written when non-NULL (constant 1 / 2 for REF / SYM); required for ASYM
+ * The outputs are the inputs of slimk_w2a8_repack.  w 16-byte aligned, ldw % 8 == 0, packed and
+ * ldp 2-byte aligned. */
+int slimk_w2a8_quantize_weight(const void* w, int ldw, int w_dtype, int N, int K, int group_size, int mode,
+                               uint8_t* packed, int ldp, uint16_t* scales, uint8_t* zp, void* stream);
+
 /* Per-token activation quantisation (no upstream counterpart; upstream feeds FP8,
  * wgmma_sm90_W2A8.cu:533-536).
  *   x [M][ldx] fp16 or bf16 (x_dtype)

@@ -14,6 +14,7 @@ OK = 0
 F16, BF16 = 0, 1
 KERNEL_AUTO, KERNEL_SKINNY, KERNEL_TILED = 0, 1, 2
 DUMP_NONE, DUMP_GROUPS, DUMP_SUM = 0, 1, 2
+QUANT_REF, QUANT_SYM, QUANT_ASYM = 0, 1, 2
 
 # every symbol include/slimk_w2a8.h declares: (restype, argtypes)
 _vp, _i, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
@@ -28,6 +29,7 @@ SIGNATURES = {
     "slimk_w2a8_gemm_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
     "slimk_w2a8_workspace_init": (_i, [_vp, _sz, _vp]),
     "slimk_w2a8_repack": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
+    "slimk_w2a8_quantize_weight": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp]),
     "slimk_w2a8_act_quant": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _vp]),
     "slimk_w2a8_gemm": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i,
                              _vp, _i, _i, _vp, _i, _vp, _sz, _i, _i, _vp]),

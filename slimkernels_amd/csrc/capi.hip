@@ -206,6 +206,23 @@ int slimk_w2a8_repack(const uint8_t* w_packed, int ldw, const uint16_t* scales, 
                       "repack");
 }
 
+int slimk_w2a8_quantize_weight(const void* w, int ldw, int w_dtype, int N, int K, int group_size, int mode,
+                               uint8_t* packed, int ldp, uint16_t* scales, uint8_t* zp, void* stream) {
+    if (!w || !packed || !scales) return fail(SLIMK_ERR_NULL_POINTER, "quantize_weight: NULL buffer");
+    if (N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "N=%d must be positive", N);
+    if (int rc = check_kg(K, group_size)) return rc;
+    if (w_dtype != SLIMK_F16 && w_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "w_dtype=%d", w_dtype);
+    if (mode < SLIMK_QUANT_REF || mode > SLIMK_QUANT_ASYM) return fail(SLIMK_ERR_BAD_ENUM, "mode=%d", mode);
+    if (mode == SLIMK_QUANT_ASYM && !zp) return fail(SLIMK_ERR_NULL_POINTER, "quantize_weight: per-group zero-points need zp");
+    if (ldw < K || ldp < K / 4) return fail(SLIMK_ERR_BAD_SHAPE, "ldw=%d / ldp=%d too small for K=%d", ldw, ldp, K);
+    if (!aligned16(w) || ldw % 8 != 0 || (reinterpret_cast<uintptr_t>(packed) & 1u) || ldp % 2 != 0 ||
+        (reinterpret_cast<uintptr_t>(scales) & 1u))
+        return fail(SLIMK_ERR_MISALIGNED, "quantize_weight: w 16-byte aligned, ldw %% 8 == 0, packed / ldp / scales 2-byte aligned");
+    return hip_result(w2a8::launch_quantize_weight(w, ldw, w_dtype == SLIMK_BF16, N, K, group_size, mode, packed, ldp,
+                                                   scales, zp, (hipStream_t)stream),
+                      "quantize_weight");
+}
+
 int slimk_w2a8_act_quant(const void* x, int ldx, int x_dtype, int M, int K, int group_size,
                          int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, void* stream) {
     if (!x || !q || !s_a) return fail(SLIMK_ERR_NULL_POINTER, "act_quant: NULL buffer");

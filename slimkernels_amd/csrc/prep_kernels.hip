@@ -153,6 +153,85 @@ hipError_t launch_act_quant(const void* x, int ldx, bool x_bf16, int M, int K, i
     return hipGetLastError();
 }
 
+// ------------------------------------------------------------------ weight quantisation
+// fp16 / bf16 weights [N][ldw] -> the interchange format: packed 2-bit codes [N][ldp] (four codes per
+// byte along K, first code in bits 7:6: matrix_packer.py:33-34 upstream), group scales [G][N] fp16
+// and zero-points [G][N] (quantization.py:29-53 upstream for mode 0; the symmetric and asymmetric
+// level sets otherwise).  All arithmetic in binary32 with IEEE division and round-half-even, the
+// scale rounded to fp16 once for storage after the codes are made with the fp32 one.
+// Each thread handles 8 consecutive elements of one row (one 16-byte load); the group_size / 8
+// threads of a group sit in one wave and meet through shuffles.
+//   mode 0: zero-point 1, scale = absmax / 1.5      (upstream quantizer)
+//   mode 1: zero-point 2, scale = absmax / 2        (levels -2..1)
+//   mode 2: scale = (max - min) / 3, zero-point = clip(rne(-min / scale), 0, 3) per group
+template <bool BF16>
+__global__ __launch_bounds__(256) void quantize_weight_kernel(const uint16_t* __restrict__ w, int ldw, int N, int K,
+                                                              int group_size, int mode, uint8_t* __restrict__ packed,
+                                                              int ldp, uint16_t* __restrict__ scales,
+                                                              uint8_t* __restrict__ zp) {
+    const int n = blockIdx.y;
+    const int v = blockIdx.x * 256 + threadIdx.x;  // 8-element vector of the row
+    const bool on = v < K / 8;                      // K / 8 is a multiple of a group's threads: whole groups on or off
+    float f[8];
+    if (on) {
+        load8<BF16>(w + (size_t)n * ldw + (size_t)v * 8, f);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = 0.0f;
+    }
+    float hi = f[0], lo = f[0], amax = fabsf(f[0]);
+#pragma unroll
+    for (int i = 1; i < 8; ++i) {
+        hi = fmaxf(hi, f[i]);
+        lo = fminf(lo, f[i]);
+        amax = fmaxf(amax, fabsf(f[i]));
+    }
+    const int tpg = group_size / 8;
+    for (int off = 1; off < tpg; off <<= 1) {
+        hi = fmaxf(hi, __shfl_xor(hi, off, 64));
+        lo = fminf(lo, __shfl_xor(lo, off, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    }
+    const float tiny = 1e-9f;
+    float s, zero;
+    if (mode == 0) {
+        s = fmaxf(amax, tiny) / 1.5f;
+        zero = 1.0f;
+    } else if (mode == 1) {
+        s = fmaxf(amax, tiny) / 2.0f;
+        zero = 2.0f;
+    } else {
+        s = fmaxf(hi - lo, tiny) / 3.0f;
+        zero = fminf(fmaxf(rintf(-lo / s), 0.0f), 3.0f);
+    }
+    if (!on) return;
+    uint32_t bytes = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float level = fminf(fmaxf(rintf(f[i] / s) + zero, 0.0f), 3.0f);
+        const uint32_t code = (uint32_t)(int)level;
+        bytes |= code << ((i >> 2) * 8 + 6 - 2 * (i & 3));  // byte i / 4, first code of a byte in bits 7:6
+    }
+    *reinterpret_cast<uint16_t*>(packed + (size_t)n * ldp + (size_t)v * 2) = (uint16_t)bytes;
+    if (v % tpg == 0) {
+        const size_t g = (size_t)(v / tpg);
+        scales[g * N + n] = __builtin_bit_cast(uint16_t, (_Float16)s);
+        if (zp) zp[g * N + n] = (uint8_t)(int)zero;
+    }
+}
+
+hipError_t launch_quantize_weight(const void* w, int ldw, bool w_bf16, int N, int K, int group_size, int mode,
+                                  uint8_t* packed, int ldp, uint16_t* scales, uint8_t* zp, hipStream_t stream) {
+    const dim3 grid((unsigned)((K / 8 + 255) / 256), (unsigned)N), block(256);
+    if (w_bf16)
+        quantize_weight_kernel<true><<<grid, block, 0, stream>>>((const uint16_t*)w, ldw, N, K, group_size, mode, packed,
+                                                                ldp, scales, zp);
+    else
+        quantize_weight_kernel<false><<<grid, block, 0, stream>>>((const uint16_t*)w, ldw, N, K, group_size, mode, packed,
+                                                                 ldp, scales, zp);
+    return hipGetLastError();
+}
+
 // ------------------------------------------------------------------ fill / probe
 __global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t* p, size_t n_dwords) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n_dwords; i += (size_t)gridDim.x * 256) p[i] = 0u;

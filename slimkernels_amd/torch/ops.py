@@ -106,6 +106,35 @@ def repack_w2(packed, scales, zp=None, group_size: int = 128, zp_const: int = 2,
     return W2A8Weight(w_r, s_r, zp_r, int(zp_const), N, K, group_size)
 
 
+def quantize_weight_gpu(weight_nk: torch.Tensor, group_size: int = 128, mode: str = "sym"):
+    """Group-wise 2-bit quantisation of an fp16 / bf16 weight [N, K] on the GPU: the same numbers as
+    ``slimkernels_amd.prepare_w2`` on the host.  Returns (packed uint8 [N, K/4], scales float16 [G, N],
+    zero-points uint8 [G, N]) as device tensors in the interchange layout."""
+    L = _lib.lib()
+    _require_cuda(weight_nk, "weight")
+    if weight_nk.dim() != 2 or weight_nk.dtype not in _DT:
+        raise ValueError("weight must be a 2-D float16 or bfloat16 tensor [N, K]")
+    modes = {"ref": _lib.QUANT_REF, "sym": _lib.QUANT_SYM, "asym": _lib.QUANT_ASYM}
+    if mode not in modes:
+        raise ValueError(f"unknown quantizer mode {mode!r} (expected 'ref', 'sym' or 'asym')")
+    w = weight_nk if weight_nk.stride(1) == 1 and weight_nk.stride(0) % 8 == 0 and weight_nk.data_ptr() % 16 == 0 \
+        else weight_nk.contiguous()
+    N, K = w.shape
+    if group_size not in (64, 128, 256) or K % group_size != 0:
+        raise ValueError(f"unsupported K={K}, group_size={group_size} (group_size in (64, 128, 256), K % group_size == 0)")
+    dev = w.device
+    packed = torch.empty((N, K // 4), dtype=torch.uint8, device=dev)
+    scales = torch.empty((K // group_size, N), dtype=torch.float16, device=dev)
+    zero = torch.empty((K // group_size, N), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(L.slimk_w2a8_quantize_weight(w.data_ptr(), w.stride(0), _DT[w.dtype], N, K, group_size, modes[mode],
+                                                packed.data_ptr(), packed.stride(0), scales.data_ptr(), zero.data_ptr(),
+                                                _stream_ptr(dev)))
+        if w is not weight_nk:
+            torch.cuda.current_stream(dev).synchronize()  # the contiguous copy is consumed by the enqueued kernel
+    return packed, scales, zero
+
+
 def load_w2_weight(path, device="cuda", mmap=True) -> W2A8Weight:
     """Read a weight file written by ``slimkernels_amd.packed_format.save_w2`` (the interchange
     layout) and re-lay it for the GPU: the streaming layout exists only in device memory."""
@@ -244,9 +273,15 @@ class W2A8Linear(torch.nn.Module):
     @classmethod
     def from_float(cls, weight_nk, group_size=128, mode="sym", bias=None, out_dtype=torch.float16, device="cuda"):
         from ..quantization import prepare_w2
+        uniform = {"sym": 2, "ref": 1}.get(mode)
+        if isinstance(weight_nk, torch.Tensor) and weight_nk.is_cuda and weight_nk.dtype in _DT:
+            # quantise where the weight already is (same numbers as the host path)
+            packed, scales, zero = quantize_weight_gpu(weight_nk.detach(), group_size, mode)
+            w = repack_w2(packed, scales, None if uniform is not None else zero, group_size,
+                          zp_const=uniform if uniform is not None else 0, device=weight_nk.device)
+            return cls(w, bias, out_dtype)
         w_np = weight_nk.detach().float().cpu().numpy() if isinstance(weight_nk, torch.Tensor) else np.asarray(weight_nk)
         packed, scales, zero = prepare_w2(w_np, group_size, mode)
-        uniform = {"sym": 2, "ref": 1}.get(mode)
         w = repack_w2(packed, scales, None if uniform is not None else zero, group_size,
                       zp_const=uniform if uniform is not None else 0, device=device)
         return cls(w, bias, out_dtype)

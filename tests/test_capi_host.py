@@ -120,6 +120,16 @@ def test_repack_and_act_quant_validation(L):
     assert a(FAKE, 100, 0, 1, 4096, 128, FAKE, 4096, FAKE, FAKE, 4, None) == 2
     assert a(FAKE, 4096 + 4, 0, 1, 4096, 128, FAKE, 4096, FAKE, FAKE, 4, None) == 3
     assert a(FAKE, 4096, 0, 5, 4096, 128, FAKE, 4096, FAKE, FAKE, 4, None) == 2        # ldr < M
+    qw = L.slimk_w2a8_quantize_weight  # (w, ldw, dtype, N, K, group, mode, packed, ldp, scales, zp, stream)
+    assert qw(None, 4096, 0, 64, 4096, 128, 1, FAKE, 1024, FAKE, None, None) == 1
+    assert qw(FAKE, 4096, 0, 64, 4096, 128, 2, FAKE, 1024, FAKE, None, None) == 1      # per-group zero-points need zp
+    assert qw(FAKE, 4096, 0, 0, 4096, 128, 1, FAKE, 1024, FAKE, None, None) == 2
+    assert qw(FAKE, 4096, 0, 64, 4096, 100, 1, FAKE, 1024, FAKE, None, None) == 2
+    assert qw(FAKE, 4096, 0, 64, 4096, 128, 1, FAKE, 1000, FAKE, None, None) == 2      # ldp < K/4
+    assert qw(FAKE, 4096, 2, 64, 4096, 128, 1, FAKE, 1024, FAKE, None, None) == 4      # dtype
+    assert qw(FAKE, 4096, 0, 64, 4096, 128, 3, FAKE, 1024, FAKE, None, None) == 4      # mode
+    assert qw(FAKE, 4100, 0, 64, 4096, 128, 1, FAKE, 1024, FAKE, None, None) == 3      # ldw % 8
+    assert qw(FAKE, 4096, 0, 64, 4096, 128, 1, FAKE + 1, 1024, FAKE, None, None) == 3
     assert L.slimk_w2a8_workspace_init(None, 64, None) == 1
     assert L.slimk_w2a8_workspace_init(FAKE, 0, None) == 0                             # nothing to do
     assert L.slimk_w2a8_read_probe(FAKE, 24, FAKE, None) == 3

@@ -35,6 +35,43 @@ def test_repack_matches_layout_definition(gpu_ops, N, K, g, with_zp):
         np.testing.assert_array_equal(w.zp_r.cpu().numpy().reshape(K // g, strips, 16, 4), layout.repack_group_values(zp))
 
 
+# ------------------------------------------------------------------ weight quantisation on the GPU
+@pytest.mark.parametrize("N,K,g,mode,bf16", [(64, 256, 128, "sym", False), (100, 512, 64, "asym", False),
+                                             (7, 768, 256, "ref", False), (130, 1024, 128, "asym", True),
+                                             (33, 8192, 128, "sym", True), (256, 4096, 64, "ref", False)])
+def test_weight_quantisation_on_gpu_bit_exact(gpu_ops, N, K, g, mode, bf16):
+    """fp16 / bf16 weight -> packed codes, fp16 scales, zero-points: the host functions' numbers."""
+    from slimkernels_amd import prepare_w2
+    _say("quantize_weight", N, K, g, mode, bf16)
+    rng = np.random.default_rng(N + K)
+    w = rng.normal(0, 0.02, (N, K)).astype(np.float32)
+    w[0, :g] = 0.0                                   # an all-zero group: scale floor, codes = zero-point
+    w[min(1, N - 1), 3] = 0.5                        # an outlier that sets its group's scale
+    wt = torch.from_numpy(w).to(torch.bfloat16 if bf16 else torch.float16)
+    # ties: values at exactly (level + 0.5) * scale of their group (scale = absmax / 2 resp. / 1.5)
+    if mode != "asym":
+        div = 2.0 if mode == "sym" else 1.5
+        wt[min(2, N - 1), :g] = 0.0
+        wt[min(2, N - 1), 0] = 1.0
+        for i, lv in enumerate((0.5, -0.5, 1.5, -1.5, 2.5, -2.5)):
+            wt[min(2, N - 1), 1 + i] = lv / div
+    host = prepare_w2(wt.float().numpy(), g, mode)
+    packed, scales, zero = gpu_ops.quantize_weight_gpu(wt.cuda(), g, mode)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(packed.cpu().numpy(), host[0])
+    np.testing.assert_array_equal(scales.cpu().numpy().view(np.uint16), host[1].view(np.uint16))
+    np.testing.assert_array_equal(zero.cpu().numpy(), host[2])
+    # a strided view (rows of a wider matrix) takes the same path
+    wide = torch.zeros(N, K + 8, dtype=wt.dtype, device="cuda")
+    wide[:, :K] = wt.cuda()
+    packed2, scales2, zero2 = gpu_ops.quantize_weight_gpu(wide[:, :K], g, mode)
+    assert torch.equal(packed, packed2) and torch.equal(scales, scales2) and torch.equal(zero, zero2)
+    # and the layer built from the device tensor equals the one built on the host
+    lin_d = gpu_ops.W2A8Linear.from_float(wt.cuda(), g, mode)
+    lin_h = gpu_ops.W2A8Linear.from_float(wt.float().numpy(), g, mode)
+    assert torch.equal(lin_d.weight.w_r, lin_h.weight.w_r) and torch.equal(lin_d.weight.s_r, lin_h.weight.s_r)
+
+
 # ------------------------------------------------------------------ activation quantisation
 @pytest.mark.parametrize("M,K,g,bf16,outliers", [(1, 4096, 128, False, True), (16, 4096, 128, False, True),
                                                  (77, 4096, 128, False, False), (3, 13824, 128, False, False),
