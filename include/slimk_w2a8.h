@@ -171,6 +171,20 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
                     void* workspace, size_t workspace_bytes,
                     int kernel, int split_k, void* stream);
 
+/* The GEMM for at most four token rows with the activation quantisation inside: x [M][ldx] fp16 or
+ * bf16 (x_dtype) takes the place of q, s_a and rowsum, and every workgroup quantises the rows itself
+ * (same numbers as slimk_w2a8_act_quant) while its first weights are on the way - one launch
+ * instead of two on the latency-bound decode path.  M <= 4 and M * K <= 32768, else
+ * SLIMK_ERR_UNSUPPORTED.  The result is bit-identical with slimk_w2a8_act_quant followed by
+ * slimk_w2a8_gemm (skinny kernel, same split_k).  Workspace and split_k as for slimk_w2a8_gemm
+ * with SLIMK_KERNEL_SKINNY.  x 16-byte aligned, ldx % 8 == 0.
+ * No upstream counterpart (upstream feeds already quantised FP8, wgmma_sm90_W2A8.cu:533-536). */
+int slimk_w2a8_gemm_fused(const void* x, int ldx, int x_dtype,
+                          const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
+                          int M, int N, int K, int group_size,
+                          void* out, int ldo, int out_dtype,
+                          void* workspace, size_t workspace_bytes, int split_k, void* stream);
+
 /* One problem of a grouped launch: the arguments of slimk_w2a8_gemm that describe data. */
 typedef struct slimk_w2a8_problem {
     const int8_t* q;

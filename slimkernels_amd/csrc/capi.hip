@@ -326,6 +326,50 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
     return hip_result(w2a8::launch_tiled(p, gs, asym, out_bf16, st), "tiled gemm");
 }
 
+int slimk_w2a8_gemm_fused(const void* x, int ldx, int x_dtype,
+                          const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
+                          int M, int N, int K, int group_size,
+                          void* out, int ldo, int out_dtype,
+                          void* workspace, size_t workspace_bytes, int split_k, void* stream) {
+    if (!x || !w_r || !s_r || !out) return fail(SLIMK_ERR_NULL_POINTER, "gemm_fused: NULL buffer");
+    if (M <= 0 || N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "M=%d, N=%d must be positive", M, N);
+    if (int rc = check_kg(K, group_size)) return rc;
+    if (x_dtype != SLIMK_F16 && x_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "x_dtype=%d", x_dtype);
+    if (out_dtype != SLIMK_F16 && out_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "out_dtype=%d", out_dtype);
+    if (zp_const < 0 || zp_const > 3) return fail(SLIMK_ERR_BAD_SHAPE, "zp_const=%d must be 0..3", zp_const);
+    if (ldx < K || ldo < N) return fail(SLIMK_ERR_BAD_SHAPE, "ldx=%d / ldo=%d too small for K=%d / N=%d", ldx, ldo, K, N);
+    if (M > w2a8::kFusedMaxRows || (size_t)M * K > (size_t)w2a8::kFusedMaxBytes)
+        return fail(SLIMK_ERR_UNSUPPORTED, "gemm_fused handles M <= %d with M * K <= %d (M=%d, K=%d)", w2a8::kFusedMaxRows,
+                    w2a8::kFusedMaxBytes, M, K);
+    if (int rc = check_extent(M, N, K, K)) return rc;
+    if (!aligned16(x) || ldx % 8 != 0 || !aligned16(w_r) || !aligned16(s_r) || (zp_r && !aligned16(zp_r)) ||
+        (reinterpret_cast<uintptr_t>(out) & 1u))
+        return fail(SLIMK_ERR_MISALIGNED, "gemm_fused: x, w_r, s_r, zp_r must be 16-byte aligned; ldx %% 8 == 0; out 2-byte aligned");
+    const int G = K / group_size;
+    if (split_k <= 0) split_k = auto_split(M, N, K, group_size, SLIMK_KERNEL_SKINNY);
+    if (split_k > G) return fail(SLIMK_ERR_BAD_SHAPE, "split_k=%d exceeds the number of groups %d", split_k, G);
+    const int gps = groups_per_split(G, group_size, split_k);
+    split_k = (G + gps - 1) / gps;
+
+    w2a8::GemmParams p{};
+    p.x = reinterpret_cast<const uint16_t*>(x); p.ldx = ldx; p.x_bf16 = x_dtype == SLIMK_BF16 ? 1 : 0;
+    p.w_r = w_r; p.s_r = s_r; p.zp_r = zp_r; p.out = out; p.ldo = ldo;
+    p.M = M; p.N = N; p.K = K; p.G = G; p.steps = K / w2a8::kStepK; p.strips = strips_of(N);
+    p.zp_const = zp_const; p.split = split_k; p.groups_per_split = gps;
+    if (split_k > 1) {
+        const size_t need = slimk_w2a8_gemm_workspace_bytes(M, N, K, group_size, SLIMK_KERNEL_SKINNY, split_k);
+        if (!workspace) return fail(SLIMK_ERR_WORKSPACE, "split_k=%d needs a workspace of %zu bytes", split_k, need);
+        if (workspace_bytes < need)
+            return fail(SLIMK_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, need);
+        if (!aligned16(workspace)) return fail(SLIMK_ERR_MISALIGNED, "workspace must be 16-byte aligned");
+        p.ws_counter = reinterpret_cast<unsigned*>(workspace);
+        p.ws_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counter_bytes(p.strips));
+    }
+    return hip_result(w2a8::launch_skinny_fused(p, group_size / w2a8::kStepK, skinny_waves(M, N, K, split_k), zp_r != nullptr,
+                                                out_dtype == SLIMK_BF16, (hipStream_t)stream),
+                      "fused skinny gemm");
+}
+
 int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int group_size, int out_dtype,
                             void* stream) {
     if (!problems) return fail(SLIMK_ERR_NULL_POINTER, "gemm_grouped: problems is NULL");

@@ -40,7 +40,16 @@ struct SkinnyMeta {
     int32_t rowsum[kDepth][16];
 };
 
-template <int NWP, bool WIDE>
+// FUSED: the workgroup quantises the (at most four) token rows itself before it needs them.
+struct FusedRows {
+    int8_t q[kFusedMaxBytes];                  // [row][K]
+    v4i rowsum[kFusedMaxBytes / kStepK];       // [group]: the rows' sums of q over the group (rows past M: 0)
+    float s_a[kFusedMaxRows];
+    float amax[16][kFusedMaxRows];             // per wave, then reduced
+};
+struct NoFusedRows {};
+
+template <int NWP, bool WIDE, bool FUSED = false>
 struct SkinnySmem {
     union {
         SkinnyMeta meta[NWP];
@@ -48,6 +57,7 @@ struct SkinnySmem {
     };
     v4u atile[WIDE ? NWP : 1][kDepth][64];  // WIDE: a wave's activation fragments of one chunk, in MFMA operand order
     int last;
+    typename std::conditional<FUSED, FusedRows, NoFusedRows>::type fused;
 };
 
 // One wave's share of one strip and one block of 16 token rows (a problem with 17..32 rows is
@@ -60,6 +70,9 @@ struct SkinnySmem {
 //         stores its results itself; NWP: all the workgroup's waves, meeting in LDS)
 //   ASYM  per-(group, channel) zero-points from zp_r instead of the uniform zp_const
 //   DUMP  verification build: exact int32 group sums are written out
+//   FUSED the activations arrive as fp16 / bf16 rows (at most four, rows x K <= 32 KiB) and every
+//         workgroup quantises them itself into LDS while its first weights are on the way: the numbers
+//         of act_quant_kernel (per-token scale, int8 values, per-group sums), no separate launch
 //   WIDE  activations are fetched two steps wide (whole 128-byte lines of the row-major tokens: half
 //         the cache lines of a step-by-step fetch once there are eight rows or more) and turned into
 //         MFMA operand order through a wave-private LDS tile; no barrier, the wave only meets itself
@@ -70,10 +83,11 @@ struct SkinnySmem {
 // product over the groups (16 tokens x 16 channels x up to 4 groups of a chunk) and goes through
 // one v_mfma_f32_16x16x4_f32 per chunk and sub-block, accumulating straight into the fp32 running
 // sums (same D layout as the int8 MFMA).  The verification build folds it in integers instead.
-template <int J, int GS, int NWK, int NWP, bool ASYM, bool DUMP, bool NT, bool WIDE, typename OutT>
+template <int J, int GS, int NWK, int NWP, bool ASYM, bool DUMP, bool NT, bool WIDE, bool FUSED, typename OutT>
 __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip, const int split, const int mblk,
-                                            const int kwave, const int pwave, SkinnySmem<NWP, WIDE>& sm) {
+                                            const int kwave, const int pwave, SkinnySmem<NWP, WIDE, FUSED>& sm) {
     static_assert(!(WIDE && DUMP), "the verification build fetches step by step");
+    static_assert(!FUSED || (!WIDE && !DUMP && NWK == NWP), "fused activation quantisation: the plain production body");
     constexpr int MB = 1;
     static_assert(NWK == 1 || NWK == NWP, "K is split over one wave or over the whole workgroup");
     constexpr int kThreads = NWP * 64;
@@ -100,7 +114,9 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
 
     // token scales for the epilogue, fetched first
     float sa[NWK == 1 ? MB * J : kOutPerThread];
-    if (NWK == 1) {  // this wave stores D fragments itself: rows mb*16 + quad*4 + j
+    if (FUSED) {
+        // set once the rows are quantised
+    } else if (NWK == 1) {  // this wave stores D fragments itself: rows mb*16 + quad*4 + j
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
@@ -143,17 +159,29 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     v4i m_scale;     // scales: up to 4 groups x 128 B = 512 B per wave: lanes 0..31, 16 B each
     v4i m_zp;        // zero-points: up to 4 groups x 64 B: lanes 0..15
     v4i m_rs[MB];    // row sums: lane -> (group lane >> 2, rows 4*(lane & 3) ..): lanes 0..15
-    auto fetch_meta = [&](int gfirst) {  // groups gfirst .. gfirst + kGroupsPerChunk - 1, clamped to g1 - 1
-        const size_t sgi = (size_t)min(gfirst + (lane >> 3), g1 - 1) * p.strips + strip;
-        m_scale = *reinterpret_cast<const v4i*>(reinterpret_cast<const char*>(p.s_r) + sgi * 128 + (lane & 7) * 16);
+    auto fused_rowsum = [&](int g) -> v4i {
+        if constexpr (FUSED) return sm.fused.rowsum[g];
+        else return v4i{0, 0, 0, 0};
+    };
+    // (FUSED: the row sums come from LDS once the rows are quantised; the entry path fetches the
+    // global part before that and the row sums after it)
+    auto fetch_meta = [&](int gfirst, bool global_part = true, bool rowsum_part = true) {  // groups gfirst .. gfirst + kGroupsPerChunk - 1, clamped to g1 - 1
         const int gq = min(gfirst + (lane >> 2), g1 - 1);
-        if (ASYM)
-            m_zp = *reinterpret_cast<const v4i*>(reinterpret_cast<const char*>(p.zp_r) +
-                                                 ((size_t)gq * p.strips + strip) * 64 + (lane & 3) * 16);
-        const int32_t* rp = rsp + (size_t)gq * p.ldr;
+        if (global_part) {
+            const size_t sgi = (size_t)min(gfirst + (lane >> 3), g1 - 1) * p.strips + strip;
+            m_scale = *reinterpret_cast<const v4i*>(reinterpret_cast<const char*>(p.s_r) + sgi * 128 + (lane & 7) * 16);
+            if (ASYM)
+                m_zp = *reinterpret_cast<const v4i*>(reinterpret_cast<const char*>(p.zp_r) +
+                                                     ((size_t)gq * p.strips + strip) * 64 + (lane & 3) * 16);
+        }
+        if (FUSED) {
+            if (rowsum_part) m_rs[0] = (lane & 3) == 0 ? fused_rowsum(gq) : v4i{0, 0, 0, 0};  // rows 0..3 only
+        } else {
+            const int32_t* rp = rsp + (size_t)gq * p.ldr;
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-            m_rs[mb] = *reinterpret_cast<const v4i*>(rp + min(mb * 16 + (lane & 3) * 4, ldr - 4));
+            for (int mb = 0; mb < MB; ++mb)
+                m_rs[mb] = *reinterpret_cast<const v4i*>(rp + min(mb * 16 + (lane & 3) * 4, ldr - 4));
+        }
     };
     auto park_meta = [&](int gfirst) {  // the registers hold groups gfirst ..
         // a group past the end of the range (ragged last chunk) gets zero scales: it then adds nothing
@@ -173,7 +201,7 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     v4u aring[kDepth][MB];
     auto issue = [&](int slot, int step) {  // step is wave-uniform
         wring[slot] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane, step * wstride + wbase, NT ? kStreamOnce : 0);
-        if (!WIDE) {
+        if (!WIDE && !FUSED) {
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
                 aring[slot][mb] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, aoff[mb], step * kStepK, 0);
@@ -215,12 +243,141 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     if (s0 < s1) {
         // Same issue order as inside the loop (metadata first, then the ring), fenced, so that the
         // wait counts the compiler derives for the loop head hold on the entry path as well.
-        fetch_meta(stepof(0) / GS);
+        fetch_meta(stepof(0) / GS, true, !FUSED);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < kDepth; ++i) issue(i, stepof(i));
         if (WIDE) fetch_wide(0);
         __builtin_amdgcn_sched_barrier(0);
+    }
+
+    if constexpr (FUSED) {
+        // ---- the workgroup quantises the token rows (every wave takes part, also one without steps),
+        // while the loads above are on the way.  Pass 1: per-row absmax.  Pass 2: q = clip(rne(x / s)),
+        // the per-group sums of q; IEEE binary32 division, as act_quant_kernel.
+        FusedRows& fr = sm.fused;
+        constexpr int tpg = GS * 8;  // threads per scale group (8 elements each)
+        const int nvec = p.K / 8;
+        const bool bf16 = p.x_bf16 != 0;
+        auto load8 = [&](const uint16_t* src, float (&f)[8]) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(src);
+            const uint32_t wds[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (bf16) {
+                    f[2 * i] = __uint_as_float(wds[i] << 16);
+                    f[2 * i + 1] = __uint_as_float(wds[i] & 0xffff0000u);
+                } else {
+                    f[2 * i] = half_bits_to_float((uint16_t)(wds[i] & 0xffffu));
+                    f[2 * i + 1] = half_bits_to_float((uint16_t)(wds[i] >> 16));
+                }
+            }
+        };
+        auto quantise8 = [&](const float (&f)[8], float s, uint32_t& lo, uint32_t& hi) -> int {
+            int sum = 0;
+            lo = 0; hi = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float r = rintf(f[i] / s);
+                r = fminf(fmaxf(r, -127.0f), 127.0f);
+                const int qi = (int)r;
+                sum += qi;
+                if (i < 4) lo |= (uint32_t)(qi & 0xff) << (8 * i);
+                else hi |= (uint32_t)(qi & 0xff) << (8 * (i - 4));
+            }
+            return sum;
+        };
+        constexpr int kKeep = 4;  // 8-element vectors of the row a thread keeps in registers between the passes
+        if (J == 1 && nvec <= kKeep * kThreads) {
+            // one token row (the decode case): the row is read once and stays in registers
+            float f[kKeep][8];
+            float amax = 0.0f;
+#pragma unroll
+            for (int it = 0; it < kKeep; ++it) {
+                const int v = tid + it * kThreads;
+                if (v < nvec) {
+                    load8(p.x + (size_t)v * 8, f[it]);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(f[it][i]));
+                }
+            }
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+            if (lane == 0) fr.amax[pwave][0] = amax;
+            __syncthreads();
+            float a = fr.amax[0][0];
+            for (int w = 1; w < NWP; ++w) a = fmaxf(a, fr.amax[w][0]);
+            const float s = fmaxf(a, 1e-9f) / 127.0f;
+            if (tid < kFusedMaxRows) fr.s_a[tid] = s;
+#pragma unroll
+            for (int it = 0; it < kKeep; ++it) {
+                const int v = tid + it * kThreads;
+                if (v < nvec) {  // whole groups of threads are in or out
+                    uint32_t lo, hi;
+                    int sum = quantise8(f[it], s, lo, hi);
+                    *reinterpret_cast<uint2*>(&fr.q[(size_t)v * 8]) = make_uint2(lo, hi);
+                    for (int off = 1; off < tpg; off <<= 1) sum += __shfl_xor(sum, off, 64);
+                    if (v % tpg == 0) fr.rowsum[v / tpg] = v4i{sum, 0, 0, 0};
+                }
+            }
+        } else {
+            float amax[kFusedMaxRows] = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (int v = tid; v < nvec; v += kThreads) {
+#pragma unroll
+                for (int m = 0; m < kFusedMaxRows; ++m) {
+                    if (m < p.M) {
+                        float f[8];
+                        load8(p.x + (size_t)m * p.ldx + (size_t)v * 8, f);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) amax[m] = fmaxf(amax[m], fabsf(f[i]));
+                    }
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < kFusedMaxRows; ++m) {
+#pragma unroll
+                for (int off = 32; off >= 1; off >>= 1) amax[m] = fmaxf(amax[m], __shfl_xor(amax[m], off, 64));
+                if (lane == 0) fr.amax[pwave][m] = amax[m];
+            }
+            __syncthreads();
+            float srow[kFusedMaxRows];
+#pragma unroll
+            for (int m = 0; m < kFusedMaxRows; ++m) {
+                float a = fr.amax[0][m];
+                for (int w = 1; w < NWP; ++w) a = fmaxf(a, fr.amax[w][m]);
+                srow[m] = fmaxf(a, 1e-9f) / 127.0f;
+            }
+            if (tid < kFusedMaxRows) fr.s_a[tid] = srow[tid];
+            for (int v = tid; v < nvec; v += kThreads) {
+                int sums[kFusedMaxRows] = {0, 0, 0, 0};
+#pragma unroll
+                for (int m = 0; m < kFusedMaxRows; ++m) {
+                    if (m < p.M) {
+                        float f[8];
+                        load8(p.x + (size_t)m * p.ldx + (size_t)v * 8, f);
+                        uint32_t lo, hi;
+                        sums[m] = quantise8(f, srow[m], lo, hi);
+                        *reinterpret_cast<uint2*>(&fr.q[(size_t)m * p.K + (size_t)v * 8]) = make_uint2(lo, hi);
+                    }
+                }
+#pragma unroll
+                for (int m = 0; m < kFusedMaxRows; ++m)
+                    for (int off = 1; off < tpg; off <<= 1) sums[m] += __shfl_xor(sums[m], off, 64);
+                if (v % tpg == 0) fr.rowsum[v / tpg] = v4i{sums[0], sums[1], sums[2], sums[3]};
+            }
+        }
+        __syncthreads();
+        if (NWK == 1) {
+#pragma unroll
+            for (int j = 0; j < J; ++j) sa[j] = fr.s_a[min(quad * 4 + j, kFusedMaxRows - 1)];
+        } else {
+#pragma unroll
+            for (int i = 0; i < kOutPerThread; ++i) sa[i] = fr.s_a[min((tid + kThreads * i) >> 6, kFusedMaxRows - 1)];
+        }
+    }
+
+    if (s0 < s1) {
+        if (FUSED) fetch_meta(stepof(0) / GS, false, true);  // the row sums of the first chunk, now that they exist
 
         v4i acc[MB][4];
         v4h sc;          // the group's four sub-block scales, kept in fp16: the drain's fma reads them as such
@@ -261,6 +418,12 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
                 }
             }
 
+            if constexpr (FUSED) {
+                const int8_t* qrow = &sm.fused.q[(size_t)min(col, M - 1) * p.K + quad * 16];
+#pragma unroll
+                for (int i = 0; i < kDepth; ++i)
+                    aring[i][0] = *reinterpret_cast<const v4u*>(qrow + (size_t)stepof(it + i) * kStepK);
+            }
             if (WIDE) {
                 park_wide();                  // this chunk's fragments: registers -> LDS tile
                 fetch_wide(it + kDepth);      // next chunk's: global -> registers
@@ -439,7 +602,15 @@ template <int J, int GS, int NW, bool ASYM, bool DUMP, bool NT, bool WIDE, typen
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const GemmParams p) {
     __shared__ __attribute__((aligned(16))) SkinnySmem<NW, WIDE> sm;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keeps ranges and bases in SGPRs
-    skinny_body<J, GS, NW, NW, ASYM, DUMP, NT, WIDE, OutT>(p, blockIdx.x, blockIdx.y, blockIdx.z, wave, wave, sm);
+    skinny_body<J, GS, NW, NW, ASYM, DUMP, NT, WIDE, false, OutT>(p, blockIdx.x, blockIdx.y, blockIdx.z, wave, wave, sm);
+}
+
+// The same with the activation quantisation inside (at most four token rows, given as fp16 / bf16).
+template <int J, int GS, int NW, bool ASYM, typename OutT>
+__global__ __launch_bounds__(NW * 64) void skinny_fused_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(16))) SkinnySmem<NW, false, true> sm;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    skinny_body<J, GS, NW, NW, ASYM, false, true, false, true, OutT>(p, blockIdx.x, blockIdx.y, 0, wave, wave, sm);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -949,6 +1120,38 @@ hipError_t launch_skinny_grouped(const GroupedParams& gp, int gs, bool asym, boo
     if (gs == 1) launch_grouped_zm<1>(gp, total_wgs, asym, out_bf16, stream);
     else if (gs == 2) launch_grouped_zm<2>(gp, total_wgs, asym, out_bf16, stream);
     else launch_grouped_zm<4>(gp, total_wgs, asym, out_bf16, stream);
+    return hipGetLastError();
+}
+
+template <int J, int GS, int NW>
+static void launch_fused_jgn(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
+    const dim3 grid(p.strips, p.split), block(NW * 64);
+    if (asym) {
+        if (out_bf16) skinny_fused_kernel<J, GS, NW, true, OutBF16><<<grid, block, 0, stream>>>(p);
+        else skinny_fused_kernel<J, GS, NW, true, OutF16><<<grid, block, 0, stream>>>(p);
+    } else {
+        if (out_bf16) skinny_fused_kernel<J, GS, NW, false, OutBF16><<<grid, block, 0, stream>>>(p);
+        else skinny_fused_kernel<J, GS, NW, false, OutF16><<<grid, block, 0, stream>>>(p);
+    }
+}
+
+template <int GS>
+static void launch_fused_gs(const GemmParams& p, int waves, bool asym, bool out_bf16, hipStream_t stream) {
+    if (p.M == 1) {
+        if (waves >= 16) launch_fused_jgn<1, GS, 16>(p, asym, out_bf16, stream);
+        else if (waves >= 8) launch_fused_jgn<1, GS, 8>(p, asym, out_bf16, stream);
+        else launch_fused_jgn<1, GS, 4>(p, asym, out_bf16, stream);
+    } else {
+        if (waves >= 16) launch_fused_jgn<4, GS, 16>(p, asym, out_bf16, stream);
+        else if (waves >= 8) launch_fused_jgn<4, GS, 8>(p, asym, out_bf16, stream);
+        else launch_fused_jgn<4, GS, 4>(p, asym, out_bf16, stream);
+    }
+}
+
+hipError_t launch_skinny_fused(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, hipStream_t stream) {
+    if (gs == 1) launch_fused_gs<1>(p, waves, asym, out_bf16, stream);
+    else if (gs == 2) launch_fused_gs<2>(p, waves, asym, out_bf16, stream);
+    else launch_fused_gs<4>(p, waves, asym, out_bf16, stream);
     return hipGetLastError();
 }
 

@@ -40,6 +40,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 
 struct GemmParams {
     const int8_t* q;        // [M][ldq]
+    const uint16_t* x;      // fused activation quantisation only: [M][ldx] fp16 / bf16 bits
     const float* s_a;       // [M]
     const int32_t* rowsum;  // [G][ldr]
     const uint32_t* w_r;    // repacked codes
@@ -50,6 +51,7 @@ struct GemmParams {
     float* ws_partial;      // split-K partial tiles
     unsigned* ws_counter;   // split-K arrival counters (zero between calls)
     int ldq, ldr, ldo;
+    int ldx, x_bf16;        // fused activation quantisation only
     int M, N, K;
     int G;                  // number of scale groups = K / group_size
     int steps;              // K / 64
@@ -62,6 +64,8 @@ struct GemmParams {
 
 // Problem table of a grouped skinny launch; passed by value in the kernel arguments (< 4 KiB).
 constexpr int kGroupedWavesPerWg = 8;  // wavefronts per workgroup of the grouped skinny kernel
+constexpr int kFusedMaxRows = 4;       // fused activation quantisation: at most this many token rows ...
+constexpr int kFusedMaxBytes = 32768;  // ... and rows x K int8 values (held in LDS)
 constexpr int kSharedParts = 2;  // k-parts per workgroup when one problem runs through the shared-activation workgroups
 constexpr int kMaxGroup = 24;
 struct GroupedParams {

@@ -27,6 +27,10 @@ hipError_t launch_read_probe(const void* src, size_t bytes, uint32_t* sink, hipS
 // gs = 64-element steps per scale group (1, 2 or 4); waves = wavefronts per workgroup (4, 8 or 16)
 hipError_t launch_skinny(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, hipStream_t stream);
 
+// the same kernel with the activation quantisation inside: p.x / p.ldx / p.x_bf16 instead of p.q, p.s_a, p.rowsum;
+// at most kFusedMaxRows token rows with rows x K <= kFusedMaxBytes
+hipError_t launch_skinny_fused(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, hipStream_t stream);
+
 // one problem of 17..32 token rows through the shared-activation workgroups (kSharedParts k-parts x
 // 8 / kSharedParts strips per workgroup, p.split K splits across workgroups)
 hipError_t launch_skinny_shared(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);

@@ -130,6 +130,15 @@ def test_repack_and_act_quant_validation(L):
     assert qw(FAKE, 4096, 0, 64, 4096, 128, 3, FAKE, 1024, FAKE, None, None) == 4      # mode
     assert qw(FAKE, 4100, 0, 64, 4096, 128, 1, FAKE, 1024, FAKE, None, None) == 3      # ldw % 8
     assert qw(FAKE, 4096, 0, 64, 4096, 128, 1, FAKE + 1, 1024, FAKE, None, None) == 3
+    # (x, ldx, dtype, w_r, s_r, zp_r, zp_const, M, N, K, group, out, ldo, out_dtype, ws, ws_bytes, split, stream)
+    gf = L.slimk_w2a8_gemm_fused
+    assert gf(None, 4096, 0, FAKE, FAKE, None, 2, 1, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 0, None) == 1
+    assert gf(FAKE, 4096, 0, FAKE, FAKE, None, 2, 5, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 0, None) == 7   # more than four rows
+    assert gf(FAKE, 16384, 0, FAKE, FAKE, None, 2, 4, 4096, 16384, 128, FAKE, 4096, 0, None, 0, 0, None) == 7  # rows x K > 32768
+    assert gf(FAKE, 4000, 0, FAKE, FAKE, None, 2, 1, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 0, None) == 2   # ldx < K
+    assert gf(FAKE, 4100, 0, FAKE, FAKE, None, 2, 1, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 0, None) == 3   # ldx % 8
+    assert gf(FAKE, 4096, 2, FAKE, FAKE, None, 2, 1, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 0, None) == 4
+    assert gf(FAKE, 14336, 0, FAKE, FAKE, None, 2, 1, 4096, 14336, 128, FAKE, 4096, 0, None, 0, 0, None) == 5  # wants split 4: no workspace
     assert L.slimk_w2a8_workspace_init(None, 64, None) == 1
     assert L.slimk_w2a8_workspace_init(FAKE, 0, None) == 0                             # nothing to do
     assert L.slimk_w2a8_read_probe(FAKE, 24, FAKE, None) == 3

@@ -374,3 +374,45 @@ def test_grouped_kernel_shape_classes(gpu_ops, oracle, g, mode, shapes):
     for (M, N, K), o, (ref, scales) in zip(shapes, outs, refs):
         pu.assert_out_close(pu.out_tensor_bits(o), ref["out_bits"], False,
                             pu.reorder_bound(ref["acc"], scales, ref["s_a"]), f"grouped {M}x{N}x{K} g{g} {mode}")
+
+
+# ------------------------------------------------------------------ activation quantisation inside the GEMM
+@pytest.mark.parametrize("M,N,K,g,mode,xdt,out,split", [
+    (1, 4096, 4096, 128, "sym", "float16", "float16", 0),
+    (1, 100, 256, 64, "asym", "bfloat16", "bfloat16", 0),
+    (2, 192, 14336, 128, "sym", "float16", "float16", 0),      # long K, few strips: K split across workgroups
+    (3, 640, 8192, 256, "asym", "float16", "bfloat16", 2),
+    (4, 1024, 8192, 64, "ref", "bfloat16", "float16", 1),
+    (4, 64, 2368, 64, "sym", "float16", "float16", 0),         # 37 steps: a ragged last chunk
+    (1, 5120, 28672, 64, "sym", "float16", "bfloat16", 0),
+])
+def test_fused_activation_quantisation_matches_two_launches(gpu_ops, oracle, M, N, K, g, mode, xdt, out, split):
+    """At most four token rows: slimk_w2a8_gemm_fused quantises the rows inside the GEMM kernel.  Same
+    bits as act-quant followed by the skinny kernel with the same split, and the oracle's output."""
+    _say("fused", M, N, K, g, mode, xdt, out, split)
+    case = pu.small_case(M, N, K, g, mode, seed=M + N + K, out_dtype=out)
+    packed, scales, zero = pu.quantized_weight(case)
+    x = workloads.make_activation(case)
+    w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, x)
+    if xdt == "bfloat16":
+        xd = xd.to(torch.bfloat16)
+        x = xd.float().cpu().numpy().astype(np.float32)
+    odt = pu.torch_dtype(case)
+    fused = gpu_ops.w2a8_linear_fused(xd, w, odt, split_k=split)
+    two = gpu_ops.w2a8_gemm(gpu_ops.quantize_act_int8(xd, g), w, odt, kernel="skinny", split_k=split)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(pu.out_tensor_bits(fused), pu.out_tensor_bits(two))
+    if xdt == "float16":
+        ref = oracle.reference_forward(x, packed, scales, zero, g, out_bf16=(out == "bfloat16"), want_acc=True)
+        pu.assert_out_close(pu.out_tensor_bits(fused), ref["out_bits"], out == "bfloat16",
+                            pu.reorder_bound(ref["acc"], scales, ref["s_a"]), case.name)
+    # a strided view of a wider buffer, and the layer's forward (which picks the fused path for few rows)
+    wide = torch.zeros(M, K + 16, dtype=xd.dtype, device="cuda")
+    wide[:, :K] = xd
+    np.testing.assert_array_equal(pu.out_tensor_bits(gpu_ops.w2a8_linear_fused(wide[:, :K], w, odt, split_k=split)),
+                                  pu.out_tensor_bits(fused))
+    lin = gpu_ops.W2A8Linear(w, None, odt)
+    np.testing.assert_array_equal(pu.out_tensor_bits(lin(xd)), pu.out_tensor_bits(
+        gpu_ops.w2a8_gemm(gpu_ops.quantize_act_int8(xd, g), w, odt)))
+    with pytest.raises(ValueError):
+        gpu_ops.w2a8_linear_fused(torch.zeros(5, K, dtype=xd.dtype, device="cuda"), w, odt)
