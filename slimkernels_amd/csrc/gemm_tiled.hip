@@ -9,6 +9,9 @@
 // What bounds the kernel is the vector ALU next to the matrix core, not the matrix core: every
 // accumulator must be drained into an fp32 running sum once per scale group (v_cvt_f32_i32 +
 // v_fma_f32 per element per group -- at group 128 that is as many VALU cycles as MFMA cycles).
+// Measured on one CU: a SIMD spends max(16, 8 + 4 V) cycles per v_mfma_i32_16x16x64_i8 that has V
+// vector instructions beside it (the MFMA holds the issue port for 8 cycles, a vector instruction
+// for 4); the main loop below has V = 5.3, so 0.55 of the matrix core is its ceiling.
 // Everything else is arranged to add as little VALU work as possible:
 //  * the high bit of every 2-bit field is flipped (one v_xor per dword) and the field moved to
 //    the top of its byte (v_lshlrev + v_and), so each operand byte reads as 64 * (code - 2):
