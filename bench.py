@@ -373,17 +373,45 @@ def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, d
                        "TOPS": round(nops / (us * 1e-6) / 1e12, 1), "frac_int8_mfma": round(nops / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4)})
     cache.clear()
     detail["other_configs"] = others
+
+    # ---- W4A8: 4-bit weights held as two 2-bit planes over a reduction of 2K (hi plane: scales 4s, zero-points
+    # zp >> 2; lo plane: scales s, zero-points zp & 3), the activation row laid down twice, one launch of the
+    # same kernels.  Timing on random codes in the streaming layout (parity: tests/test_w4a8.py).  Bytes are those
+    # of a 4-bit layout: N K / 2 + 2 N G (scales) + N G / 2 (4-bit zero-points) + M K + 4 M + 2 M N.
+    from slimkernels_amd.torch import w4 as tw4
+    w4rows = []
+    for (N, K, g, copies, Ms) in ((14336, 4096, 128, 12, (1, 16, 2048)), (28672, 8192, 128, 4, (1, 16))):
+        torch.cuda.empty_cache()
+        ws4 = [tw4.W4A8Weight(random_weight(N, 2 * K, g, True), N, K, g) for _ in range(copies)]
+        for M in Ms:
+            cold = M <= 16
+            use = ws4 if cold else ws4[:1] * 4
+            x = torch.randn(M, K, device=dev, dtype=torch.float16)
+            qa = ops.quantize_act_int8(x, g)
+            qa2 = tw4._twice(qa)
+            out = torch.empty((M, N), dtype=torch.float16, device=dev)
+            for w in (use if cold else use[:1]):
+                ops.w2a8_gemm(qa2, w.planes, torch.float16, out=out)
+            us = time_graph(torch, lambda: [ops.w2a8_gemm(qa2, w.planes, torch.float16, out=out) for w in use], len(use), replays=4)
+            G = K // g
+            nb = N * K // 2 + 2 * N * G + N * G // 2 + M * K + 4 * M + 2 * M * N
+            nops = 2 * M * N * K
+            w4rows.append({"shape": f"{N}x{K}", "M": M, "group": g, "weights": "cold" if cold else "warm", "us": round(us, 2),
+                           "GBps": round(nb / (us * 1e-6) / 1e9, 1), "frac_hbm": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                           "TOPS": round(nops / (us * 1e-6) / 1e12, 1), "frac_int8_mfma": round(nops / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4)})
+        del ws4
+    detail["w4a8"] = w4rows
     return detail
 
 
 def cpu_baseline(np, workloads, shapes):
-    """The reference CPU path on a bounded sample of the same workload: the four Llama linears at
-    M in {1, 16, 32}, through the oracle's torch-CPU-int-matmul restatement, on this box's host cores."""
+    """The reference CPU path on a bounded sample of the same workload: one step (the four Llama linears at
+    M in {1, 2, 4, 8, 16, 32}), through the oracle's torch-CPU-int-matmul restatement, on this box's host cores."""
     import torch
     from oracle import w2a8_oracle as orc
     torch.set_num_threads(min(16, os.cpu_count() or 1))
     tot_bytes, tot_s, c_port_s = 0, 0.0, 0.0
-    for name, M in [(n, m) for n in workloads.LLAMA8B_LINEARS for m in (1, 16, 32)]:
+    for name, M in [(n, m) for n in workloads.LLAMA8B_LINEARS for m in workloads.DECODE_M]:
         N, K = workloads.LLAMA8B_LINEARS[name]
         c = workloads.Case("c2", M, N, K, outliers=True)
         packed, scales, zero = shapes[name].host
@@ -398,8 +426,8 @@ def cpu_baseline(np, workloads, shapes):
         tot_bytes += workloads.algorithmic_bytes(c)
     return {"value": round(tot_bytes / tot_s / 1e9, 4), "unit": "GB/s", "cores": torch.get_num_threads(),
             "kind": "port",
-            "sample": "the four c2 shapes at M in {1,16,32} once each (act-quant + unpack + torch CPU int32 matmul per group + "
-                      "fp32 epilogue); algorithmic bytes / wall seconds",
+            "sample": "one step of the workload, once: the four c2 shapes at M in {1,2,4,8,16,32} (act-quant + unpack + torch CPU "
+                      "int32 matmul per group + fp32 epilogue); algorithmic bytes / wall seconds",
             "seconds": round(tot_s, 3), "host_cpus": os.cpu_count(),
             "scalar_c_port_1core_GBps": round(tot_bytes / c_port_s / 1e9, 4)}
 

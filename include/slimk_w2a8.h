@@ -31,6 +31,13 @@
  *
  * Shape limits: K % 64 == 0, group_size in {64, 128, 256}, K % group_size == 0.
  * M, N >= 1 are otherwise arbitrary (ragged tiles are handled inside).
+ *
+ * 4-bit weights (upstream: the notebook kernel w4matmul_splitk,
+ * slimkernels/triton/gemm_splitk.ipynb cell 0) need no entry point of their own:
+ * a code c = 4 * hi + lo is two 2-bit digits, and a W4 GEMM over K with G groups
+ * is these calls over K' = 2K with 2G groups -- columns 0..K-1 the hi digits with
+ * scales 4 * s and zero-points zp >> 2, columns K..2K-1 the lo digits with scales
+ * s and zero-points zp & 3 -- against q and its row sums laid down twice.
  */
 #ifndef SLIMK_W2A8_H
 #define SLIMK_W2A8_H

@@ -270,6 +270,62 @@ def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
     return ((u + 0x7FFF + lsb) >> 16).astype(np.uint16)
 
 
+# --------------------------------------------------------------------------- 4-bit weights
+# Upstream has no W4 quantiser (gemm_splitk.ipynb cell 0 multiplies by random packed codes); the level
+# sets below are this build's: "sym" levels -8..7 with s = absmax / 8, "asym" s = (max - min) / 15.
+# Pinned in tests/test_w4a8.py by closed forms, brute force on small inputs and the notebook's
+# unpack expression; parity with upstream is unpinned for want of an upstream definition.
+
+def np_pack_w4(codes: np.ndarray) -> np.ndarray:
+    """Two codes per byte along the row, first code in the high nibble."""
+    c = np.asarray(codes, np.uint8)
+    c2 = c.reshape(c.shape[0], -1, 2)
+    return ((c2[..., 0] << 4) | c2[..., 1]).astype(np.uint8)
+
+
+def np_unpack_w4(packed: np.ndarray) -> np.ndarray:
+    b = np.asarray(packed, np.uint8)
+    return np.stack([b >> 4, b & 15], axis=-1).reshape(b.shape[0], -1).astype(np.uint8)
+
+
+def np_unpack_uint32_kn(b: np.ndarray) -> np.ndarray:
+    """gemm_splitk.ipynb cell 0: code of element k is ``(b[k // 8, n] >> (k % 8) * 4) & 0xF``; returns [N, K]."""
+    b = np.asarray(b).astype(np.uint64)
+    K = b.shape[0] * 8
+    k = np.arange(K)
+    return ((b[k // 8, :] >> ((k % 8) * 4)[:, None].astype(np.uint64)) & 15).astype(np.uint8).T.copy()
+
+
+def np_quantize_w4(w_kn: np.ndarray, group_size: int, mode: str):
+    w = np.asarray(w_kn, np.float32)
+    K, N = w.shape
+    G = K // group_size
+    r = w.reshape(G, group_size, N)
+    one = np.float32
+    if mode == "sym":
+        s = np.maximum(np.abs(r).max(axis=1), one(1e-9)) / one(8.0)
+        zp = np.full((G, N), 8, np.float32)
+    elif mode == "asym":
+        mx, mn = r.max(axis=1), r.min(axis=1)
+        s = np.maximum(mx - mn, one(1e-9)) / one(15.0)
+        zp = np.clip(np.round(-mn / s), 0, 15).astype(np.float32)
+    else:
+        raise ValueError(mode)
+    s = s.astype(np.float32)
+    codes = np.clip(np.round(r / s[:, None, :]) + zp[:, None, :], 0, 15).astype(np.uint8)
+    return codes.reshape(K, N), s, zp.astype(np.uint8)
+
+
+def w4_reference_forward(x_half: np.ndarray, codes_nk: np.ndarray, scale_half: np.ndarray, zp: np.ndarray,
+                         group_size: int, out_bf16: bool = False):
+    """act-quant -> exact int32 per-group sums of q * (code - zp) -> the W2 path's epilogue
+    (t = fmaf(float(acc_g), scale[g, n], t) in ascending g, then * s_a, one cast)."""
+    q, s_a, rs = c_act_quant(x_half, group_size)
+    acc = np_gemm_acc_blas(q, np.asarray(codes_nk, np.uint8), np.asarray(zp, np.uint8), group_size)
+    out_bits, out_f32 = c_epilogue(acc, scale_half, s_a, out_bf16)
+    return dict(q=q, s_a=s_a, rowsum=rs, acc=acc, out_bits=out_bits, out_f32=out_f32)
+
+
 # --------------------------------------------------------------------------- whole-path helper
 
 def reference_forward(x_half: np.ndarray, packed: np.ndarray, scale_half: np.ndarray, zp: np.ndarray,

@@ -1,0 +1,129 @@
+"""W4A8 through the W2A8 kernels: a 4-bit weight is held as two 2-bit planes over a reduction of 2K
+(see slimkernels_amd/w4.py for the identity), the activation row is laid down twice, and every GEMM is one
+launch of the W2 kernels.  Upstream's only W4 code is the notebook kernel ``w4matmul_splitk(a, b, c)``
+(slimkernels/triton/gemm_splitk.ipynb cell 0); its call form is mirrored at the bottom."""
+from __future__ import annotations
+
+import dataclasses
+from typing import Optional
+
+import numpy as np
+import torch
+
+from .. import w4 as host_w4
+from .ops import (QuantizedActivation, W2A8Weight, _DT, _require_cuda, fused_applies, quantize_act_int8, repack_w2,
+                  w2a8_gemm, w2a8_linear_fused)
+
+
+@dataclasses.dataclass
+class W4A8Weight:
+    """A 4-bit weight [N, K] as the W2 operand over 2K (hi plane, then lo plane)."""
+    planes: W2A8Weight
+    N: int
+    K: int
+    group_size: int
+
+    @property
+    def device(self):
+        return self.planes.device
+
+
+def repack_w4(packed4, scales, zp=None, group_size: int = 128, zp_const: int = 8, device="cuda") -> W4A8Weight:
+    """packed4: uint8 [N, K/2] (pack_w4 layout), scales: float16 [G, N], zp: uint8 [G, N] with values 0..15 or
+    None for a uniform zero-point ``zp_const`` (8: the symmetric levels -8..7).  numpy arrays or tensors."""
+    packed4 = packed4.cpu().numpy() if isinstance(packed4, torch.Tensor) else np.asarray(packed4)
+    scales = scales.cpu().numpy() if isinstance(scales, torch.Tensor) else np.asarray(scales)
+    if packed4.dtype != np.uint8 or packed4.ndim != 2:
+        raise ValueError("packed4 must be a 2-D uint8 array [N, K/2]")
+    N, K = packed4.shape[0], packed4.shape[1] * 2
+    if scales.dtype != np.float16 or scales.ndim != 2 or K % group_size != 0 or scales.shape != (K // group_size, N):
+        raise ValueError(f"scales must be float16 [K/group_size, N] = {(K // max(group_size, 1), N)}")
+    if zp is None:
+        if not 0 <= int(zp_const) <= 15:
+            raise ValueError("zp_const must be in 0..15")
+        zp = np.full(scales.shape, int(zp_const), dtype=np.uint8)
+    else:
+        zp = zp.cpu().numpy() if isinstance(zp, torch.Tensor) else np.asarray(zp)
+    packed2, scales2, zp2 = host_w4.split_planes(host_w4.unpack_w4(packed4), scales, zp)
+    return W4A8Weight(repack_w2(packed2, scales2, zp2, group_size, device=device), N, K, group_size)
+
+
+def _twice(qa: QuantizedActivation) -> QuantizedActivation:
+    """The activation operand over 2K: the int8 row and its per-group sums laid down twice."""
+    return QuantizedActivation(torch.cat([qa.q, qa.q], dim=1), qa.s_a, torch.cat([qa.rowsum, qa.rowsum], dim=0),
+                               qa.group_size)
+
+
+def w4a8_gemm(qa: QuantizedActivation, w: W4A8Weight, out_dtype=torch.float16, *, kernel: str = "auto",
+              split_k: int = 0, dump: Optional[str] = None, out: Optional[torch.Tensor] = None):
+    """out[M, N] = dequant( q @ (codes4 - zp4)^T ) for ``qa`` = quantize_act_int8(x) over K.  With ``dump`` =
+    "groups" also returns the int32 accumulators [M, N, G] (4 * hi-plane + lo-plane sums, exact)."""
+    M, K = qa.q.shape
+    if K != w.K or qa.group_size != w.group_size:
+        raise ValueError(f"activation K={K}/group {qa.group_size} does not match weight K={w.K}/group {w.group_size}")
+    if dump not in (None, "groups"):
+        raise ValueError("dump must be None or 'groups'")
+    res = w2a8_gemm(_twice(qa), w.planes, out_dtype, kernel=kernel, split_k=split_k, dump=dump, out=out)
+    if dump is None:
+        return res
+    y, acc = res
+    G = K // w.group_size
+    return y, acc[:, :, :G] * 4 + acc[:, :, G:]
+
+
+def w4a8_linear(x: torch.Tensor, w: W4A8Weight, out_dtype=torch.float16) -> torch.Tensor:
+    """x [M, K] fp16 / bf16 -> out [M, N]; one token row goes through the single-launch kernel that quantises
+    the row itself."""
+    _require_cuda(x, "x")
+    if x.dim() != 2 or x.dtype not in _DT:
+        raise ValueError("x must be a 2-D float16 or bfloat16 tensor [M, K]")
+    if x.shape[1] != w.K:
+        raise ValueError(f"activation K={x.shape[1]} does not match weight K={w.K}")
+    if x.shape[0] == 1 and fused_applies(1, 2 * w.K):
+        return w2a8_linear_fused(torch.cat([x, x], dim=1), w.planes, out_dtype)
+    return w4a8_gemm(quantize_act_int8(x, w.group_size), w, out_dtype)
+
+
+class W4A8Linear(torch.nn.Module):
+    """y = x @ W^T with W held as 4-bit codes (+ optional bias), a swap-in for nn.Linear."""
+
+    def __init__(self, weight: W4A8Weight, bias: Optional[torch.Tensor] = None, out_dtype=torch.float16):
+        super().__init__()
+        self.weight = weight
+        self.bias = bias
+        self.out_dtype = out_dtype
+        self.in_features, self.out_features = weight.K, weight.N
+
+    @classmethod
+    def from_float(cls, weight_nk, group_size=128, mode="sym", bias=None, out_dtype=torch.float16, device="cuda"):
+        w_np = weight_nk.detach().float().cpu().numpy() if isinstance(weight_nk, torch.Tensor) else np.asarray(weight_nk)
+        packed4, scales, zero = host_w4.prepare_w4(w_np, group_size, mode)
+        return cls(repack_w4(packed4, scales, zero, group_size, device=device), bias, out_dtype)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, x.shape[-1])
+        if x2.dtype not in _DT:
+            x2 = x2.to(self.out_dtype)
+        y = w4a8_linear(x2, self.weight, self.out_dtype)
+        if self.bias is not None:
+            y = y + self.bias
+        return y.reshape(*lead, self.out_features)
+
+
+def w4matmul_splitk(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor) -> torch.Tensor:
+    """The call form of the upstream notebook kernel (gemm_splitk.ipynb cell 0): ``a`` [M, K] fp16, ``b`` the
+    packed weight [K/8, N] (eight 4-bit codes per 32-bit word along K, code k % 8 at bits 4 * (k % 8)),
+    ``c`` [M, N] fp16, which receives ``c += a @ codes`` -- the raw codes 0..15 are the weight values, there
+    are no scales and no zero-point.  Here the product runs as W4A8 (``a`` is quantised per token row to int8),
+    so it agrees with the fp16 product to the activation quantisation error.  Repacks on every call."""
+    _require_cuda(a, "a")
+    codes = host_w4.codes_from_uint32_kn(b.cpu().numpy() if isinstance(b, torch.Tensor) else b)   # [N, K]
+    N, K = codes.shape
+    if a.shape[1] != K or tuple(c.shape) != (a.shape[0], N):
+        raise ValueError(f"shapes do not agree: a {tuple(a.shape)}, b unpacks to K={K}, N={N}, c {tuple(c.shape)}")
+    group = 128 if K % 128 == 0 else 64
+    ones = np.ones((K // group, N), dtype=np.float16)
+    w = repack_w4(host_w4.pack_w4(codes), ones, None, group, zp_const=0, device=a.device)
+    c += w4a8_linear(a if a.dtype in _DT else a.half(), w, c.dtype if c.dtype in _DT else torch.float16).to(c.dtype)
+    return c

@@ -1,0 +1,202 @@
+"""W4A8: 4-bit weights run as two 2-bit planes through the W2A8 kernels.
+
+Upstream's W4 code is one notebook kernel on random packed integers (slimkernels/triton/gemm_splitk.ipynb
+cell 0) with no quantiser and no tests, so there are no upstream vectors to carry over: the host functions
+are pinned by hand-computed cases, closed forms, brute force and the notebook's unpack expression, and the GPU
+path by the oracle's exact integer sums and its epilogue (the tolerance of the W2 path, written in
+parity_utils.assert_out_close: 1 ULP of the output type or rtol 1e-3, plus the fp32 re-association bound)."""
+import numpy as np
+import pytest
+import torch
+
+from slimkernels_amd import w4
+import parity_utils as pu
+
+
+# ---------------------------------------------------------------- host format and quantiser (CPU)
+
+def test_pack_w4_known_answer_and_round_trip():
+    codes = np.array([[1, 2, 15, 0], [8, 8, 3, 12]], dtype=np.uint8)
+    packed = w4.pack_w4(codes)
+    np.testing.assert_array_equal(packed, np.array([[0x12, 0xF0], [0x88, 0x3C]], dtype=np.uint8))
+    np.testing.assert_array_equal(w4.unpack_w4(packed), codes)
+    every = np.arange(256, dtype=np.uint8).reshape(1, 256)
+    np.testing.assert_array_equal(w4.pack_w4(w4.unpack_w4(every)), every)
+
+
+def test_pack_w4_rejects_bad_input():
+    with pytest.raises(ValueError):
+        w4.pack_w4(np.zeros((2, 4), dtype=np.int32))
+    with pytest.raises(ValueError):
+        w4.pack_w4(np.zeros((2, 3), dtype=np.uint8))
+    with pytest.raises(ValueError):
+        w4.pack_w4(np.full((2, 4), 16, dtype=np.uint8))
+
+
+def test_uint32_operand_of_the_notebook(oracle):
+    rng = np.random.default_rng(0)
+    b = rng.integers(0, 2**32, size=(4, 5), dtype=np.uint64).astype(np.uint32)   # K = 32, N = 5
+    codes = w4.codes_from_uint32_kn(b)
+    assert codes.shape == (5, 32) and codes.dtype == np.uint8
+    for n in range(5):           # the notebook's expression, element by element
+        for k in range(32):
+            assert codes[n, k] == (int(b[k // 8, n]) >> ((k % 8) * 4)) & 0xF
+    np.testing.assert_array_equal(codes, oracle.np_unpack_uint32_kn(b))
+    np.testing.assert_array_equal(w4.codes_from_uint32_kn(b.view(np.int32)), codes)   # signed storage, same bits
+
+
+def test_quantize_w4_sym_closed_form():
+    # one group of 8 rows, two columns; absmax 4 -> s = 0.5, codes = rne(w / 0.5) + 8 clipped to 0..15
+    col0 = np.array([-4.0, -3.75, -0.25, 0.0, 0.25, 0.75, 3.4, 4.0], dtype=np.float32)
+    col1 = col0[::-1] * 2
+    codes, scales, zp = w4.quantize_w4(np.stack([col0, col1], axis=1), group_size=8, mode="sym")
+    np.testing.assert_array_equal(scales, np.array([[0.5, 1.0]], dtype=np.float32))
+    np.testing.assert_array_equal(zp, np.array([[8, 8]], dtype=np.uint8))
+    # -4 -> 0; -3.75/0.5 = -7.5 -> -8 (ties to even) -> 0; -0.25/0.5 = -0.5 -> -0 -> 8; 0.25/0.5 = 0.5 -> 0 -> 8;
+    # 0.75/0.5 = 1.5 -> 2 -> 10; 3.4/0.5 = 6.8 -> 7 -> 15; 4/0.5 = 8 -> 16 clipped to 15
+    np.testing.assert_array_equal(codes[:, 0], np.array([0, 0, 8, 8, 8, 10, 15, 15], dtype=np.uint8))
+    np.testing.assert_array_equal(codes[:, 1], codes[::-1, 0])
+
+
+@pytest.mark.parametrize("mode", ["sym", "asym"])
+def test_quantize_w4_against_brute_force_and_the_oracle(oracle, mode):
+    rng = np.random.default_rng(3)
+    w = (rng.standard_normal((64, 6)) * 0.05).astype(np.float32)
+    w[5, 2] = 0.0
+    codes, scales, zp = w4.quantize_w4(w, group_size=16, mode=mode)
+    oc, os_, oz = oracle.np_quantize_w4(w, 16, mode)
+    np.testing.assert_array_equal(codes, oc)
+    np.testing.assert_array_equal(scales, os_)
+    np.testing.assert_array_equal(zp, oz)
+    for g in range(4):           # scalar restatement, element by element
+        for n in range(6):
+            col = w[16 * g:16 * g + 16, n]
+            if mode == "sym":
+                s = np.float32(max(np.abs(col).max(), np.float32(1e-9))) / np.float32(8.0)
+                z = 8
+            else:
+                s = np.float32(max(col.max() - col.min(), np.float32(1e-9))) / np.float32(15.0)
+                z = int(np.clip(np.round(np.float32(-col.min()) / s), 0, 15))
+            assert scales[g, n] == s and zp[g, n] == z
+            for i, v in enumerate(col):
+                assert codes[16 * g + i, n] == int(np.clip(np.round(np.float32(v) / s) + z, 0, 15))
+    # every level is within half a step of the value it stands for, inside the clip range
+    deq = (codes.astype(np.float32).reshape(4, 16, 6) - zp[:, None, :]) * scales[:, None, :]
+    inside = (codes > 0) & (codes < 15)
+    assert np.all(np.abs(deq.reshape(64, 6) - w)[inside] <= np.repeat(scales, 16, axis=0)[inside] * 0.5 + 1e-9)
+
+
+def test_split_planes_identity():
+    rng = np.random.default_rng(5)
+    N, K, g = 7, 256, 64
+    codes = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    scales = (rng.random((K // g, N)) * 0.01 + 0.001).astype(np.float16)
+    zp = rng.integers(0, 16, size=(K // g, N), dtype=np.uint8)
+    packed2, scales2, zp2 = w4.split_planes(codes, scales, zp)
+    from slimkernels_amd import unpack_matrix
+    planes = unpack_matrix(packed2)
+    assert planes.shape == (N, 2 * K) and scales2.shape == (2 * K // g, N) and zp2.max() <= 3
+    np.testing.assert_array_equal(planes[:, :K].astype(np.int32) * 4 + planes[:, K:], codes)
+    np.testing.assert_array_equal(zp2[:K // g].astype(np.int32) * 4 + zp2[K // g:], zp)
+    np.testing.assert_array_equal(scales2[K // g:], scales)
+    np.testing.assert_array_equal(scales2[:K // g].astype(np.float32), scales.astype(np.float32) * 4)
+    # the identity the GPU path rests on, on integers: sum q (c - zp) = 4 sum q (hi - zh) + sum q (lo - zl)
+    q = rng.integers(-127, 128, size=(3, K)).astype(np.int64)
+    for gi in range(K // g):
+        ks = slice(gi * g, (gi + 1) * g)
+        want = q[:, ks] @ (codes[:, ks].astype(np.int64) - zp[gi][:, None]).T
+        hi = q[:, ks] @ (planes[:, :K][:, ks].astype(np.int64) - zp2[gi][:, None]).T
+        lo = q[:, ks] @ (planes[:, K:][:, ks].astype(np.int64) - zp2[K // g + gi][:, None]).T
+        np.testing.assert_array_equal(4 * hi + lo, want)
+    with pytest.raises(ValueError, match="overflows"):
+        w4.split_planes(codes, np.full_like(scales, 30000.0), zp)
+
+
+# ---------------------------------------------------------------- the GPU path
+
+def _plane_bound(oracle, ref, codes, scales, zp, g):
+    """The fp32 re-association bound of the sum as the GPU forms it: 2G terms per output, the hi-plane sums
+    times 4 * scale and the lo-plane sums times scale (a plane's term can be larger than their sum)."""
+    hi = oracle.np_gemm_acc_blas(ref["q"], codes >> 2, zp >> 2, g)
+    lo = oracle.np_gemm_acc_blas(ref["q"], codes & 3, zp & 3, g)
+    np.testing.assert_array_equal(4 * hi + lo, ref["acc"])
+    return pu.reorder_bound(np.concatenate([4 * hi, lo], axis=2), np.concatenate([scales, scales], axis=0), ref["s_a"])
+
+
+def _w4_case(M, N, K, g, mode, seed, outliers=False):
+    rng = np.random.default_rng(seed)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32) if mode == "sym" else \
+        rng.uniform(-0.05, 0.05, size=(N, K)).astype(np.float32)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    if outliers:
+        x[:, rng.choice(K, max(1, K // 1000), replace=False)] *= 20
+    return w, x.astype(np.float16)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K,g,mode,out,kernel", [
+    (1, 256, 512, 128, "sym", "float16", "auto"),
+    (5, 192, 256, 64, "asym", "float16", "skinny"),
+    (16, 4096, 4096, 128, "sym", "float16", "auto"),
+    (32, 1024, 2048, 128, "asym", "bfloat16", "auto"),
+    (77, 320, 1024, 128, "asym", "float16", "tiled"),
+    (256, 512, 1024, 128, "sym", "bfloat16", "auto"),
+])
+def test_w4a8_gemm_against_the_oracle(gpu_ops, oracle, M, N, K, g, mode, out, kernel):
+    from slimkernels_amd.torch import w4 as tw4
+    print(f"W4A8 M={M} N={N} K={K} g={g} {mode} {out} {kernel}", flush=True)
+    w, x = _w4_case(M, N, K, g, mode, seed=M + N)
+    packed4, scales, zp = w4.prepare_w4(w, g, mode)
+    codes = w4.unpack_w4(packed4)
+    bf16 = out == "bfloat16"
+    ref = oracle.w4_reference_forward(x, codes, scales, zp, g, bf16)
+    wd = tw4.repack_w4(packed4, scales, zp, g)
+    qa = gpu_ops.quantize_act_int8(torch.from_numpy(x).cuda(), g)
+    np.testing.assert_array_equal(qa.q.cpu().numpy(), ref["q"])
+    odt = torch.bfloat16 if bf16 else torch.float16
+    y, acc = tw4.w4a8_gemm(qa, wd, odt, kernel=kernel, dump="groups")
+    np.testing.assert_array_equal(acc.cpu().numpy(), ref["acc"])          # int32 sums: exact
+    y2 = tw4.w4a8_gemm(qa, wd, odt, kernel=kernel)
+    bound = _plane_bound(oracle, ref, codes, scales, zp, g)
+    for t, what in ((y, "with dump"), (y2, "production kernels")):
+        pu.assert_out_close(pu.out_tensor_bits(t), ref["out_bits"], bf16, bound, f"W4A8 {what}")
+
+
+@pytest.mark.gpu
+def test_w4a8_linear_and_decode_row(gpu_ops, oracle):
+    from slimkernels_amd.torch import w4 as tw4
+    w, x = _w4_case(3, 384, 1024, 128, "sym", seed=11)
+    lin = tw4.W4A8Linear.from_float(w, 128, "sym")
+    packed4, scales, zp = w4.prepare_w4(w, 128, "sym")
+    xd = torch.from_numpy(x).cuda()
+    codes = w4.unpack_w4(packed4)
+    ref = oracle.w4_reference_forward(x, codes, scales, zp, 128)
+    bound = _plane_bound(oracle, ref, codes, scales, zp, 128)
+    y = lin(xd.reshape(1, 3, 1024))
+    assert y.shape == (1, 3, 384)
+    pu.assert_out_close(pu.out_tensor_bits(y.reshape(3, 384)), ref["out_bits"], False, bound, "W4A8Linear")
+    # one row: the single-launch kernel that quantises the row itself
+    ref1 = oracle.w4_reference_forward(x[:1], codes, scales, zp, 128)
+    y1 = lin(xd[:1])
+    pu.assert_out_close(pu.out_tensor_bits(y1), ref1["out_bits"], False,
+                        _plane_bound(oracle, ref1, codes, scales, zp, 128), "W4A8Linear one row")
+
+
+@pytest.mark.gpu
+def test_w4matmul_splitk_call_form(gpu_ops):
+    """c += a @ codes with the notebook's operand layout; against the fp32 product of the same operands the
+    only difference is the int8 quantisation of a (|error| <= s_a / 2 per element of a)."""
+    from slimkernels_amd.torch import w4 as tw4
+    rng = np.random.default_rng(2)
+    M, N, K = 4, 64, 256
+    a = rng.standard_normal((M, K)).astype(np.float16)
+    b = rng.integers(0, 2**32, size=(K // 8, N), dtype=np.uint64).astype(np.uint32)
+    codes = w4.codes_from_uint32_kn(b).astype(np.float32)                 # [N, K]
+    c0 = rng.standard_normal((M, N)).astype(np.float16)
+    c = torch.from_numpy(c0.copy()).cuda()
+    out = tw4.w4matmul_splitk(torch.from_numpy(a).cuda(), torch.from_numpy(b.view(np.int32)), c)
+    assert out is c
+    want = c0.astype(np.float32) + a.astype(np.float32) @ codes.T
+    s_a = np.abs(a.astype(np.float32)).max(axis=1) / 127
+    tol = (s_a / 2)[:, None] * codes.sum(axis=1)[None, :] + 1e-3 * np.abs(want) + 0.26   # + fp16 rounding of c (|c| < 512)
+    assert np.all(np.abs(c.float().cpu().numpy() - want) <= tol)
