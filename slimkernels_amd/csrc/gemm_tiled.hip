@@ -460,12 +460,16 @@ int tiled_fast_max_split(int M, int strips, int steps) {
 // about two workgroups per CU exist.  Measured: a workgroup alone on a CU spends about 0.7 us per
 // 128-element stage and two on a CU about 1.25 us for both; a split costs the reducing workgroup
 // about a microsecond plus 0.8 us per partial tile it reads.  Hence up to eight splits, each at
-// least eight stages (K >= 1024 per split) long; with more tiles than that a split gains nothing.
+// least eight stages (K >= 1024 per split) long; with more tiles than that a split gains nothing
+// unless the reduction is long.
 int tiled_fast_auto_split(int M, int strips, int steps) {
     int bm, tiles;
     tiled_fast_tiles(M, strips, &bm, &tiles);
-    if (bm != 64 || steps % fast::kStageSteps != 0 || tiles > 128) return 1;
+    if (bm != 64 || steps % fast::kStageSteps != 0) return 1;
     const int stages = steps / fast::kStageSteps;
+    // one workgroup per CU on most CUs and a long reduction: two halves (measured at 128 x 28672 x 8192,
+    // 224 tiles of 64 stages: 67.5 -> 61.2 us; at 32 stages per tile the halves are slower: 28.1 -> 31.6 us)
+    if (tiles > 128) return tiles <= 256 && stages >= 64 ? 2 : 1;
     int split = 512 / tiles;
     if (split > 8) split = 8;
     if (split > stages / 8) split = stages / 8;
