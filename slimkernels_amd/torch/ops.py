@@ -69,8 +69,13 @@ def repack_w2(packed, scales, zp=None, group_size: int = 128, zp_const: int = 2,
     zp: uint8 [G, N] or None for a uniform zero-point ``zp_const``.  numpy arrays or tensors."""
     L = _lib.lib()
     dev = torch.device(device)
-    packed_t = torch.as_tensor(np.ascontiguousarray(packed) if isinstance(packed, np.ndarray) else packed)
-    scales_t = torch.as_tensor(np.ascontiguousarray(scales) if isinstance(scales, np.ndarray) else scales)
+    def host(a):  # torch wants writable memory under a tensor: a read-only array (a mapped file) is copied
+        if not isinstance(a, np.ndarray):
+            return a
+        a = np.ascontiguousarray(a)
+        return a if a.flags.writeable else a.copy()
+    packed_t = torch.as_tensor(host(packed))
+    scales_t = torch.as_tensor(host(scales))
     if packed_t.dtype != torch.uint8 or packed_t.dim() != 2:
         raise ValueError("packed must be a 2-D uint8 array [N, K/4]")
     if scales_t.dtype != torch.float16 or scales_t.dim() != 2:
@@ -83,7 +88,7 @@ def repack_w2(packed, scales, zp=None, group_size: int = 128, zp_const: int = 2,
     scales_d = scales_t.to(dev).contiguous()
     zp_d = None
     if zp is not None:
-        zp_t = torch.as_tensor(np.ascontiguousarray(zp) if isinstance(zp, np.ndarray) else zp)
+        zp_t = torch.as_tensor(host(zp))
         if zp_t.dtype != torch.uint8 or tuple(zp_t.shape) != tuple(scales_t.shape):
             raise ValueError("zp must be uint8 with the shape of scales")
         zp_d = zp_t.to(dev).contiguous()
