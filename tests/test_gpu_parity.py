@@ -76,7 +76,11 @@ def test_weight_quantisation_on_gpu_bit_exact(gpu_ops, N, K, g, mode, bf16):
 @pytest.mark.parametrize("M,K,g,bf16,outliers", [(1, 4096, 128, False, True), (16, 4096, 128, False, True),
                                                  (77, 4096, 128, False, False), (3, 13824, 128, False, False),
                                                  (5, 8192, 64, True, False), (33, 256, 256, False, False),
-                                                 (2, 64, 64, False, False)])
+                                                 (2, 64, 64, False, False),
+                                                 # many rows, long rows, odd row counts
+                                                 (64, 4096, 128, False, True), (77, 8192, 64, True, False),
+                                                 (130, 14336, 128, False, True), (67, 192, 64, False, False),
+                                                 (65, 6144, 256, True, False), (66, 16448, 64, False, False)])
 def test_act_quant_bit_exact(gpu_ops, oracle, M, K, g, bf16, outliers):
     _say("act_quant", M, K, g, bf16)
     case = pu.small_case(M, 64, K, g, "sym", seed=M * 7 + K, outliers=outliers)
