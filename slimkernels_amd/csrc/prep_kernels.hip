@@ -71,6 +71,21 @@ hipError_t launch_repack(const uint8_t* w_packed, int ldw, const uint16_t* scale
 // per-group sums of q, all with IEEE binary32 division (this file is compiled
 // without fast-math).  Each thread handles 8 consecutive elements (one 16-byte load).
 template <bool BF16>
+__device__ __forceinline__ void widen8(const uint4& raw, float (&v)[8]) {
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (BF16) {
+            v[2 * i] = __uint_as_float(w[i] << 16);
+            v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        } else {
+            v[2 * i] = half_bits_to_float((uint16_t)(w[i] & 0xffffu));
+            v[2 * i + 1] = half_bits_to_float((uint16_t)(w[i] >> 16));
+        }
+    }
+}
+
+template <bool BF16>
 __device__ __forceinline__ void load8(const uint16_t* p, float (&v)[8]) {
     const uint4 raw = *reinterpret_cast<const uint4*>(p);
     const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
@@ -142,8 +157,87 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
     }
 }
 
+// The same with the row read once: a thread keeps its KEEP 16-byte vectors (K <= 2048 * KEEP) in registers
+// between the absmax pass and the quantising pass, all of its loads in flight together.  With many rows the
+// two-pass kernel moves every row twice (the second time from L2) in phases that the workgroups of a round
+// go through together; this one moves it once.  Same arithmetic per element: bit-identical results.
+template <bool BF16, int KEEP>
+__global__ __launch_bounds__(256) void act_quant_keep_kernel(const uint16_t* __restrict__ x, int ldx, int K,
+                                                             int group_size, int8_t* __restrict__ q, int ldq,
+                                                             float* __restrict__ s_a,
+                                                             int32_t* __restrict__ rowsum, int ldr) {
+    __shared__ float red[4];
+    const int m = blockIdx.x;
+    const int tid = threadIdx.x;
+    const uint16_t* xr = x + (size_t)m * ldx;
+    const int nvec = K / 8;
+    uint4 raw[KEEP];
+#pragma unroll
+    for (int it = 0; it < KEEP; ++it) {
+        const int v = it * 256 + tid;
+        raw[it] = v < nvec ? *reinterpret_cast<const uint4*>(xr + (size_t)v * 8) : make_uint4(0, 0, 0, 0);
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int it = 0; it < KEEP; ++it) {
+        float f[8];
+        widen8<BF16>(raw[it], f);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(f[i]));
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    if ((tid & 63) == 0) red[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const float s = fmaxf(amax, 1e-9f) / 127.0f;
+    if (tid == 0) s_a[m] = s;
+
+    const int tpg = group_size / 8;  // threads per scale group: 8, 16 or 32
+    int8_t* qr = q + (size_t)m * ldq;
+#pragma unroll
+    for (int it = 0; it < KEEP; ++it) {
+        const int v = it * 256 + tid;
+        int sum = 0;
+        if (v < nvec) {
+            float f[8];
+            widen8<BF16>(raw[it], f);
+            uint32_t lo = 0, hi = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float r = rintf(f[i] / s);
+                r = fminf(fmaxf(r, -127.0f), 127.0f);
+                const int qi = (int)r;
+                sum += qi;
+                if (i < 4) lo |= (uint32_t)(qi & 0xff) << (8 * i);
+                else hi |= (uint32_t)(qi & 0xff) << (8 * (i - 4));
+            }
+            *reinterpret_cast<uint2*>(qr + (size_t)v * 8) = make_uint2(lo, hi);
+        }
+        for (int off = 1; off < tpg; off <<= 1) sum += __shfl_xor(sum, off, 64);
+        if (rowsum && v < nvec && (v % tpg) == 0) rowsum[(size_t)(v / tpg) * ldr + m] = sum;
+    }
+}
+
+template <bool BF16>
+static void launch_act_quant_keep(const void* x, int ldx, int M, int K, int group_size, int8_t* q, int ldq, float* s_a,
+                                  int32_t* rowsum, int ldr, hipStream_t stream) {
+    const dim3 grid((unsigned)M), block(256);
+    if (K <= 4096)
+        act_quant_keep_kernel<BF16, 2><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr);
+    else if (K <= 8192)
+        act_quant_keep_kernel<BF16, 4><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr);
+    else
+        act_quant_keep_kernel<BF16, 8><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr);
+}
+
 hipError_t launch_act_quant(const void* x, int ldx, bool x_bf16, int M, int K, int group_size,
                             int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, hipStream_t stream) {
+    if (K <= 16384) {
+        if (x_bf16) launch_act_quant_keep<true>(x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, stream);
+        else launch_act_quant_keep<false>(x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, stream);
+        return hipGetLastError();
+    }
     if (x_bf16)
         act_quant_kernel<true><<<dim3(M), dim3(256), 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q,
                                                                  ldq, s_a, rowsum, ldr);
