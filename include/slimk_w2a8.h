@@ -216,6 +216,8 @@ typedef struct slimk_w2a8_problem {
  * kernel arguments (so the call is graph-capturable and the array may be reused at once).
  * All problems share group_size and out_dtype, and either all carry per-group zero-points
  * (zp_r non-NULL) or none does (each then uses its own zp_const); M, N, K may differ.
+ * The order of the entries is the caller's to choose: inside the launch the problems run longest
+ * reduction first and, among equal reductions, most token rows first.
  * No split-K, no workspace.  A launch too small to cover the chip splits its longest reductions
  * further inside the workgroups; a lone problem that slimk_w2a8_gemm would run unsplit is handed
  * to that kernel (faster for one problem).
