@@ -11,16 +11,21 @@ from typing import Callable, Iterable, List, Optional
 import torch
 
 from .ops import W2A8Linear
+from .w4 import W4A8Linear
 
 
 def replace_linears(model: torch.nn.Module, group_size: int = 128, mode: str = "sym",
                     skip: Iterable[str] = ("lm_head",), out_dtype=None,
-                    predicate: Optional[Callable[[str, torch.nn.Linear], bool]] = None) -> List[str]:
-    """Replace every eligible ``nn.Linear`` under ``model`` by a ``W2A8Linear`` and return the dotted names
+                    predicate: Optional[Callable[[str, torch.nn.Linear], bool]] = None, bits: int = 2) -> List[str]:
+    """Replace every eligible ``nn.Linear`` under ``model`` by a ``W2A8Linear`` (``bits=2``) or a ``W4A8Linear``
+    (``bits=4``: modes "sym" and "asym", quantised on the host) and return the dotted names
     of the layers replaced.  Eligible: ``in_features`` a multiple of ``group_size``, the last name component
     not in ``skip`` (the output head stays in floating point by default), and ``predicate(name, layer)`` true
     when one is given.  ``out_dtype`` defaults to the dtype of each layer's weight (fp16 or bf16; other dtypes
     give fp16).  The model must already be on the GPU: the layers are built on the device of their weight."""
+    if bits not in (2, 4):
+        raise ValueError("bits must be 2 or 4")
+    layer_type = W2A8Linear if bits == 2 else W4A8Linear
     skip = set(skip)
     done = []
     for parent_name, parent in list(model.named_modules()):
@@ -37,6 +42,6 @@ def replace_linears(model: torch.nn.Module, group_size: int = 128, mode: str = "
                 raise ValueError(f"{name}: move the model to the GPU before replace_linears (weight is on {w.device})")
             dt = out_dtype or (w.dtype if w.dtype in (torch.float16, torch.bfloat16) else torch.float16)
             bias = child.bias.detach().to(dt) if child.bias is not None else None
-            setattr(parent, child_name, W2A8Linear.from_float(w, group_size, mode, bias=bias, out_dtype=dt))
+            setattr(parent, child_name, layer_type.from_float(w, group_size, mode, bias=bias, out_dtype=dt, device=w.device))
             done.append(name)
     return done

@@ -22,17 +22,19 @@ def _tiny_llama():
     return transformers.LlamaForCausalLM(cfg).eval()
 
 
-def _dequantised_copy(model, names, group_size):
-    """The model with each listed linear's weight replaced by what its 2-bit codes and fp16 scales stand for."""
+def _dequantised_copy(model, names, group_size, bits=2):
+    """The model with each listed linear's weight replaced by what its 2- or 4-bit codes and fp16 scales stand for."""
     from slimkernels_amd.quantization import quantize_w2
+    from slimkernels_amd.w4 import quantize_w4
     ref = copy.deepcopy(model)
     mods = dict(ref.named_modules())
     for name in names:
         lin = mods[name]
         w = lin.weight.detach().float().cpu().numpy()                 # [N, K]
-        codes, scales, _ = quantize_w2(np.ascontiguousarray(w.T), group_size, "sym")   # [K, N], [G, N]
+        quantise, zero = (quantize_w2, 2.0) if bits == 2 else (quantize_w4, 8.0)
+        codes, scales, _ = quantise(np.ascontiguousarray(w.T), group_size, "sym")   # [K, N], [G, N]
         s16 = scales.astype(np.float16).astype(np.float32)
-        deq = (codes.astype(np.float32) - 2.0).reshape(-1, group_size, w.shape[0]) * s16[:, None, :]
+        deq = (codes.astype(np.float32) - zero).reshape(-1, group_size, w.shape[0]) * s16[:, None, :]
         lin.weight.data = torch.from_numpy(np.ascontiguousarray(deq.reshape(w.shape[1], w.shape[0]).T)).to(lin.weight)
     return ref
 
@@ -59,13 +61,15 @@ def test_replace_linears_skips_what_it_cannot_take():
 
 
 @pytest.mark.gpu
-def test_llama_block_with_w2a8_linears(gpu_ops):
+@pytest.mark.parametrize("bits", [2, 4])
+def test_llama_block_with_w2a8_linears(gpu_ops, bits):
     model = _tiny_llama().half().cuda()
     quant = copy.deepcopy(model)
-    names = gpu_ops.replace_linears(quant, group_size=128)
+    names = gpu_ops.replace_linears(quant, group_size=128, bits=bits)
     assert len(names) == 14 and "lm_head" not in names            # 7 projections x 2 layers
-    assert all(isinstance(dict(quant.named_modules())[n], gpu_ops.W2A8Linear) for n in names)
-    ref = _dequantised_copy(model, names, 128)
+    layer_type = gpu_ops.W2A8Linear if bits == 2 else gpu_ops.W4A8Linear
+    assert all(isinstance(dict(quant.named_modules())[n], layer_type) for n in names)
+    ref = _dequantised_copy(model, names, 128, bits)
 
     g = torch.Generator().manual_seed(1)
     for shape in ((1, 12), (3, 5), (1, 1)):
