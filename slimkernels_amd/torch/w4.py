@@ -48,6 +48,28 @@ def repack_w4(packed4, scales, zp=None, group_size: int = 128, zp_const: int = 8
     return W4A8Weight(repack_w2(packed2, scales2, zp2, group_size, device=device), N, K, group_size)
 
 
+def save_w4(path, packed4, scales, zp=None, group_size: int = 128, zp_const: int = 8):
+    """Write a 4-bit weight to the on-disk container of slimkernels_amd.packed_format as its two 2-bit planes over
+    2K (mode tag "w4planes"): the file holds what the W2 entry points consume, in the interchange layout."""
+    from ..packed_format import save_w2
+    packed4 = np.asarray(packed4)
+    scales = np.asarray(scales)
+    if zp is None:
+        zp = np.full(scales.shape, int(zp_const), dtype=np.uint8)
+    packed2, scales2, zp2 = host_w4.split_planes(host_w4.unpack_w4(packed4), scales, np.asarray(zp))
+    save_w2(path, packed2, scales2, zp2, group_size, mode="w4planes")
+
+
+def load_w4_weight(path, device="cuda", mmap=True) -> W4A8Weight:
+    """A file written by save_w4 -> the weight on the GPU."""
+    from ..packed_format import load_w2
+    d = load_w2(path, mmap=mmap)
+    if d["mode"] != "w4planes" or d["zp"] is None or d["K"] % 2 != 0:
+        raise ValueError(f"{path}: not a two-plane W4 file (mode {d['mode']!r})")
+    planes = repack_w2(d["packed"], d["scales"], d["zp"], d["group_size"], device=device)
+    return W4A8Weight(planes, d["N"], d["K"] // 2, d["group_size"])
+
+
 def _twice(qa: QuantizedActivation) -> QuantizedActivation:
     """The activation operand over 2K: the int8 row and its per-group sums laid down twice."""
     return QuantizedActivation(torch.cat([qa.q, qa.q], dim=1), qa.s_a, torch.cat([qa.rowsum, qa.rowsum], dim=0),

@@ -200,3 +200,25 @@ def test_w4matmul_splitk_call_form(gpu_ops):
     s_a = np.abs(a.astype(np.float32)).max(axis=1) / 127
     tol = (s_a / 2)[:, None] * codes.sum(axis=1)[None, :] + 1e-3 * np.abs(want) + 0.26   # + fp16 rounding of c (|c| < 512)
     assert np.all(np.abs(c.float().cpu().numpy() - want) <= tol)
+
+
+@pytest.mark.gpu
+def test_w4_weight_through_the_file_container(gpu_ops, tmp_path):
+    from slimkernels_amd.torch import w4 as tw4
+    w, x = _w4_case(4, 192, 512, 128, "asym", seed=21)
+    packed4, scales, zp = w4.prepare_w4(w, 128, "asym")
+    path = str(tmp_path / "layer.w4")
+    tw4.save_w4(path, packed4, scales, zp, 128)
+    from_file = tw4.load_w4_weight(path)
+    direct = tw4.repack_w4(packed4, scales, zp, 128)
+    assert (from_file.N, from_file.K, from_file.group_size) == (192, 512, 128)
+    assert torch.equal(from_file.planes.w_r, direct.planes.w_r) and torch.equal(from_file.planes.s_r, direct.planes.s_r)
+    assert torch.equal(from_file.planes.zp_r, direct.planes.zp_r)
+    xd = torch.from_numpy(x).cuda()
+    assert torch.equal(tw4.w4a8_linear(xd, from_file), tw4.w4a8_linear(xd, direct))
+    # a W2 file is not taken for a W4 one
+    from slimkernels_amd import prepare_w2, save_w2
+    p2, s2, _ = prepare_w2(w, 128, "sym")
+    save_w2(str(tmp_path / "layer.w2"), p2, s2, None, 128, "sym")
+    with pytest.raises(ValueError, match="not a two-plane W4 file"):
+        tw4.load_w4_weight(str(tmp_path / "layer.w2"))
