@@ -389,7 +389,7 @@ def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, d
             use = ws4 if cold else ws4[:1] * 4
             x = torch.randn(M, K, device=dev, dtype=torch.float16)
             qa = ops.quantize_act_int8(x, g)
-            qa2 = tw4._twice(qa)
+            qa2 = tw4.activation_twice(qa)
             out = torch.empty((M, N), dtype=torch.float16, device=dev)
             for w in (use if cold else use[:1]):
                 ops.w2a8_gemm(qa2, w.planes, torch.float16, out=out)

@@ -70,7 +70,7 @@ def load_w4_weight(path, device="cuda", mmap=True) -> W4A8Weight:
     return W4A8Weight(planes, d["N"], d["K"] // 2, d["group_size"])
 
 
-def _twice(qa: QuantizedActivation) -> QuantizedActivation:
+def activation_twice(qa: QuantizedActivation) -> QuantizedActivation:
     """The activation operand over 2K: the int8 row and its per-group sums laid down twice."""
     return QuantizedActivation(torch.cat([qa.q, qa.q], dim=1), qa.s_a, torch.cat([qa.rowsum, qa.rowsum], dim=0),
                                qa.group_size)
@@ -85,7 +85,7 @@ def w4a8_gemm(qa: QuantizedActivation, w: W4A8Weight, out_dtype=torch.float16, *
         raise ValueError(f"activation K={K}/group {qa.group_size} does not match weight K={w.K}/group {w.group_size}")
     if dump not in (None, "groups"):
         raise ValueError("dump must be None or 'groups'")
-    res = w2a8_gemm(_twice(qa), w.planes, out_dtype, kernel=kernel, split_k=split_k, dump=dump, out=out)
+    res = w2a8_gemm(activation_twice(qa), w.planes, out_dtype, kernel=kernel, split_k=split_k, dump=dump, out=out)
     if dump is None:
         return res
     y, acc = res
