@@ -93,6 +93,14 @@ def w4a8_gemm(qa: QuantizedActivation, w: W4A8Weight, out_dtype=torch.float16, *
     return y, acc[:, :, :G] * 4 + acc[:, :, G:]
 
 
+def w4a8_gemm_grouped(problems, out_dtype=torch.float16):
+    """Several independent W4A8 GEMMs of at most 32 token rows in ONE launch (the grouped kernel of the W2 path):
+    ``problems`` is a list of (qa, w4, out) with ``qa`` = quantize_act_int8(x) over K, ``w4`` a W4A8Weight and
+    ``out`` [M, N] of ``out_dtype``.  All problems share the group size."""
+    from .ops import w2a8_gemm_grouped
+    return w2a8_gemm_grouped([(activation_twice(qa), w.planes, out) for qa, w, out in problems], out_dtype)
+
+
 def w4a8_linear(x: torch.Tensor, w: W4A8Weight, out_dtype=torch.float16) -> torch.Tensor:
     """x [M, K] fp16 / bf16 -> out [M, N]; one token row goes through the single-launch kernel that quantises
     the row itself."""

@@ -222,3 +222,22 @@ def test_w4_weight_through_the_file_container(gpu_ops, tmp_path):
     save_w2(str(tmp_path / "layer.w2"), p2, s2, None, 128, "sym")
     with pytest.raises(ValueError, match="not a two-plane W4 file"):
         tw4.load_w4_weight(str(tmp_path / "layer.w2"))
+
+
+@pytest.mark.gpu
+def test_w4a8_grouped_launch(gpu_ops, oracle):
+    from slimkernels_amd.torch import w4 as tw4
+    probs, refs = [], []
+    for i, (M, N, K) in enumerate(((1, 512, 1024), (16, 320, 2048), (32, 256, 512), (5, 1000, 1024))):
+        w, x = _w4_case(M, N, K, 128, "asym", seed=40 + i)
+        packed4, scales, zp = w4.prepare_w4(w, 128, "asym")
+        codes = w4.unpack_w4(packed4)
+        ref = oracle.w4_reference_forward(x, codes, scales, zp, 128)
+        qa = gpu_ops.quantize_act_int8(torch.from_numpy(x).cuda(), 128)
+        out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+        probs.append((qa, tw4.repack_w4(packed4, scales, zp, 128), out))
+        refs.append((ref, _plane_bound(oracle, ref, codes, scales, zp, 128)))
+    tw4.w4a8_gemm_grouped(probs, torch.float16)
+    torch.cuda.synchronize()
+    for (_, _, out), (ref, bound) in zip(probs, refs):
+        pu.assert_out_close(pu.out_tensor_bits(out), ref["out_bits"], False, bound, "W4A8 grouped")
