@@ -402,6 +402,23 @@ def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, d
                            "TOPS": round(nops / (us * 1e-6) / 1e12, 1), "frac_int8_mfma": round(nops / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4)})
         del ws4
     detail["w4a8"] = w4rows
+
+    # the decode sweep of the headline with 4-bit weights, as one grouped launch: every GEMM has its own weight
+    # (24 weights, 430 MB of 4-bit planes in all: more than the last-level cache, so every launch streams from HBM)
+    torch.cuda.empty_cache()
+    probs4, bytes4 = [], 0
+    for c in cases:
+        G = c.K // 128
+        w4w = tw4.W4A8Weight(random_weight(c.N, 2 * c.K, 128, True), c.N, c.K, 128)
+        _, qa, _ = acts[(c.N, c.K, c.M)]
+        probs4.append((tw4.activation_twice(qa), w4w.planes, torch.empty((c.M, c.N), dtype=torch.float16, device=dev)))
+        bytes4 += c.N * c.K // 2 + 2 * c.N * G + c.N * G // 2 + c.M * c.K + 4 * c.M + 2 * c.M * c.N
+    ops.w2a8_gemm_grouped(probs4, torch.float16)
+    us = time_graph(torch, lambda: [ops.w2a8_gemm_grouped(probs4, torch.float16) for _ in range(4)], 4, replays=10)
+    detail["w4a8_decode_sweep_grouped"] = {"gemms": len(probs4), "bytes": bytes4, "us": round(us, 2),
+                                           "GBps": round(bytes4 / (us * 1e-6) / 1e9, 1),
+                                           "frac_hbm": round(bytes4 / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                                           "note": "the int8 rows are laid down twice before the timed region (48 small copies, as act-quant is timed apart)"}
     return detail
 
 

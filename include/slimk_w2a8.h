@@ -154,6 +154,14 @@ int slimk_w2a8_quantize_weight(const void* w, int ldw, int w_dtype, int N, int K
 int slimk_w2a8_act_quant(const void* x, int ldx, int x_dtype, int M, int K, int group_size,
                          int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, void* stream);
 
+/* The same with the quantised row and its group sums laid down `copies` (1..4) times: q [M][ldq] holds the row
+ * at columns c * K .. c * K + K - 1 for c < copies (ldq >= copies * K), rowsum is [copies * G][ldr] with group g
+ * of copy c in row c * G + g.  This is the activation operand of a reduction over copies * K whose weight is
+ * several digit planes of one matrix (4-bit weights as two 2-bit planes: copies = 2, see the top of this file).
+ * No upstream counterpart. */
+int slimk_w2a8_act_quant_rep(const void* x, int ldx, int x_dtype, int M, int K, int group_size, int copies,
+                             int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, void* stream);
+
 /* The GEMM.  Counterpart of gemm_tn (wgmma_sm90_W2A8.cu:428-437); alpha/beta, unused
  * upstream (:408), are dropped.
  *   q, ldq, s_a, rowsum, ldr : outputs of slimk_w2a8_act_quant

@@ -223,21 +223,28 @@ int slimk_w2a8_quantize_weight(const void* w, int ldw, int w_dtype, int N, int K
                       "quantize_weight");
 }
 
-int slimk_w2a8_act_quant(const void* x, int ldx, int x_dtype, int M, int K, int group_size,
-                         int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, void* stream) {
+int slimk_w2a8_act_quant_rep(const void* x, int ldx, int x_dtype, int M, int K, int group_size, int copies,
+                             int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, void* stream) {
     if (!x || !q || !s_a) return fail(SLIMK_ERR_NULL_POINTER, "act_quant: NULL buffer");
     if (M <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "M=%d must be positive", M);
+    if (copies < 1 || copies > 4) return fail(SLIMK_ERR_BAD_SHAPE, "copies=%d must be 1..4", copies);
     if (int rc = check_kg(K, group_size)) return rc;
     if (x_dtype != SLIMK_F16 && x_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "x_dtype=%d", x_dtype);
-    if (ldx < K || ldq < K) return fail(SLIMK_ERR_BAD_SHAPE, "ldx=%d / ldq=%d smaller than K=%d", ldx, ldq, K);
+    if (ldx < K || (long long)ldq < (long long)copies * K)
+        return fail(SLIMK_ERR_BAD_SHAPE, "ldx=%d smaller than K=%d or ldq=%d smaller than copies * K", ldx, K, ldq);
     if (rowsum && ldr < M) return fail(SLIMK_ERR_BAD_SHAPE, "ldr=%d smaller than M=%d", ldr, M);
     if (!aligned16(x) || !aligned16(q) || ldx % 8 != 0 || ldq % 16 != 0)
         return fail(SLIMK_ERR_MISALIGNED, "act_quant: x, q must be 16-byte aligned, ldx %% 8 == 0, ldq %% 16 == 0");
     if (rowsum && (!aligned16(rowsum) || ldr % 4 != 0))
         return fail(SLIMK_ERR_MISALIGNED, "act_quant: rowsum must be 16-byte aligned and ldr %% 4 == 0");
     return hip_result(w2a8::launch_act_quant(x, ldx, x_dtype == SLIMK_BF16, M, K, group_size, q, ldq, s_a,
-                                             rowsum, ldr, (hipStream_t)stream),
+                                             rowsum, ldr, copies, (hipStream_t)stream),
                       "act_quant");
+}
+
+int slimk_w2a8_act_quant(const void* x, int ldx, int x_dtype, int M, int K, int group_size,
+                         int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, void* stream) {
+    return slimk_w2a8_act_quant_rep(x, ldx, x_dtype, M, K, group_size, 1, q, ldq, s_a, rowsum, ldr, stream);
 }
 
 int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,

@@ -105,7 +105,7 @@ template <bool BF16>
 __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restrict__ x, int ldx, int K,
                                                         int group_size, int8_t* __restrict__ q, int ldq,
                                                         float* __restrict__ s_a,
-                                                        int32_t* __restrict__ rowsum, int ldr) {
+                                                        int32_t* __restrict__ rowsum, int ldr, int copies) {
     __shared__ float red[4];
     const int m = blockIdx.x;
     const int tid = threadIdx.x;
@@ -149,11 +149,13 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
                 if (i < 4) lo |= (uint32_t)(qi & 0xff) << (8 * i);
                 else hi |= (uint32_t)(qi & 0xff) << (8 * (i - 4));
             }
-            *reinterpret_cast<uint2*>(qr + (size_t)v * 8) = make_uint2(lo, hi);
+            for (int cp = 0; cp < copies; ++cp)   // copies > 1: the row laid down again K further on
+                *reinterpret_cast<uint2*>(qr + (size_t)cp * K + (size_t)v * 8) = make_uint2(lo, hi);
         }
         // nvec is a multiple of tpg, so a group's threads are all valid or all idle
         for (int off = 1; off < tpg; off <<= 1) sum += __shfl_xor(sum, off, 64);
-        if (rowsum && v < nvec && (v % tpg) == 0) rowsum[(size_t)(v / tpg) * ldr + m] = sum;
+        if (rowsum && v < nvec && (v % tpg) == 0)
+            for (int cp = 0; cp < copies; ++cp) rowsum[((size_t)cp * (nvec / tpg) + v / tpg) * ldr + m] = sum;
     }
 }
 
@@ -165,7 +167,7 @@ template <bool BF16, int KEEP>
 __global__ __launch_bounds__(256) void act_quant_keep_kernel(const uint16_t* __restrict__ x, int ldx, int K,
                                                              int group_size, int8_t* __restrict__ q, int ldq,
                                                              float* __restrict__ s_a,
-                                                             int32_t* __restrict__ rowsum, int ldr) {
+                                                             int32_t* __restrict__ rowsum, int ldr, int copies) {
     __shared__ float red[4];
     const int m = blockIdx.x;
     const int tid = threadIdx.x;
@@ -212,38 +214,40 @@ __global__ __launch_bounds__(256) void act_quant_keep_kernel(const uint16_t* __r
                 if (i < 4) lo |= (uint32_t)(qi & 0xff) << (8 * i);
                 else hi |= (uint32_t)(qi & 0xff) << (8 * (i - 4));
             }
-            *reinterpret_cast<uint2*>(qr + (size_t)v * 8) = make_uint2(lo, hi);
+            for (int cp = 0; cp < copies; ++cp)   // copies > 1: the row laid down again K further on
+                *reinterpret_cast<uint2*>(qr + (size_t)cp * K + (size_t)v * 8) = make_uint2(lo, hi);
         }
         for (int off = 1; off < tpg; off <<= 1) sum += __shfl_xor(sum, off, 64);
-        if (rowsum && v < nvec && (v % tpg) == 0) rowsum[(size_t)(v / tpg) * ldr + m] = sum;
+        if (rowsum && v < nvec && (v % tpg) == 0)
+            for (int cp = 0; cp < copies; ++cp) rowsum[((size_t)cp * (nvec / tpg) + v / tpg) * ldr + m] = sum;
     }
 }
 
 template <bool BF16>
 static void launch_act_quant_keep(const void* x, int ldx, int M, int K, int group_size, int8_t* q, int ldq, float* s_a,
-                                  int32_t* rowsum, int ldr, hipStream_t stream) {
+                                  int32_t* rowsum, int ldr, int copies, hipStream_t stream) {
     const dim3 grid((unsigned)M), block(256);
     if (K <= 4096)
-        act_quant_keep_kernel<BF16, 2><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr);
+        act_quant_keep_kernel<BF16, 2><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
     else if (K <= 8192)
-        act_quant_keep_kernel<BF16, 4><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr);
+        act_quant_keep_kernel<BF16, 4><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
     else
-        act_quant_keep_kernel<BF16, 8><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr);
+        act_quant_keep_kernel<BF16, 8><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
 }
 
 hipError_t launch_act_quant(const void* x, int ldx, bool x_bf16, int M, int K, int group_size,
-                            int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, hipStream_t stream) {
+                            int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, int copies, hipStream_t stream) {
     if (K <= 16384) {
-        if (x_bf16) launch_act_quant_keep<true>(x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, stream);
-        else launch_act_quant_keep<false>(x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, stream);
+        if (x_bf16) launch_act_quant_keep<true>(x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies, stream);
+        else launch_act_quant_keep<false>(x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies, stream);
         return hipGetLastError();
     }
     if (x_bf16)
         act_quant_kernel<true><<<dim3(M), dim3(256), 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q,
-                                                                 ldq, s_a, rowsum, ldr);
+                                                                 ldq, s_a, rowsum, ldr, copies);
     else
         act_quant_kernel<false><<<dim3(M), dim3(256), 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q,
-                                                                  ldq, s_a, rowsum, ldr);
+                                                                  ldq, s_a, rowsum, ldr, copies);
     return hipGetLastError();
 }
 

@@ -14,7 +14,7 @@ hipError_t launch_repack(const uint8_t* w_packed, int ldw, const uint16_t* scale
                          hipStream_t stream);
 
 hipError_t launch_act_quant(const void* x, int ldx, bool x_bf16, int M, int K, int group_size,
-                            int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, hipStream_t stream);
+                            int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, int copies, hipStream_t stream);
 
 // mode: 0 upstream quantizer (zero-point 1), 1 symmetric levels (zero-point 2), 2 per-group zero-points
 hipError_t launch_quantize_weight(const void* w, int ldw, bool w_bf16, int N, int K, int group_size, int mode,

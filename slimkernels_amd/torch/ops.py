@@ -149,8 +149,10 @@ def load_w2_weight(path, device="cuda", mmap=True) -> W2A8Weight:
                      zp_const=f["zp_const"] if f["zp_const"] is not None else 0, device=device)
 
 
-def quantize_act_int8(x: torch.Tensor, group_size: int = 128) -> QuantizedActivation:
-    """Per-token symmetric int8 quantisation: x [M, K] fp16/bf16 -> q, s_a, per-group row sums."""
+def quantize_act_int8(x: torch.Tensor, group_size: int = 128, copies: int = 1) -> QuantizedActivation:
+    """Per-token symmetric int8 quantisation: x [M, K] fp16/bf16 -> q, s_a, per-group row sums.  With
+    ``copies`` > 1 the quantised row and its group sums are laid down that many times (q [M, copies * K],
+    rowsum [copies * G, ...]): the operand of a reduction over copies * K, as the 4-bit weights take it."""
     L = _lib.lib()
     _require_cuda(x, "x")
     if x.dim() != 2 or x.dtype not in _DT:
@@ -159,13 +161,14 @@ def quantize_act_int8(x: torch.Tensor, group_size: int = 128) -> QuantizedActiva
         x = x.contiguous()
     M, K = x.shape
     ldr = (M + 3) // 4 * 4
-    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    copies = int(copies)
+    q = torch.empty((M, max(copies, 1) * K), dtype=torch.int8, device=x.device)
     s_a = torch.empty((M,), dtype=torch.float32, device=x.device)
-    rowsum = torch.empty((max(K // group_size, 1), ldr), dtype=torch.int32, device=x.device)
+    rowsum = torch.empty((max(copies, 1) * max(K // group_size, 1), ldr), dtype=torch.int32, device=x.device)
     with torch.cuda.device(x.device):
-        _lib.check(L.slimk_w2a8_act_quant(x.data_ptr(), x.stride(0), _DT[x.dtype], M, K, group_size,
-                                          q.data_ptr(), q.stride(0), s_a.data_ptr(), rowsum.data_ptr(), ldr,
-                                          _stream_ptr(x.device)))
+        _lib.check(L.slimk_w2a8_act_quant_rep(x.data_ptr(), x.stride(0), _DT[x.dtype], M, K, group_size, copies,
+                                              q.data_ptr(), q.stride(0), s_a.data_ptr(), rowsum.data_ptr(), ldr,
+                                              _stream_ptr(x.device)))
     return QuantizedActivation(q, s_a, rowsum, group_size)
 
 

@@ -111,7 +111,8 @@ def w4a8_linear(x: torch.Tensor, w: W4A8Weight, out_dtype=torch.float16) -> torc
         raise ValueError(f"activation K={x.shape[1]} does not match weight K={w.K}")
     if x.shape[0] == 1 and fused_applies(1, 2 * w.K):
         return w2a8_linear_fused(torch.cat([x, x], dim=1), w.planes, out_dtype)
-    return w4a8_gemm(quantize_act_int8(x, w.group_size), w, out_dtype)
+    # one quantisation launch writes the row and its group sums twice: the operand over 2K
+    return w2a8_gemm(quantize_act_int8(x, w.group_size, copies=2), w.planes, out_dtype)
 
 
 class W4A8Linear(torch.nn.Module):

@@ -120,6 +120,12 @@ def test_repack_and_act_quant_validation(L):
     assert a(FAKE, 100, 0, 1, 4096, 128, FAKE, 4096, FAKE, FAKE, 4, None) == 2
     assert a(FAKE, 4096 + 4, 0, 1, 4096, 128, FAKE, 4096, FAKE, FAKE, 4, None) == 3
     assert a(FAKE, 4096, 0, 5, 4096, 128, FAKE, 4096, FAKE, FAKE, 4, None) == 2        # ldr < M
+    rep = L.slimk_w2a8_act_quant_rep  # (x, ldx, dtype, M, K, group, copies, q, ldq, s_a, rowsum, ldr, stream)
+    assert rep(FAKE, 4096, 0, 1, 4096, 128, 0, FAKE, 8192, FAKE, FAKE, 4, None) == 2
+    assert rep(FAKE, 4096, 0, 1, 4096, 128, 5, FAKE, 32768, FAKE, FAKE, 4, None) == 2
+    assert rep(FAKE, 4096, 0, 1, 4096, 128, 2, FAKE, 4096, FAKE, FAKE, 4, None) == 2   # ldq < copies * K
+    assert b"copies * K" in L.slimk_w2a8_last_error()
+    assert rep(None, 4096, 0, 1, 4096, 128, 2, FAKE, 8192, FAKE, FAKE, 4, None) == 1
     qw = L.slimk_w2a8_quantize_weight  # (w, ldw, dtype, N, K, group, mode, packed, ldp, scales, zp, stream)
     assert qw(None, 4096, 0, 64, 4096, 128, 1, FAKE, 1024, FAKE, None, None) == 1
     assert qw(FAKE, 4096, 0, 64, 4096, 128, 2, FAKE, 1024, FAKE, None, None) == 1      # per-group zero-points need zp

@@ -163,6 +163,23 @@ def test_w4a8_gemm_against_the_oracle(gpu_ops, oracle, M, N, K, g, mode, out, ke
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("M,K,g,bf16,copies", [(1, 1024, 128, False, 2), (5, 4096, 128, True, 2), (33, 8192, 64, False, 2),
+                                                (7, 14336, 128, False, 2), (3, 20480, 128, True, 2), (2, 512, 64, False, 3)])
+def test_act_quant_laid_down_several_times(gpu_ops, M, K, g, bf16, copies):
+    """One launch that writes the quantised row and its group sums ``copies`` times gives exactly what the
+    plain launch gives, repeated (all three kernels of the launcher: K <= 4096, <= 16384, beyond)."""
+    print(f"act_quant copies: M={M} K={K} g={g} bf16={bf16} copies={copies}", flush=True)
+    gen = torch.Generator().manual_seed(M * 131 + K)
+    x = (torch.randn((M, K), generator=gen) * 3).to(torch.bfloat16 if bf16 else torch.float16).cuda()
+    one = gpu_ops.quantize_act_int8(x, g)
+    rep = gpu_ops.quantize_act_int8(x, g, copies=copies)
+    assert rep.q.shape == (M, copies * K) and rep.rowsum.shape[0] == copies * (K // g)
+    assert torch.equal(rep.q, torch.cat([one.q] * copies, dim=1))
+    assert torch.equal(rep.rowsum[:, :M], torch.cat([one.rowsum[:, :M]] * copies, dim=0))
+    assert torch.equal(rep.s_a, one.s_a)
+
+
+@pytest.mark.gpu
 def test_w4a8_linear_and_decode_row(gpu_ops, oracle):
     from slimkernels_amd.torch import w4 as tw4
     w, x = _w4_case(3, 384, 1024, 128, "sym", seed=11)
