@@ -233,6 +233,26 @@ typedef struct slimk_w2a8_problem {
 int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int group_size, int out_dtype,
                             void* stream);
 
+/* Weight-only form: x [M][ldx] fp16 activations are NOT quantised; the 2-bit codes are widened to fp16 in
+ * front of the fp16 matrix cores and every scale group's fp32 sum is scaled into the fp32 result:
+ *   out[m][n] = cast( sum_g scales[g][n] * sum_{k in g} x[m][k] * (code[n][k] - zp[g][n]) ).
+ * Same repacked weight operands as slimk_w2a8_gemm (w_r, s_r, zp_r / zp_const).  Built for few token rows
+ * (the weight stream bounds the time); any M works, 16 rows at a time, each re-reading the weights.
+ * K % 128 == 0; x_dtype must be SLIMK_F16 (bf16 activations: SLIMK_ERR_UNSUPPORTED); x 16-byte aligned,
+ * ldx % 8 == 0.  split_k: K splits across workgroups, 0 = choose; with more than one the caller supplies
+ * slimk_w2a16_gemm_workspace_bytes(...) bytes of workspace (fp32 partial sums, summed in split order by a
+ * second kernel: results do not depend on timing).  The workspace needs no initialisation.
+ * Replaces the upstream notebook kernel w2matmul(a, b, c) (slimkernels/triton/gemm_splitk.ipynb cell 1:
+ * `b = ((b >> 4) & 0b11).to(tl.float16); accumulator = tl.dot(a, b, accumulator)`), which has no scales,
+ * no zero-point and reads one field per word. */
+int slimk_w2a16_gemm_auto_split_k(int M, int N, int K, int group_size);
+size_t slimk_w2a16_gemm_workspace_bytes(int M, int N, int K, int group_size, int split_k);
+int slimk_w2a16_gemm(const void* x, int ldx, int x_dtype,
+                     const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
+                     int M, int N, int K, int group_size,
+                     void* out, int ldo, int out_dtype,
+                     void* workspace, size_t workspace_bytes, int split_k, void* stream);
+
 /* Streaming-read calibration kernel: sums `bytes` (multiple of 16) of device memory into
  * sink[0..] so that a profiler can relate its FETCH_SIZE counter to a known byte count and
  * the benchmark can quote the achievable HBM read rate next to the GEMM's. */

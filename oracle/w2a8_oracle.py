@@ -326,6 +326,26 @@ def w4_reference_forward(x_half: np.ndarray, codes_nk: np.ndarray, scale_half: n
     return dict(q=q, s_a=s_a, rowsum=rs, acc=acc, out_bits=out_bits, out_f32=out_f32)
 
 
+def w2a16_reference_forward(x_half: np.ndarray, codes_nk: np.ndarray, scale_half: np.ndarray, zp: np.ndarray,
+                            group_size: int):
+    """The weight-only form in float64: out[m, n] = sum_g scale[g, n] * sum_{k in g} x[m, k] * (code[n, k] - zp[g, n])
+    with the fp16 activations as they are (the notebook kernel w2matmul, gemm_splitk.ipynb cell 1, widens the
+    2-bit fields to fp16 in front of an fp32-accumulating dot; it has no scales and no zero-point, which are
+    this path's own).  Returns (out float64 [M, N], mag float64 [M, N]) where mag = sum_g |scale| * sum_k |x| * |code - zp|
+    bounds the terms, for a tolerance on an fp32 accumulation in any order."""
+    x = np.asarray(x_half, np.float16).astype(np.float64)
+    codes = np.asarray(codes_nk, np.uint8)
+    N, K = codes.shape
+    M = x.shape[0]
+    G = K // group_size
+    w = codes.astype(np.float64).reshape(N, G, group_size) - np.asarray(zp, np.float64).T[:, :, None]
+    s = np.asarray(scale_half, np.float16).astype(np.float64).T                       # [N, G]
+    xg = x.reshape(M, G, group_size)
+    out = np.einsum("mgk,ngk,ng->mn", xg, w, s, optimize=True)
+    mag = np.einsum("mgk,ngk,ng->mn", np.abs(xg), np.abs(w), np.abs(s), optimize=True)
+    return out, mag
+
+
 # --------------------------------------------------------------------------- whole-path helper
 
 def reference_forward(x_half: np.ndarray, packed: np.ndarray, scale_half: np.ndarray, zp: np.ndarray,

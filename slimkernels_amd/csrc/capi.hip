@@ -502,6 +502,57 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
                       "grouped skinny gemm");
 }
 
+int slimk_w2a16_gemm_auto_split_k(int M, int N, int K, int group_size) {
+    if (M <= 0 || N <= 0 || !shape_ok(K, group_size) || K % 128 != 0) return 0;
+    return w2a8::w2a16_auto_split(M, strips_of(N), K / w2a8::kStepK, group_size / w2a8::kStepK);
+}
+
+size_t slimk_w2a16_gemm_workspace_bytes(int M, int N, int K, int group_size, int split_k) {
+    if (split_k <= 0) split_k = slimk_w2a16_gemm_auto_split_k(M, N, K, group_size);
+    if (split_k <= 1 || M <= 0 || N <= 0) return 0;
+    return (size_t)split_k * (size_t)M * (size_t)N * sizeof(float);
+}
+
+int slimk_w2a16_gemm(const void* x, int ldx, int x_dtype,
+                     const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
+                     int M, int N, int K, int group_size,
+                     void* out, int ldo, int out_dtype,
+                     void* workspace, size_t workspace_bytes, int split_k, void* stream) {
+    if (!x || !w_r || !s_r || !out) return fail(SLIMK_ERR_NULL_POINTER, "w2a16_gemm: NULL buffer");
+    if (M <= 0 || N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "M=%d, N=%d must be positive", M, N);
+    if (int rc = check_kg(K, group_size)) return rc;
+    if (K % 128 != 0) return fail(SLIMK_ERR_UNSUPPORTED, "w2a16_gemm: K=%d must be a multiple of 128", K);
+    if (x_dtype != SLIMK_F16 && x_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "x_dtype=%d", x_dtype);
+    if (x_dtype != SLIMK_F16) return fail(SLIMK_ERR_UNSUPPORTED, "w2a16_gemm: activations must be fp16");
+    if (out_dtype != SLIMK_F16 && out_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "out_dtype=%d", out_dtype);
+    if (zp_const < 0 || zp_const > 3) return fail(SLIMK_ERR_BAD_SHAPE, "zp_const=%d must be 0..3", zp_const);
+    if (ldx < K || ldo < N) return fail(SLIMK_ERR_BAD_SHAPE, "ldx=%d / ldo=%d too small for K=%d / N=%d", ldx, ldo, K, N);
+    if (int rc = check_extent(M, N, K, 2 * ldx)) return rc;
+    if (!aligned16(x) || ldx % 8 != 0 || !aligned16(w_r) || !aligned16(s_r) || (zp_r && !aligned16(zp_r)) ||
+        (reinterpret_cast<uintptr_t>(out) & 1u))
+        return fail(SLIMK_ERR_MISALIGNED, "w2a16_gemm: x, w_r, s_r, zp_r must be 16-byte aligned; ldx %% 8 == 0; out 2-byte aligned");
+    const int gs = group_size / w2a8::kStepK, steps = K / w2a8::kStepK;
+    const int granules = steps / (gs > 2 ? gs : 2);
+    if (split_k <= 0) split_k = w2a8::w2a16_auto_split(M, strips_of(N), steps, gs);
+    if (split_k > 64 || (split_k > 1 && split_k * 4 > granules))
+        return fail(SLIMK_ERR_BAD_SHAPE, "split_k=%d: at most 64 and at most a quarter of the %d K granules", split_k, granules);
+
+    w2a8::W2A16Params p{};
+    p.x = reinterpret_cast<const uint16_t*>(x); p.ldx = ldx;
+    p.w_r = w_r; p.s_r = s_r; p.zp_r = zp_r; p.out = out; p.ldo = ldo;
+    p.M = M; p.N = N; p.K = K; p.G = K / group_size; p.steps = steps; p.strips = strips_of(N);
+    p.zp_const = zp_const; p.split = split_k;
+    if (split_k > 1) {
+        const size_t need = (size_t)split_k * (size_t)M * (size_t)N * sizeof(float);
+        if (!workspace) return fail(SLIMK_ERR_WORKSPACE, "split_k=%d needs a workspace of %zu bytes", split_k, need);
+        if (workspace_bytes < need)
+            return fail(SLIMK_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, need);
+        if (!aligned16(workspace)) return fail(SLIMK_ERR_MISALIGNED, "workspace must be 16-byte aligned");
+        p.ws = reinterpret_cast<float*>(workspace);
+    }
+    return hip_result(w2a8::launch_w2a16(p, gs, out_dtype == SLIMK_BF16, (hipStream_t)stream), "w2a16_gemm");
+}
+
 int slimk_w2a8_read_probe(const void* src, size_t bytes, uint32_t* sink, void* stream) {
     if (!src || !sink) return fail(SLIMK_ERR_NULL_POINTER, "read_probe: NULL buffer");
     if (bytes == 0 || bytes % 16 != 0 || !aligned16(src))

@@ -1,0 +1,230 @@
+// Weight-only W2 GEMM for gfx950: fp16 activations times 2-bit weights on the fp16 matrix cores
+// (v_mfma_f32_16x16x32_f16), fp32 accumulation, the few-token-rows regime where the weight stream
+// bounds the time.  Upstream's sketch of this form is the notebook kernel `w2matmul`
+// (slimkernels/triton/gemm_splitk.ipynb cell 1: 2-bit fields widened to fp16 in front of tl.dot).
+//
+//   out[m][n] = sum_g scale[g][n] * sum_{k in group g} x[m][k] * (code[n][k] - zp[g][n])
+//
+// The weights are the repacked units of the W2A8 kernels (w2a8_common.h), read once.  A unit's dword i
+// holds, in 2-bit field p of byte b, the code of channel p*16 + col at k = quad*16 + 4*i + b.  Widening
+// without shifts: (dword & (0x00030003 << 2p)) | 0x64006400 is the fp16 pair (1024 + 4^p*code) of bytes 0
+// and 2, the same on (dword >> 8) the pair of bytes 1 and 3; one packed fp16 subtraction of
+// 1024 + 4^p*zp leaves 4^p * (code - zp), exact, and 4^-p goes into the fp32 scale.  The lane's eight
+// k-values of one MFMA therefore come in the order 0,2,1,3,4,6,5,7; the activation operand is put in
+// the same order with two v_perm_b32 per register pair.
+//
+// Work split: a workgroup is four wavefronts that take four K-parts of ONE strip of 64 channels and
+// 16 token rows and add their sums up through LDS; blockIdx.y splits K further across workgroups
+// (fp32 partial sums to a workspace, summed in split order by a second kernel: deterministic).
+// Activations are read straight from global memory (they stay in L2; rows past M are out of range of the
+// buffer descriptor and read as zero without a memory access).
+#include "w2a8_launch.h"
+
+namespace w2a8 {
+
+namespace {
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+constexpr int kWaves = 4;        // K-parts per workgroup
+constexpr int kChunkSteps = 2;   // steps (of 64) per loop iteration
+
+// GS = steps per scale group (1, 2 or 4); ZP = per-group zero-points; PARTIAL = write fp32 partials
+template <int GS, bool ZP, bool PARTIAL, typename OutT>
+__global__ __launch_bounds__(256) void w2a16_kernel(const W2A16Params p) {
+    __shared__ float red[kWaves][16][64];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 15, quad = lane >> 4;
+    const int strip = blockIdx.x;
+    const int m0 = (int)blockIdx.z * 16;
+
+    // K-parts in granules of max(GS, 2) steps, dealt out evenly over split * 4 parts (a part may be empty)
+    constexpr int kGranule = GS > kChunkSteps ? GS : kChunkSteps;
+    const int n_gran = p.steps / kGranule;
+    const int parts = p.split * kWaves;
+    const int part = (int)blockIdx.y * kWaves + wave;
+    const int gr0 = (int)((long long)part * n_gran / parts), gr1 = (int)((long long)(part + 1) * n_gran / parts);
+    const int step0 = gr0 * kGranule;
+    const int n_chunks = (gr1 - gr0) * (kGranule / kChunkSteps);
+
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(p.x), 0, (int)min((size_t)p.M * p.ldx * 2, (size_t)0x7fffffff), 0x00020000);
+    const uint32_t x_lane = ((uint32_t)(m0 + col) * (uint32_t)p.ldx + quad * 16) * 2;   // bytes
+    const uint32_t* w_lane = p.w_r + ((size_t)strip * 64 + lane) * 4;
+    const size_t w_step = (size_t)p.strips * kUnitDwords;                               // dwords between steps
+    const uint16_t* s_lane = p.s_r + ((size_t)strip * 16 + col) * 4;
+    const uint8_t* z_lane = ZP ? p.zp_r + ((size_t)strip * 16 + col) * 4 : nullptr;
+    const size_t sz_group = (size_t)p.strips * 64;                                      // elements between groups
+
+    constexpr int kGPC = GS == 1 ? 2 : 1;  // scale groups that start or continue in one chunk
+    struct Chunk {
+        v4i w[kChunkSteps];
+        v4u a[kChunkSteps][2];
+        uint2 s[kGPC];
+        uint32_t z[kGPC];
+    };
+    auto load = [&](int c) {
+        Chunk ch;
+        const int st = step0 + c * kChunkSteps;
+#pragma unroll
+        for (int s = 0; s < kChunkSteps; ++s) {
+            ch.w[s] = *reinterpret_cast<const v4i*>(w_lane + (size_t)(st + s) * w_step);
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                ch.a[s][h] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_lane + (uint32_t)((st + s) * kStepK * 2 + h * 16), 0, 0);
+        }
+#pragma unroll
+        for (int gi = 0; gi < kGPC; ++gi) {
+            const int g = (st + gi) / GS;   // GS == 1: groups st, st + 1; otherwise the group of step st
+            ch.s[gi] = *reinterpret_cast<const uint2*>(s_lane + (size_t)g * sz_group);
+            ch.z[gi] = ZP ? *reinterpret_cast<const uint32_t*>(z_lane + (size_t)g * sz_group) : 0u;
+        }
+        return ch;
+    };
+
+    float t[4][4];
+    v4f acc[4];
+#pragma unroll
+    for (int pp = 0; pp < 4; ++pp) {
+        acc[pp] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) t[pp][j] = 0.f;
+    }
+
+    if (n_chunks > 0) {
+        Chunk cur = load(0);
+        for (int c = 0; c < n_chunks; ++c) {
+            const Chunk nxt = load(min(c + 1, n_chunks - 1));   // the last iteration re-reads its own chunk
+#pragma unroll
+            for (int s = 0; s < kChunkSteps; ++s) {
+                const int gi = GS == 1 ? s : 0;
+                // 1024 + 4^p * zp as an fp16 pair, per sub-block
+                uint32_t zm[4];
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) {
+                    const uint32_t z = ZP ? (cur.z[gi] >> (8 * pp)) & 0xffu : (uint32_t)p.zp_const;
+                    zm[pp] = (0x6400u | (z << (2 * pp))) * 0x00010001u;
+                }
+                const v4i wf = cur.w[s] ^ (int)0x80808080u;      // field 3 is stored with its high bit flipped
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const v4u d = cur.a[s][h];
+                    const v4u ap = {__builtin_amdgcn_perm(d[1], d[0], 0x05040100u), __builtin_amdgcn_perm(d[1], d[0], 0x07060302u),
+                                    __builtin_amdgcn_perm(d[3], d[2], 0x05040100u), __builtin_amdgcn_perm(d[3], d[2], 0x07060302u)};
+                    const uint32_t e0 = (uint32_t)wf[2 * h], e1 = (uint32_t)wf[2 * h + 1];
+                    const uint32_t o0 = e0 >> 8, o1 = e1 >> 8;
+#pragma unroll
+                    for (int pp = 0; pp < 4; ++pp) {
+                        const uint32_t mask = 0x00030003u << (2 * pp);
+                        const v4u braw = {(e0 & mask) | 0x64006400u, (o0 & mask) | 0x64006400u,
+                                          (e1 & mask) | 0x64006400u, (o1 & mask) | 0x64006400u};
+                        const v4u zraw = {zm[pp], zm[pp], zm[pp], zm[pp]};
+                        const v8h b = __builtin_bit_cast(v8h, braw) - __builtin_bit_cast(v8h, zraw);
+                        acc[pp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, ap), b, acc[pp], 0, 0, 0);
+                    }
+                }
+                // end of a scale group: fold the group's sums into the running sums
+                const bool group_ends = GS <= kChunkSteps ? ((s + 1) % GS == 0)
+                                                          : (((step0 + c * kChunkSteps + s + 1) % GS) == 0);
+                if (group_ends) {
+#pragma unroll
+                    for (int pp = 0; pp < 4; ++pp) {
+                        const uint32_t raw = pp < 2 ? cur.s[gi].x : cur.s[gi].y;
+                        const float sc = half_bits_to_float((uint16_t)((pp & 1) ? raw >> 16 : raw & 0xffffu)) *
+                                         (1.0f / (float)(1 << (2 * pp)));
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) t[pp][j] = __builtin_fmaf(acc[pp][j], sc, t[pp][j]);
+                        acc[pp] = v4f{0.f, 0.f, 0.f, 0.f};
+                    }
+                }
+            }
+            cur = nxt;
+        }
+    }
+
+    // the four K-parts of the workgroup meet in LDS; wave w finishes sub-block w
+#pragma unroll
+    for (int pp = 0; pp < 4; ++pp)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) red[wave][pp * 4 + j][lane] = t[pp][j];
+    __syncthreads();
+    const int n = strip * kStripN + wave * 16 + col;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float v = red[0][wave * 4 + j][lane];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) v += red[w][wave * 4 + j][lane];
+        const int m = m0 + quad * 4 + j;
+        if (m < p.M && n < p.N) {
+            if (PARTIAL) p.ws[((size_t)blockIdx.y * p.M + m) * p.N + n] = v;
+            else reinterpret_cast<uint16_t*>(p.out)[(size_t)m * p.ldo + n] = OutT::cast(v);
+        }
+    }
+}
+
+template <typename OutT>
+__global__ __launch_bounds__(256) void w2a16_reduce_kernel(const float* __restrict__ ws, int split, int M, int N,
+                                                           uint16_t* __restrict__ out, int ldo) {
+    const size_t total = (size_t)M * N;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        float v = ws[i];
+        for (int s = 1; s < split; ++s) v += ws[(size_t)s * total + i];
+        out[(i / N) * ldo + i % N] = OutT::cast(v);
+    }
+}
+
+template <int GS, bool ZP, bool PARTIAL>
+void launch_one(const W2A16Params& p, bool out_bf16, dim3 grid, hipStream_t stream) {
+    if (out_bf16) w2a16_kernel<GS, ZP, PARTIAL, OutBF16><<<grid, dim3(256), 0, stream>>>(p);
+    else w2a16_kernel<GS, ZP, PARTIAL, OutF16><<<grid, dim3(256), 0, stream>>>(p);
+}
+
+template <int GS>
+void launch_gs(const W2A16Params& p, bool out_bf16, dim3 grid, hipStream_t stream) {
+    const bool zp = p.zp_r != nullptr, partial = p.split > 1;
+    if (zp) {
+        if (partial) launch_one<GS, true, true>(p, out_bf16, grid, stream);
+        else launch_one<GS, true, false>(p, out_bf16, grid, stream);
+    } else {
+        if (partial) launch_one<GS, false, true>(p, out_bf16, grid, stream);
+        else launch_one<GS, false, false>(p, out_bf16, grid, stream);
+    }
+}
+
+}  // namespace
+
+// K splits across workgroups: enough workgroups for about three per CU, every K-part at least two
+// granules (256 reduction elements at group size <= 128) long.
+int w2a16_auto_split(int M, int strips, int steps, int gs) {
+    const int granule = gs > kChunkSteps ? gs : kChunkSteps;
+    const int n_gran = steps / granule;
+    const long long base = (long long)strips * ((M + 15) / 16);
+    long long split = (768 + base - 1) / base;
+    const int cap = n_gran / (2 * kWaves);
+    if (split > cap) split = cap;
+    if (split > 64) split = 64;
+    return split < 1 ? 1 : (int)split;
+}
+
+hipError_t launch_w2a16(const W2A16Params& p, int gs, bool out_bf16, hipStream_t stream) {
+    const dim3 grid((unsigned)p.strips, (unsigned)p.split, (unsigned)((p.M + 15) / 16));
+    if (gs == 1) launch_gs<1>(p, out_bf16, grid, stream);
+    else if (gs == 2) launch_gs<2>(p, out_bf16, grid, stream);
+    else launch_gs<4>(p, out_bf16, grid, stream);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    if (p.split > 1) {
+        const size_t total = (size_t)p.M * p.N;
+        const unsigned blocks = (unsigned)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
+        if (out_bf16)
+            w2a16_reduce_kernel<OutBF16><<<dim3(blocks), dim3(256), 0, stream>>>(p.ws, p.split, p.M, p.N, (uint16_t*)p.out, p.ldo);
+        else
+            w2a16_reduce_kernel<OutF16><<<dim3(blocks), dim3(256), 0, stream>>>(p.ws, p.split, p.M, p.N, (uint16_t*)p.out, p.ldo);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace w2a8

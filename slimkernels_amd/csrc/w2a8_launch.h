@@ -47,6 +47,23 @@ bool tiled_fast_supported(const GemmParams& p, int gs, bool asym);
 int tiled_fast_auto_split(int M, int strips, int steps);
 int tiled_fast_max_split(int M, int strips, int steps);
 size_t tiled_fast_workspace_tiles(int M, int strips);
+// Weight-only form (fp16 activations on the fp16 matrix cores, gemm_w2a16.hip).
+struct W2A16Params {
+    const uint16_t* x;      // [M][ldx] fp16 bits
+    const uint32_t* w_r;    // repacked codes
+    const uint16_t* s_r;    // [G][strips][16][4] fp16 bits
+    const uint8_t* zp_r;    // [G][strips][16][4] or nullptr
+    void* out;              // [M][ldo] fp16 / bf16 bits
+    float* ws;              // [split][M][N] partial sums when split > 1
+    int ldx, ldo;
+    int M, N, K;
+    int G, steps, strips;
+    int zp_const;
+    int split;              // K splits across workgroups (grid.y)
+};
+int w2a16_auto_split(int M, int strips, int steps, int gs);
+hipError_t launch_w2a16(const W2A16Params& p, int gs, bool out_bf16, hipStream_t stream);
+
 hipError_t launch_tiled_generic(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
 
 }  // namespace w2a8

@@ -257,6 +257,39 @@ def w2a8_linear_fused(x: torch.Tensor, w: W2A8Weight, out_dtype=torch.float16, *
     return out
 
 
+def w2a16_gemm(x: torch.Tensor, w: W2A8Weight, out_dtype=torch.float16, *, split_k: int = 0,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The weight-only form: out[M, N] = x @ dequant(W)^T with the fp16 activations x [M, K] as they are (no
+    activation quantisation), the 2-bit codes widened to fp16 in front of the fp16 matrix cores, fp32 sums.
+    Built for few token rows; K must be a multiple of 128."""
+    L = _lib.lib()
+    _require_cuda(x, "x")
+    if x.dim() != 2 or x.dtype != torch.float16:
+        raise ValueError("x must be a 2-D float16 tensor [M, K]")
+    if out_dtype not in _DT:
+        raise ValueError("out_dtype must be torch.float16 or torch.bfloat16")
+    M, K = x.shape
+    if K != w.K:
+        raise ValueError(f"activation K={K} does not match weight K={w.K}")
+    if x.stride(1) != 1 or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
+        x = x.contiguous()
+    dev = x.device
+    if out is None:
+        out = torch.empty((M, w.N), dtype=out_dtype, device=dev)
+    with torch.cuda.device(dev):
+        ws_bytes = L.slimk_w2a16_gemm_workspace_bytes(M, w.N, K, w.group_size, split_k)
+        ws = getattr(w, "_partials16", None)      # its own buffer: the W2A8 workspace holds counters that must stay zero
+        if ws_bytes and (ws is None or ws.numel() < ws_bytes):
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            w._partials16 = ws
+        _lib.check(L.slimk_w2a16_gemm(
+            x.data_ptr(), x.stride(0), _DT[x.dtype], w.w_r.data_ptr(), w.s_r.data_ptr(),
+            w.zp_r.data_ptr() if w.zp_r is not None else None, w.zp_const, M, w.N, K, w.group_size,
+            out.data_ptr(), out.stride(0), _DT[out.dtype],
+            ws.data_ptr() if ws_bytes else None, ws.numel() if ws_bytes else 0, split_k, _stream_ptr(dev)))
+    return out
+
+
 def w2a8_gemm_grouped(problems, out_dtype=torch.float16):
     """Several independent skinny (M <= 32) GEMMs in one kernel launch.
 

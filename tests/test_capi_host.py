@@ -23,7 +23,7 @@ def L():
 def declared_symbols():
     text = open(HEADER, encoding="utf-8").read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(slimk_w2a8_\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(slimk_w2a(?:8|16)_\w+)\s*\(", text)))
 
 
 def test_every_declared_symbol_is_exported_and_bound(L):

@@ -1,0 +1,155 @@
+"""The weight-only form (fp16 activations times 2-bit weights on the fp16 matrix cores).
+
+Upstream's sketch is the notebook kernel ``w2matmul`` (slimkernels/triton/gemm_splitk.ipynb cell 1): 2-bit
+fields widened to fp16 in front of an fp32-accumulating ``tl.dot``; it carries no scales and no zero-point and has
+no test or stored output, so there is nothing of upstream's to compare numbers with.  The result is floating
+point: the GPU path is held to the float64 restatement within max(1 ULP of the output type, rtol 1e-3,
+2^-17 * sum of the terms' magnitudes) -- the last admits fp32 summation in the kernel's order and is far below
+what one dropped or misplaced term would change (1 / K of that sum)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from slimkernels_amd import _lib, workloads
+import parity_utils as pu
+
+FAKE = 0x10000
+
+
+def _weights(N, K, g, mode, seed):
+    case = pu.small_case(1, N, K, g, mode, seed)
+    packed, scales, zero = pu.quantized_weight(case)
+    return case, packed, scales, zero
+
+
+# ---------------------------------------------------------------- the oracle itself
+
+def test_oracle_by_hand():
+    from oracle import w2a8_oracle as o
+    # one token row, two channels, K = 4, one group: codes - zp = [-2, -1, 0, 1] and [1, 1, -2, 0]
+    x = np.array([[1.0, 2.0, -3.0, 0.5]], np.float16)
+    codes = np.array([[0, 1, 2, 3], [3, 3, 0, 2]], np.uint8)
+    scales = np.array([[0.5, 2.0]], np.float16)
+    zp = np.array([[2, 2]], np.uint8)
+    out, mag = o.w2a16_reference_forward(x, codes, scales, zp, 4)
+    assert out.tolist() == [[0.5 * (-2 - 2 + 0 + 0.5), 2.0 * (1 + 2 + 6 + 0)]]
+    assert mag.tolist() == [[0.5 * (2 + 2 + 0 + 0.5), 2.0 * (1 + 2 + 6 + 0)]]
+
+
+@pytest.mark.parametrize("mode", ["sym", "asym"])
+def test_oracle_against_a_library_matmul_and_plain_loops(mode):
+    from oracle import w2a8_oracle as o
+    case, packed, scales, zero = _weights(48, 256, 64, mode, seed=5)
+    codes = o.np_unpack(packed)
+    x = workloads.make_activation(pu.small_case(3, 48, 256, 64, mode, 5))
+    out, _ = o.w2a16_reference_forward(x, codes, scales, zero, 64)
+    # the dequantised weight times the activations through torch's matmul, in float64
+    deq = (codes.astype(np.float64) - np.repeat(zero.T.astype(np.float64), 64, axis=1)) * \
+        np.repeat(scales.T.astype(np.float64), 64, axis=1)
+    want = torch.from_numpy(x.astype(np.float64)) @ torch.from_numpy(deq).T
+    np.testing.assert_allclose(out, want.numpy(), rtol=1e-12, atol=1e-12)
+    # a few elements by plain Python loops
+    for m, n in ((0, 0), (2, 47), (1, 17)):
+        acc = 0.0
+        for k in range(256):
+            acc += float(x[m, k]) * (int(codes[n, k]) - int(zero[k // 64, n])) * float(scales[k // 64, n])
+        assert abs(acc - out[m, n]) <= 1e-9 * max(1.0, abs(acc))
+
+
+# ---------------------------------------------------------------- host side of the entry point
+
+def test_w2a16_validation():
+    L = _lib.lib()
+    g = L.slimk_w2a16_gemm
+    # (x, ldx, x_dtype, w_r, s_r, zp_r, zp_const, M, N, K, group, out, ldo, out_dtype, ws, ws_bytes, split, stream)
+    ok = [FAKE, 4096, 0, FAKE, FAKE, None, 2, 1, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 1, None]
+
+    def call(**kw):
+        names = ["x", "ldx", "xdt", "w", "s", "zp", "zpc", "M", "N", "K", "g", "out", "ldo", "odt", "ws", "wsb", "split", "st"]
+        a = list(ok)
+        for k, v in kw.items():
+            a[names.index(k)] = v
+        return g(*a)
+
+    assert call(x=None) == 1
+    assert call(M=0) == 2
+    assert call(K=4096 + 64, ldx=4160, g=64) == 7 and b"multiple of 128" in L.slimk_w2a8_last_error()
+    assert call(xdt=1) == 7 and b"fp16" in L.slimk_w2a8_last_error()      # bf16 activations
+    assert call(xdt=2) == 4 and call(odt=5) == 4
+    assert call(zpc=4) == 2
+    assert call(ldx=4000) == 2 and call(ldo=100) == 2
+    assert call(ldx=4100) == 3 and call(x=FAKE + 2) == 3
+    assert call(g=100) == 2
+    assert call(split=4) == 5 and b"workspace" in L.slimk_w2a8_last_error()
+    assert call(split=4, ws=FAKE, wsb=1024) == 5
+    assert call(split=65) == 2 and call(K=256, ldx=256, split=2) == 2     # more K-parts than there is K
+    assert call(M=1 << 20, ldx=4096) == 7                                 # 32-bit offsets
+
+
+def test_w2a16_split_and_workspace():
+    L = _lib.lib()
+    assert L.slimk_w2a16_gemm_auto_split_k(1, 28672, 8192, 128) >= 1
+    for M, N, K, g in ((1, 4096, 4096, 128), (16, 28672, 8192, 128), (4, 256, 256, 64), (1, 14336, 4096, 256)):
+        s = L.slimk_w2a16_gemm_auto_split_k(M, N, K, g)
+        granules = K // max(g, 128)
+        assert 1 <= s <= 64 and (s == 1 or s * 4 <= granules)
+        assert L.slimk_w2a16_gemm_workspace_bytes(M, N, K, g, 0) == (0 if s == 1 else s * M * N * 4)
+        assert L.slimk_w2a16_gemm_workspace_bytes(M, N, K, g, 3) == 3 * M * N * 4
+    assert L.slimk_w2a16_gemm_auto_split_k(1, 4096, 4096 + 64, 64) == 0   # K not a multiple of 128
+
+
+# ---------------------------------------------------------------- the GPU path against the oracle
+
+def _check(got: torch.Tensor, want, mag, bf16, what):
+    g = pu.bits_to_f32(pu.out_tensor_bits(got), bf16).astype(np.float64)
+    assert np.isfinite(g).all(), f"{what}: non-finite output"
+    tol = np.maximum(np.maximum(pu.ulp_of(want.astype(np.float32), bf16), 1e-3 * np.abs(want)), 2.0 ** -17 * mag)
+    diff = np.abs(g - want)
+    bad = diff > tol
+    assert not bad.any(), (f"{what}: {int(bad.sum())} of {bad.size} outputs off; worst |diff|/tol = "
+                           f"{float((diff / tol).max()):.3g} at {np.unravel_index(np.argmax(diff / tol), diff.shape)}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K,g,mode,out,split", [
+    (1, 256, 256, 128, "sym", "float16", 0),
+    (1, 4096, 4096, 128, "sym", "float16", 0),
+    (3, 200, 512, 64, "asym", "float16", 1),       # N not a multiple of 64, per-group zero-points, group 64
+    (16, 1024, 2048, 128, "asym", "bfloat16", 0),
+    (5, 320, 2048, 256, "sym", "float16", 2),      # group 256: a group spans two loop iterations
+    (7, 192, 1792, 64, "sym", "bfloat16", 3),      # K-parts of unequal length
+    (16, 128, 128, 64, "asym", "float16", 1),      # three of the four K-parts of a workgroup are empty
+    (40, 448, 1024, 128, "ref", "float16", 0),     # several blocks of 16 token rows, uniform zero-point 1
+    (2, 14336, 4096, 128, "sym", "float16", 0),
+])
+def test_w2a16_gemm_against_the_oracle(gpu_ops, oracle, M, N, K, g, mode, out, split):
+    print(f"W2A16 M={M} N={N} K={K} g={g} {mode} {out} split={split}", flush=True)
+    case = pu.small_case(M, N, K, g, mode, seed=M * 7 + N, out_dtype=out)
+    packed, scales, zero = pu.quantized_weight(case)
+    x = workloads.make_activation(case)
+    want, mag = oracle.w2a16_reference_forward(x, oracle.np_unpack(packed), scales, zero, g)
+    w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, x)
+    y = gpu_ops.w2a16_gemm(xd, w, pu.torch_dtype(case), split_k=split)
+    assert y.shape == (M, N)
+    _check(y, want, mag, out == "bfloat16", "W2A16")
+    # a second call (the partial-sum buffer is reused) and a strided activation give the same bits
+    wide = torch.zeros((M, K + 64), dtype=torch.float16, device="cuda")
+    wide[:, :K] = xd
+    y2 = gpu_ops.w2a16_gemm(wide[:, :K], w, pu.torch_dtype(case), split_k=split)
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
+
+
+@pytest.mark.gpu
+def test_w2a16_agrees_with_the_int8_path_to_the_activation_quantisation(gpu_ops):
+    """Same weights, same activations: the W2A8 result differs from the weight-only one only by the int8
+    rounding of the activations (per-token scale absmax / 127: relative error of a sum of K terms ~ 1 %)."""
+    case = pu.small_case(4, 512, 2048, 128, "sym", seed=3)
+    packed, scales, zero = pu.quantized_weight(case)
+    w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, workloads.make_activation(case))
+    a16 = gpu_ops.w2a16_gemm(xd, w).float()
+    a8 = gpu_ops.w2a8_gemm(gpu_ops.quantize_act_int8(xd, 128), w).float()
+    err = (a16 - a8).norm() / a16.norm()
+    print(f"relative L2 difference W2A16 vs W2A8: {err:.4f}", flush=True)
+    assert 0 < err < 0.03
