@@ -419,6 +419,25 @@ def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, d
                                            "GBps": round(bytes4 / (us * 1e-6) / 1e9, 1),
                                            "frac_hbm": round(bytes4 / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
                                            "note": "the int8 rows are laid down twice before the timed region (48 small copies, as act-quant is timed apart)"}
+
+    # ---- weight-only form: fp16 activations as they are, 2-bit codes widened to fp16 in front of the fp16 matrix
+    # cores (parity: tests/test_w2a16.py).  Bytes: N K / 4 + 2 N G (scales) + 2 M K + 2 M N.
+    torch.cuda.empty_cache()
+    a16rows = []
+    for (N, K, g, copies, Ms) in ((14336, 4096, 128, 24, (1, 16)), (28672, 8192, 128, 6, (1, 16))):
+        ws16 = [random_weight(N, K, g, False) for _ in range(copies)]
+        for M in Ms:
+            x = torch.randn(M, K, device=dev, dtype=torch.float16)
+            out = torch.empty((M, N), dtype=torch.float16, device=dev)
+            for w in ws16:
+                ops.w2a16_gemm(x, w, torch.float16, out=out)
+            us = time_graph(torch, lambda: [ops.w2a16_gemm(x, w, torch.float16, out=out) for w in ws16], len(ws16), replays=4)
+            nb = N * K // 4 + 2 * N * (K // g) + 2 * M * K + 2 * M * N
+            a16rows.append({"shape": f"{N}x{K}", "M": M, "group": g, "weights": "cold",
+                            "split_k": L.slimk_w2a16_gemm_auto_split_k(M, N, K, g), "us": round(us, 2),
+                            "GBps": round(nb / (us * 1e-6) / 1e9, 1), "frac_hbm": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)})
+        del ws16
+    detail["w2a16"] = a16rows
     return detail
 
 

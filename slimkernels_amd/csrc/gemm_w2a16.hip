@@ -7,17 +7,19 @@
 //
 // The weights are the repacked units of the W2A8 kernels (w2a8_common.h), read once.  A unit's dword i
 // holds, in 2-bit field p of byte b, the code of channel p*16 + col at k = quad*16 + 4*i + b.  Widening
-// without shifts: (dword & (0x00030003 << 2p)) | 0x64006400 is the fp16 pair (1024 + 4^p*code) of bytes 0
-// and 2, the same on (dword >> 8) the pair of bytes 1 and 3; one packed fp16 subtraction of
-// 1024 + 4^p*zp leaves 4^p * (code - zp), exact, and 4^-p goes into the fp32 scale.  The lane's eight
+// without shifts: dword & (0x00030003 << 2p), read as an fp16 pair, is the pair of subnormals
+// 4^p * code * 2^-24 of bytes 0 and 2, the same on (dword >> 8) the pair of bytes 1 and 3; one packed fp16
+// fma, x * 2^15 - 4^p * zp * 2^-9, leaves 4^p * 2^-9 * (code - zp), exact, and 2^9 * 4^-p goes into the
+// fp32 scale (fp16 subnormals are operands like any other here).  The lane's eight
 // k-values of one MFMA therefore come in the order 0,2,1,3,4,6,5,7; the activation operand is put in
 // the same order with two v_perm_b32 per register pair.
 //
-// Work split: a workgroup is four wavefronts that take four K-parts of ONE strip of 64 channels and
-// 16 token rows and add their sums up through LDS; blockIdx.y splits K further across workgroups
-// (fp32 partial sums to a workspace, summed in split order by a second kernel: deterministic).
-// Activations are read straight from global memory (they stay in L2; rows past M are out of range of the
-// buffer descriptor and read as zero without a memory access).
+// Work split: a workgroup is 4, 8 or 16 wavefronts that take as many K-parts of ONE strip of 64 channels and
+// 16 token rows and add their sums up through LDS; blockIdx.y splits K further across workgroups when the
+// strips alone would leave CUs idle (fp32 partial sums to a workspace, summed in split order by a second
+// kernel: deterministic).  Activations are read straight from global memory (they stay in L2; rows past M
+// are out of range of the buffer descriptor and read as zero without a memory access).  Every wave keeps
+// three chunks of 128 reduction elements of weights in flight while it works on a fourth.
 #include "w2a8_launch.h"
 
 namespace w2a8 {
@@ -25,15 +27,16 @@ namespace w2a8 {
 namespace {
 
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
-constexpr int kWaves = 4;        // K-parts per workgroup
 constexpr int kChunkSteps = 2;   // steps (of 64) per loop iteration
 
-// GS = steps per scale group (1, 2 or 4); ZP = per-group zero-points; PARTIAL = write fp32 partials
-template <int GS, bool ZP, bool PARTIAL, typename OutT>
-__global__ __launch_bounds__(256) void w2a16_kernel(const W2A16Params p) {
+// GS = steps per scale group (1, 2 or 4); kWaves = K-parts per workgroup (4, 8 or 16); ZP = per-group
+// zero-points; PARTIAL = write fp32 partial sums instead of the output
+template <int GS, int kWaves, bool ZP, bool PARTIAL, typename OutT>
+__global__ __launch_bounds__(kWaves * 64) void w2a16_kernel(const W2A16Params p) {
     __shared__ float red[kWaves][16][64];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -42,7 +45,7 @@ __global__ __launch_bounds__(256) void w2a16_kernel(const W2A16Params p) {
     const int strip = blockIdx.x;
     const int m0 = (int)blockIdx.z * 16;
 
-    // K-parts in granules of max(GS, 2) steps, dealt out evenly over split * 4 parts (a part may be empty)
+    // K-parts in granules of max(GS, 2) steps, dealt out evenly over split * kWaves parts (a part may be empty)
     constexpr int kGranule = GS > kChunkSteps ? GS : kChunkSteps;
     const int n_gran = p.steps / kGranule;
     const int parts = p.split * kWaves;
@@ -61,22 +64,29 @@ __global__ __launch_bounds__(256) void w2a16_kernel(const W2A16Params p) {
     const size_t sz_group = (size_t)p.strips * 64;                                      // elements between groups
 
     constexpr int kGPC = GS == 1 ? 2 : 1;  // scale groups that start or continue in one chunk
-    struct Chunk {
+    struct WChunk {
         v4i w[kChunkSteps];
+    };
+    struct AChunk {
         v4u a[kChunkSteps][2];
         uint2 s[kGPC];
         uint32_t z[kGPC];
     };
-    auto load = [&](int c) {
-        Chunk ch;
+    auto load_w = [&](int c) {
+        WChunk ch;
         const int st = step0 + c * kChunkSteps;
 #pragma unroll
-        for (int s = 0; s < kChunkSteps; ++s) {
-            ch.w[s] = *reinterpret_cast<const v4i*>(w_lane + (size_t)(st + s) * w_step);
+        for (int s = 0; s < kChunkSteps; ++s) ch.w[s] = *reinterpret_cast<const v4i*>(w_lane + (size_t)(st + s) * w_step);
+        return ch;
+    };
+    auto load_a = [&](int c) {
+        AChunk ch;
+        const int st = step0 + c * kChunkSteps;
+#pragma unroll
+        for (int s = 0; s < kChunkSteps; ++s)
 #pragma unroll
             for (int h = 0; h < 2; ++h)
                 ch.a[s][h] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_lane + (uint32_t)((st + s) * kStepK * 2 + h * 16), 0, 0);
-        }
 #pragma unroll
         for (int gi = 0; gi < kGPC; ++gi) {
             const int g = (st + gi) / GS;   // GS == 1: groups st, st + 1; otherwise the group of step st
@@ -95,70 +105,96 @@ __global__ __launch_bounds__(256) void w2a16_kernel(const W2A16Params p) {
         for (int j = 0; j < 4; ++j) t[pp][j] = 0.f;
     }
 
-    if (n_chunks > 0) {
-        Chunk cur = load(0);
-        for (int c = 0; c < n_chunks; ++c) {
-            const Chunk nxt = load(min(c + 1, n_chunks - 1));   // the last iteration re-reads its own chunk
+    auto compute = [&](const WChunk& cw, const AChunk& cur, int c) {
 #pragma unroll
-            for (int s = 0; s < kChunkSteps; ++s) {
-                const int gi = GS == 1 ? s : 0;
-                // 1024 + 4^p * zp as an fp16 pair, per sub-block
-                uint32_t zm[4];
+        for (int s = 0; s < kChunkSteps; ++s) {
+            const int gi = GS == 1 ? s : 0;
+            // -zp * 4^p * 2^-9 as an fp16 pair, per sub-block
+            v2h zneg[4];
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp) {
+                const uint32_t z = ZP ? (cur.z[gi] >> (8 * pp)) & 0xffu : (uint32_t)p.zp_const;
+                const _Float16 zh = (_Float16)(-(float)(z << (2 * pp)) * (1.0f / 512.0f));
+                zneg[pp] = v2h{zh, zh};
+            }
+            const v4i wf = cw.w[s] ^ (int)0x80808080u;      // field 3 is stored with its high bit flipped
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const v4u d = cur.a[s][h];
+                const v4u ap = {__builtin_amdgcn_perm(d[1], d[0], 0x05040100u), __builtin_amdgcn_perm(d[1], d[0], 0x07060302u),
+                                __builtin_amdgcn_perm(d[3], d[2], 0x05040100u), __builtin_amdgcn_perm(d[3], d[2], 0x07060302u)};
+                const uint32_t e0 = (uint32_t)wf[2 * h], e1 = (uint32_t)wf[2 * h + 1];
+                const uint32_t o0 = e0 >> 8, o1 = e1 >> 8;
 #pragma unroll
                 for (int pp = 0; pp < 4; ++pp) {
-                    const uint32_t z = ZP ? (cur.z[gi] >> (8 * pp)) & 0xffu : (uint32_t)p.zp_const;
-                    zm[pp] = (0x6400u | (z << (2 * pp))) * 0x00010001u;
-                }
-                const v4i wf = cur.w[s] ^ (int)0x80808080u;      // field 3 is stored with its high bit flipped
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const v4u d = cur.a[s][h];
-                    const v4u ap = {__builtin_amdgcn_perm(d[1], d[0], 0x05040100u), __builtin_amdgcn_perm(d[1], d[0], 0x07060302u),
-                                    __builtin_amdgcn_perm(d[3], d[2], 0x05040100u), __builtin_amdgcn_perm(d[3], d[2], 0x07060302u)};
-                    const uint32_t e0 = (uint32_t)wf[2 * h], e1 = (uint32_t)wf[2 * h + 1];
-                    const uint32_t o0 = e0 >> 8, o1 = e1 >> 8;
-#pragma unroll
-                    for (int pp = 0; pp < 4; ++pp) {
-                        const uint32_t mask = 0x00030003u << (2 * pp);
-                        const v4u braw = {(e0 & mask) | 0x64006400u, (o0 & mask) | 0x64006400u,
-                                          (e1 & mask) | 0x64006400u, (o1 & mask) | 0x64006400u};
-                        const v4u zraw = {zm[pp], zm[pp], zm[pp], zm[pp]};
-                        const v8h b = __builtin_bit_cast(v8h, braw) - __builtin_bit_cast(v8h, zraw);
-                        acc[pp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, ap), b, acc[pp], 0, 0, 0);
-                    }
-                }
-                // end of a scale group: fold the group's sums into the running sums
-                const bool group_ends = GS <= kChunkSteps ? ((s + 1) % GS == 0)
-                                                          : (((step0 + c * kChunkSteps + s + 1) % GS) == 0);
-                if (group_ends) {
-#pragma unroll
-                    for (int pp = 0; pp < 4; ++pp) {
-                        const uint32_t raw = pp < 2 ? cur.s[gi].x : cur.s[gi].y;
-                        const float sc = half_bits_to_float((uint16_t)((pp & 1) ? raw >> 16 : raw & 0xffffu)) *
-                                         (1.0f / (float)(1 << (2 * pp)));
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) t[pp][j] = __builtin_fmaf(acc[pp][j], sc, t[pp][j]);
-                        acc[pp] = v4f{0.f, 0.f, 0.f, 0.f};
-                    }
+                    const uint32_t mask = 0x00030003u << (2 * pp);
+                    // a masked field alone is an fp16 subnormal, 4^p * code * 2^-24: one packed fma per
+                    // register pair scales it by 2^15 and takes the zero-point off (exact)
+                    const v2h up = {(_Float16)32768.0f, (_Float16)32768.0f};
+                    const v2h b0 = __builtin_elementwise_fma(__builtin_bit_cast(v2h, e0 & mask), up, zneg[pp]);
+                    const v2h b1 = __builtin_elementwise_fma(__builtin_bit_cast(v2h, o0 & mask), up, zneg[pp]);
+                    const v2h b2 = __builtin_elementwise_fma(__builtin_bit_cast(v2h, e1 & mask), up, zneg[pp]);
+                    const v2h b3 = __builtin_elementwise_fma(__builtin_bit_cast(v2h, o1 & mask), up, zneg[pp]);
+                    const v8h b = {b0[0], b0[1], b1[0], b1[1], b2[0], b2[1], b3[0], b3[1]};
+                    acc[pp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, ap), b, acc[pp], 0, 0, 0);
                 }
             }
-            cur = nxt;
+            // end of a scale group: fold the group's sums into the running sums
+            const bool group_ends = GS <= kChunkSteps ? ((s + 1) % GS == 0)
+                                                      : (((step0 + c * kChunkSteps + s + 1) % GS) == 0);
+            if (group_ends) {
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) {
+                    const uint32_t raw = pp < 2 ? cur.s[gi].x : cur.s[gi].y;
+                    const float sc = half_bits_to_float((uint16_t)((pp & 1) ? raw >> 16 : raw & 0xffffu)) *
+                                     (512.0f / (float)(1 << (2 * pp)));
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) t[pp][j] = __builtin_fmaf(acc[pp][j], sc, t[pp][j]);
+                    acc[pp] = v4f{0.f, 0.f, 0.f, 0.f};
+                }
+            }
+        }
+    };
+    // The weights, which come from HBM, are fetched three (two) chunks ahead through a ring of buffers; the
+    // activations and scales, which come from L2, one chunk ahead (two buffers).  Past the end the fetches
+    // re-read the last chunk and nobody uses them.
+    constexpr int kAhead = kWaves == 16 ? 2 : 3;   // sixteen waves leave each 128 registers: a shorter ring
+    constexpr int kRing = kAhead + 1;
+    if (n_chunks > 0) {
+        const int last = n_chunks - 1;
+        WChunk wq[kRing];
+        AChunk aq[2];
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) wq[i] = load_w(min(i, last));
+        aq[0] = load_a(0);
+        // 2 * kRing chunks per trip, so that both ring positions are compile-time constants
+        for (int c = 0; c < n_chunks; c += 2 * kRing) {
+#pragma unroll
+            for (int i = 0; i < 2 * kRing; ++i) {
+                if (c + i < n_chunks) {
+                    wq[(i + kAhead) % kRing] = load_w(min(c + i + kAhead, last));
+                    aq[(i + 1) & 1] = load_a(min(c + i + 1, last));
+                    compute(wq[i % kRing], aq[i & 1], c + i);
+                }
+            }
         }
     }
 
-    // the four K-parts of the workgroup meet in LDS; wave w finishes sub-block w
+    // the K-parts of the workgroup meet in LDS; wave w finishes 16 / kWaves of the 16 accumulator rows
 #pragma unroll
     for (int pp = 0; pp < 4; ++pp)
 #pragma unroll
         for (int j = 0; j < 4; ++j) red[wave][pp * 4 + j][lane] = t[pp][j];
     __syncthreads();
-    const int n = strip * kStripN + wave * 16 + col;
+    constexpr int kRows = 16 / kWaves;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        float v = red[0][wave * 4 + j][lane];
+    for (int i = 0; i < kRows; ++i) {
+        const int r = wave * kRows + i, pp = r >> 2, j = r & 3;
+        float v = red[0][r][lane];
 #pragma unroll
-        for (int w = 1; w < kWaves; ++w) v += red[w][wave * 4 + j][lane];
+        for (int w = 1; w < kWaves; ++w) v += red[w][r][lane];
         const int m = m0 + quad * 4 + j;
+        const int n = strip * kStripN + pp * 16 + col;
         if (m < p.M && n < p.N) {
             if (PARTIAL) p.ws[((size_t)blockIdx.y * p.M + m) * p.N + n] = v;
             else reinterpret_cast<uint16_t*>(p.out)[(size_t)m * p.ldo + n] = OutT::cast(v);
@@ -177,44 +213,66 @@ __global__ __launch_bounds__(256) void w2a16_reduce_kernel(const float* __restri
     }
 }
 
-template <int GS, bool ZP, bool PARTIAL>
+template <int GS, int W, bool ZP, bool PARTIAL>
 void launch_one(const W2A16Params& p, bool out_bf16, dim3 grid, hipStream_t stream) {
-    if (out_bf16) w2a16_kernel<GS, ZP, PARTIAL, OutBF16><<<grid, dim3(256), 0, stream>>>(p);
-    else w2a16_kernel<GS, ZP, PARTIAL, OutF16><<<grid, dim3(256), 0, stream>>>(p);
+    if (out_bf16) w2a16_kernel<GS, W, ZP, PARTIAL, OutBF16><<<grid, dim3(W * 64), 0, stream>>>(p);
+    else w2a16_kernel<GS, W, ZP, PARTIAL, OutF16><<<grid, dim3(W * 64), 0, stream>>>(p);
+}
+
+template <int GS, int W>
+void launch_w(const W2A16Params& p, bool out_bf16, dim3 grid, hipStream_t stream) {
+    const bool zp = p.zp_r != nullptr, partial = p.split > 1;
+    if (zp) {
+        if (partial) launch_one<GS, W, true, true>(p, out_bf16, grid, stream);
+        else launch_one<GS, W, true, false>(p, out_bf16, grid, stream);
+    } else {
+        if (partial) launch_one<GS, W, false, true>(p, out_bf16, grid, stream);
+        else launch_one<GS, W, false, false>(p, out_bf16, grid, stream);
+    }
 }
 
 template <int GS>
-void launch_gs(const W2A16Params& p, bool out_bf16, dim3 grid, hipStream_t stream) {
-    const bool zp = p.zp_r != nullptr, partial = p.split > 1;
-    if (zp) {
-        if (partial) launch_one<GS, true, true>(p, out_bf16, grid, stream);
-        else launch_one<GS, true, false>(p, out_bf16, grid, stream);
-    } else {
-        if (partial) launch_one<GS, false, true>(p, out_bf16, grid, stream);
-        else launch_one<GS, false, false>(p, out_bf16, grid, stream);
-    }
+void launch_gs(const W2A16Params& p, int waves, bool out_bf16, dim3 grid, hipStream_t stream) {
+    if (waves == 16) launch_w<GS, 16>(p, out_bf16, grid, stream);
+    else if (waves == 8) launch_w<GS, 8>(p, out_bf16, grid, stream);
+    else launch_w<GS, 4>(p, out_bf16, grid, stream);
 }
 
 }  // namespace
 
-// K splits across workgroups: enough workgroups for about three per CU, every K-part at least two
-// granules (256 reduction elements at group size <= 128) long.
+// K splits across workgroups: one unless the strips (x blocks of 16 token rows) alone leave most CUs idle;
+// then enough for about one workgroup per CU, every K-part at least two granules (256 reduction elements at
+// group size <= 128) long.
 int w2a16_auto_split(int M, int strips, int steps, int gs) {
     const int granule = gs > kChunkSteps ? gs : kChunkSteps;
     const int n_gran = steps / granule;
     const long long base = (long long)strips * ((M + 15) / 16);
-    long long split = (768 + base - 1) / base;
-    const int cap = n_gran / (2 * kWaves);
+    if (base >= 192) return 1;
+    long long split = (256 + base - 1) / base;
+    const int cap = n_gran / (2 * 4);
     if (split > cap) split = cap;
     if (split > 64) split = 64;
     return split < 1 ? 1 : (int)split;
 }
 
+// K-parts inside a workgroup (4, 8 or 16 wavefronts): towards 16 wavefronts per CU over the whole launch,
+// every part at least two granules long where K allows.
+static int w2a16_waves(int M, int strips, int steps, int gs, int split) {
+    const int granule = gs > kChunkSteps ? gs : kChunkSteps;
+    const int n_gran = steps / granule;
+    const long long wgs = (long long)strips * ((M + 15) / 16) * split;
+    const long long wanted = 4096 / (wgs < 1 ? 1 : wgs);
+    int waves = wanted >= 12 ? 16 : wanted >= 6 ? 8 : 4;
+    while (waves > 4 && (long long)waves * split * 2 > n_gran) waves /= 2;
+    return waves;
+}
+
 hipError_t launch_w2a16(const W2A16Params& p, int gs, bool out_bf16, hipStream_t stream) {
     const dim3 grid((unsigned)p.strips, (unsigned)p.split, (unsigned)((p.M + 15) / 16));
-    if (gs == 1) launch_gs<1>(p, out_bf16, grid, stream);
-    else if (gs == 2) launch_gs<2>(p, out_bf16, grid, stream);
-    else launch_gs<4>(p, out_bf16, grid, stream);
+    const int waves = w2a16_waves(p.M, p.strips, p.steps, gs, p.split);
+    if (gs == 1) launch_gs<1>(p, waves, out_bf16, grid, stream);
+    else if (gs == 2) launch_gs<2>(p, waves, out_bf16, grid, stream);
+    else launch_gs<4>(p, waves, out_bf16, grid, stream);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     if (p.split > 1) {
         const size_t total = (size_t)p.M * p.N;
