@@ -17,6 +17,10 @@ Reference anchors (upstream SlimKernels tree):
   dequantizer       quantization.py:83-93
 The int8 activation quantizer, int32 accumulation and epilogue have no upstream
 counterpart; tests/test_oracle.py pins them by brute force and exact identities.
+The weight-only form (w2a16_reference_forward; upstream's sketch is the notebook kernel
+w2matmul, gemm_splitk.ipynb cell 1, which has no test and no stored output) is parity
+unpinned against upstream; tests/test_w2a16.py pins it by a hand case, torch's float64
+matmul on the dequantised weight and plain loops.
 """
 from __future__ import annotations
 

@@ -158,24 +158,34 @@ __global__ __launch_bounds__(kWaves * 64) void w2a16_kernel(const W2A16Params p)
     // The weights, which come from HBM, are fetched three (two) chunks ahead through a ring of buffers; the
     // activations and scales, which come from L2, one chunk ahead (two buffers).  Past the end the fetches
     // re-read the last chunk and nobody uses them.
-    constexpr int kAhead = kWaves == 16 ? 2 : 3;   // sixteen waves leave each 128 registers: a shorter ring
-    constexpr int kRing = kAhead + 1;
+    constexpr int kAhead = kWaves == 16 ? 1 : 3;   // sixteen waves leave each 128 registers: a shorter ring
+    constexpr int kRing = kAhead + 1;              // 4 or 2: even, so the two activation buffers alternate with it
     if (n_chunks > 0) {
         const int last = n_chunks - 1;
         WChunk wq[kRing];
         AChunk aq[2];
+        aq[0] = load_a(0);
 #pragma unroll
         for (int i = 0; i < kAhead; ++i) wq[i] = load_w(min(i, last));
-        aq[0] = load_a(0);
-        // 2 * kRing chunks per trip, so that both ring positions are compile-time constants
-        for (int c = 0; c < n_chunks; c += 2 * kRing) {
+        // whole trips of kRing chunks without a branch inside (a branch makes the compiler wait for every
+        // load in flight where the paths meet); the prefetches past the end re-read the last chunk
+        int c = 0;
+        for (; c + kRing <= n_chunks; c += kRing) {
 #pragma unroll
-            for (int i = 0; i < 2 * kRing; ++i) {
-                if (c + i < n_chunks) {
-                    wq[(i + kAhead) % kRing] = load_w(min(c + i + kAhead, last));
-                    aq[(i + 1) & 1] = load_a(min(c + i + 1, last));
-                    compute(wq[i % kRing], aq[i & 1], c + i);
-                }
+            for (int i = 0; i < kRing; ++i) {
+                // activations first: loads complete in issue order, so waiting for these next time
+                // leaves the younger weight fetches in flight
+                aq[(i + 1) & 1] = load_a(min(c + i + 1, last));
+                wq[(i + kAhead) % kRing] = load_w(min(c + i + kAhead, last));
+                compute(wq[i], aq[i & 1], c + i);
+            }
+        }
+        // the last chunks (fewer than kRing): their weights are already on the way
+#pragma unroll
+        for (int i = 0; i < kRing - 1; ++i) {
+            if (c + i < n_chunks) {
+                if (c + i + 1 < n_chunks) aq[(i + 1) & 1] = load_a(c + i + 1);
+                compute(wq[i], aq[i & 1], c + i);
             }
         }
     }
@@ -256,14 +266,13 @@ int w2a16_auto_split(int M, int strips, int steps, int gs) {
 }
 
 // K-parts inside a workgroup (4, 8 or 16 wavefronts): towards 16 wavefronts per CU over the whole launch,
-// every part at least two granules long where K allows.
+// every part at least four chunks (one trip of the main loop) long where K allows.
 static int w2a16_waves(int M, int strips, int steps, int gs, int split) {
-    const int granule = gs > kChunkSteps ? gs : kChunkSteps;
-    const int n_gran = steps / granule;
+    const int chunks = steps / kChunkSteps;
     const long long wgs = (long long)strips * ((M + 15) / 16) * split;
     const long long wanted = 4096 / (wgs < 1 ? 1 : wgs);
     int waves = wanted >= 12 ? 16 : wanted >= 6 ? 8 : 4;
-    while (waves > 4 && (long long)waves * split * 2 > n_gran) waves /= 2;
+    while (waves > 4 && (long long)waves * split * 4 > chunks) waves /= 2;
     return waves;
 }
 

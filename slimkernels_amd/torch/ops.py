@@ -386,3 +386,18 @@ class W2A8Linear(torch.nn.Module):
         if self.bias is not None:
             y = y + self.bias
         return y.reshape(*lead, self.out_features)
+
+
+class W2A16Linear(W2A8Linear):
+    """The same layer with the activations left in fp16 (weight-only quantisation): forward runs the
+    weight-only kernel, meant for a few token rows; the weight object and the constructors are W2A8Linear's."""
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, x.shape[-1])
+        if x2.dtype != torch.float16:
+            x2 = x2.to(torch.float16)
+        y = w2a16_gemm(x2, self.weight, self.out_dtype)
+        if self.bias is not None:
+            y = y + self.bias
+        return y.reshape(*lead, self.out_features)

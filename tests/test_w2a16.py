@@ -153,3 +153,22 @@ def test_w2a16_agrees_with_the_int8_path_to_the_activation_quantisation(gpu_ops)
     err = (a16 - a8).norm() / a16.norm()
     print(f"relative L2 difference W2A16 vs W2A8: {err:.4f}", flush=True)
     assert 0 < err < 0.03
+
+
+@pytest.mark.gpu
+def test_w2a16_linear_layer(gpu_ops, oracle):
+    """W2A16Linear against the float64 product with the dequantised weight, bias included, leading dimensions kept."""
+    from slimkernels_amd.quantization import prepare_w2
+    rng = np.random.default_rng(21)
+    w = (rng.standard_normal((192, 512)) * 0.02).astype(np.float32)
+    bias = torch.from_numpy(rng.standard_normal(192).astype(np.float16)).cuda()
+    lin = gpu_ops.W2A16Linear.from_float(w, 128, "sym", bias=bias)
+    packed, scales, zero = prepare_w2(w, 128, "sym")
+    x = rng.standard_normal((2, 3, 512)).astype(np.float16)
+    want, mag = oracle.w2a16_reference_forward(x.reshape(6, 512), oracle.np_unpack(packed), scales, zero, 128)
+    y = lin(torch.from_numpy(x).cuda())
+    assert y.shape == (2, 3, 192)
+    got = y.reshape(6, 192).float().cpu().numpy().astype(np.float64)
+    want = want + bias.float().cpu().numpy().astype(np.float64)[None, :]
+    tol = np.maximum(2e-3 * np.abs(want), 2.0 ** -17 * mag) + 2.0 ** -10 * np.abs(bias.float().cpu().numpy())[None, :] + 1e-4
+    assert (np.abs(got - want) <= tol).all(), float((np.abs(got - want) / tol).max())
