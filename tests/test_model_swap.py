@@ -61,13 +61,13 @@ def test_replace_linears_skips_what_it_cannot_take():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("bits", [2, 4])
-def test_llama_block_with_w2a8_linears(gpu_ops, bits):
+@pytest.mark.parametrize("bits,weight_only", [(2, False), (4, False), (2, True)])
+def test_llama_block_with_w2a8_linears(gpu_ops, bits, weight_only):
     model = _tiny_llama().half().cuda()
     quant = copy.deepcopy(model)
-    names = gpu_ops.replace_linears(quant, group_size=128, bits=bits)
+    names = gpu_ops.replace_linears(quant, group_size=128, bits=bits, weight_only=weight_only)
     assert len(names) == 14 and "lm_head" not in names            # 7 projections x 2 layers
-    layer_type = gpu_ops.W2A8Linear if bits == 2 else gpu_ops.W4A8Linear
+    layer_type = gpu_ops.W2A16Linear if weight_only else gpu_ops.W2A8Linear if bits == 2 else gpu_ops.W4A8Linear
     assert all(isinstance(dict(quant.named_modules())[n], layer_type) for n in names)
     ref = _dequantised_copy(model, names, 128, bits)
 

@@ -172,3 +172,33 @@ def test_w2a16_linear_layer(gpu_ops, oracle):
     want = want + bias.float().cpu().numpy().astype(np.float64)[None, :]
     tol = np.maximum(2e-3 * np.abs(want), 2.0 ** -17 * mag) + 2.0 ** -10 * np.abs(bias.float().cpu().numpy())[None, :] + 1e-4
     assert (np.abs(got - want) <= tol).all(), float((np.abs(got - want) / tol).max())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_w2a16_seeded_random_shapes(gpu_ops, oracle, seed):
+    """Ten drawn shapes per seed: ragged N, 1..40 token rows, K any multiple of 128 the group divides, all three group
+    sizes, every zero-point mode, both output types, forced and automatic K splits (a split the entry point refuses
+    for the shape is checked to be refused, not run)."""
+    rng = np.random.default_rng(1000 + seed)
+    for i in range(10):
+        g = int(rng.choice([64, 128, 256]))
+        K = int(rng.integers(1, 17)) * 256 if g == 256 else int(rng.integers(1, 33)) * 128
+        N = int(rng.integers(1, 700))
+        M = int(rng.choice([1, 2, 3, 4, 7, 16, 17, 33, 40]))
+        mode = str(rng.choice(["sym", "asym", "ref"]))
+        out = str(rng.choice(["float16", "bfloat16"]))
+        split = int(rng.choice([0, 0, 1, 2, 3, 5]))
+        print(f"W2A16 random seed={seed} #{i}: M={M} N={N} K={K} g={g} {mode} {out} split={split}", flush=True)
+        case = pu.small_case(M, N, K, g, mode, seed=seed * 100 + i, out_dtype=out)
+        packed, scales, zero = pu.quantized_weight(case)
+        x = workloads.make_activation(case)
+        w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, x)
+        granules = K // max(g, 128)
+        if split > 1 and split * 4 > granules:
+            with pytest.raises(_lib.SlimkError):
+                gpu_ops.w2a16_gemm(xd, w, pu.torch_dtype(case), split_k=split)
+            continue
+        want, mag = oracle.w2a16_reference_forward(x, oracle.np_unpack(packed), scales, zero, g)
+        y = gpu_ops.w2a16_gemm(xd, w, pu.torch_dtype(case), split_k=split)
+        _check(y, want, mag, out == "bfloat16", f"W2A16 seed {seed} case {i}")
