@@ -157,9 +157,11 @@ def quantize_act_int8(x: torch.Tensor, group_size: int = 128, copies: int = 1) -
     _require_cuda(x, "x")
     if x.dim() != 2 or x.dtype not in _DT:
         raise ValueError("x must be a 2-D float16 or bfloat16 tensor")
-    if x.stride(1) != 1:
-        x = x.contiguous()
     M, K = x.shape
+    if x.stride(1) != 1 or x.stride(0) % 8 != 0 or x.stride(0) < K or x.data_ptr() % 16 != 0:
+        x = x.contiguous()
+        if x.data_ptr() % 16 != 0:      # contiguous already, but not at a 16-byte boundary
+            x = x.clone()
     ldr = (M + 3) // 4 * 4
     copies = int(copies)
     q = torch.empty((M, max(copies, 1) * K), dtype=torch.int8, device=x.device)
@@ -241,8 +243,10 @@ def w2a8_linear_fused(x: torch.Tensor, w: W2A8Weight, out_dtype=torch.float16, *
         raise ValueError(f"activation K={K} does not match weight K={w.K}")
     if not fused_applies(M, K):
         raise ValueError(f"w2a8_linear_fused handles M <= {FUSED_MAX_ROWS} with M * K <= {FUSED_MAX_BYTES} (M={M}, K={K})")
-    if x.stride(1) != 1 or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
+    if x.stride(1) != 1 or x.stride(0) % 8 != 0 or x.stride(0) < K or x.data_ptr() % 16 != 0:
         x = x.contiguous()
+        if x.data_ptr() % 16 != 0:      # contiguous already, but not at a 16-byte boundary
+            x = x.clone()
     dev = x.device
     if out is None:
         out = torch.empty((M, w.N), dtype=out_dtype, device=dev)
@@ -271,8 +275,10 @@ def w2a16_gemm(x: torch.Tensor, w: W2A8Weight, out_dtype=torch.float16, *, split
     M, K = x.shape
     if K != w.K:
         raise ValueError(f"activation K={K} does not match weight K={w.K}")
-    if x.stride(1) != 1 or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
+    if x.stride(1) != 1 or x.stride(0) % 8 != 0 or x.stride(0) < K or x.data_ptr() % 16 != 0:
         x = x.contiguous()
+        if x.data_ptr() % 16 != 0:      # contiguous already, but not at a 16-byte boundary
+            x = x.clone()
     dev = x.device
     if out is None:
         out = torch.empty((M, w.N), dtype=out_dtype, device=dev)

@@ -202,3 +202,26 @@ def test_w2a16_seeded_random_shapes(gpu_ops, oracle, seed):
         want, mag = oracle.w2a16_reference_forward(x, oracle.np_unpack(packed), scales, zero, g)
         y = gpu_ops.w2a16_gemm(xd, w, pu.torch_dtype(case), split_k=split)
         _check(y, want, mag, out == "bfloat16", f"W2A16 seed {seed} case {i}")
+
+
+@pytest.mark.gpu
+def test_wrappers_take_awkward_activation_views(gpu_ops):
+    """Activations that the C entry points would refuse (row pitch not a multiple of 8, rows broadcast with pitch 0,
+    a start that is not 16-byte aligned) are copied by the wrappers: same bits as from a plain tensor."""
+    case = pu.small_case(3, 256, 512, 128, "sym", seed=9)
+    packed, scales, zero = pu.quantized_weight(case)
+    w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, workloads.make_activation(case))
+    pitch = torch.zeros((3, 516), dtype=torch.float16, device="cuda")
+    pitch[:, :512] = xd
+    shifted = torch.zeros((3 * 512 + 1,), dtype=torch.float16, device="cuda")
+    shifted[1:] = xd.reshape(-1)
+    views = {"pitch 516": pitch[:, :512], "offset 2 bytes": shifted[1:].reshape(3, 512)}
+    for what, v in views.items():
+        assert torch.equal(gpu_ops.w2a16_gemm(v, w), gpu_ops.w2a16_gemm(xd, w)), what
+        a, b = gpu_ops.quantize_act_int8(v, 128), gpu_ops.quantize_act_int8(xd, 128)
+        assert torch.equal(a.q, b.q) and torch.equal(a.s_a, b.s_a), what
+    row = xd[:1].expand(3, 512)                                   # pitch 0
+    y = gpu_ops.w2a16_gemm(row, w)
+    assert torch.equal(y[0], y[1]) and torch.equal(y[0], gpu_ops.w2a16_gemm(xd[:1], w)[0])
+    one = gpu_ops.w2a8_linear_fused(shifted[1:513].reshape(1, 512), w)
+    assert torch.equal(one, gpu_ops.w2a8_linear_fused(xd[:1].contiguous(), w))
