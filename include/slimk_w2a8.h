@@ -143,6 +143,20 @@ enum slimk_quant_mode {
 int slimk_w2a8_quantize_weight(const void* w, int ldw, int w_dtype, int N, int K, int group_size, int mode,
                                uint8_t* packed, int ldp, uint16_t* scales, uint8_t* zp, void* stream);
 
+/* Group-wise 4-bit weight quantisation on the GPU, written as the W2 operand over a reduction of 2K that the
+ * GEMM entry points take for 4-bit weights (see the top of this file): code = 4 * hi + lo,
+ *   planes  [N][ldp] uint8 : hi digits (code >> 2) in bytes 0 .. K/4-1 of a row, lo digits (code & 3) in bytes
+ *                            K/4 .. 2K/4-1, four digits per byte along K, first in bits 7:6; ldp >= K/2
+ *   scales2 [2G][N] fp16   : rows 0..G-1 = 4 * s, rows G..2G-1 = s
+ *   zp2     [2G][N] uint8  : rows 0..G-1 = zp >> 2, rows G..2G-1 = zp & 3
+ * mode SLIMK_QUANT_SYM: levels -8..7, s = max(absmax, 1e-9) / 8, zp = 8; SLIMK_QUANT_ASYM: s = max(max - min, 1e-9) / 15,
+ * zp = clip(rne(-min / s), 0, 15); binary32 arithmetic, IEEE division, round-half-even, s rounded to fp16 once: the
+ * numbers of this package's host functions (slimkernels_amd/w4.py: prepare_w4 + split_planes).  The outputs go to
+ * slimk_w2a8_repack with K' = 2K.  N <= 65535.  Alignment as for slimk_w2a8_quantize_weight.
+ * Upstream has no 4-bit quantiser (its W4 kernel runs on random codes, gemm_splitk.ipynb cell 2). */
+int slimk_w2a8_quantize_weight4(const void* w, int ldw, int w_dtype, int N, int K, int group_size, int mode,
+                                uint8_t* planes, int ldp, uint16_t* scales2, uint8_t* zp2, void* stream);
+
 /* Per-token activation quantisation (no upstream counterpart; upstream feeds FP8,
  * wgmma_sm90_W2A8.cu:533-536).
  *   x [M][ldx] fp16 or bf16 (x_dtype)

@@ -30,6 +30,7 @@ SIGNATURES = {
     "slimk_w2a8_workspace_init": (_i, [_vp, _sz, _vp]),
     "slimk_w2a8_repack": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "slimk_w2a8_quantize_weight": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp]),
+    "slimk_w2a8_quantize_weight4": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp]),
     "slimk_w2a8_act_quant": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _vp]),
     "slimk_w2a8_act_quant_rep": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _vp]),
     "slimk_w2a8_gemm": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i,

@@ -223,6 +223,22 @@ int slimk_w2a8_quantize_weight(const void* w, int ldw, int w_dtype, int N, int K
                       "quantize_weight");
 }
 
+int slimk_w2a8_quantize_weight4(const void* w, int ldw, int w_dtype, int N, int K, int group_size, int mode,
+                                uint8_t* planes, int ldp, uint16_t* scales2, uint8_t* zp2, void* stream) {
+    if (!w || !planes || !scales2 || !zp2) return fail(SLIMK_ERR_NULL_POINTER, "quantize_weight4: NULL buffer");
+    if (N <= 0 || N > 65535) return fail(SLIMK_ERR_BAD_SHAPE, "N=%d must be in 1..65535", N);
+    if (int rc = check_kg(K, group_size)) return rc;
+    if (w_dtype != SLIMK_F16 && w_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "w_dtype=%d", w_dtype);
+    if (mode != SLIMK_QUANT_SYM && mode != SLIMK_QUANT_ASYM) return fail(SLIMK_ERR_BAD_ENUM, "mode=%d (SYM or ASYM)", mode);
+    if (ldw < K || ldp < K / 2) return fail(SLIMK_ERR_BAD_SHAPE, "ldw=%d / ldp=%d too small for K=%d", ldw, ldp, K);
+    if (!aligned16(w) || ldw % 8 != 0 || (reinterpret_cast<uintptr_t>(planes) & 1u) || ldp % 2 != 0 ||
+        (reinterpret_cast<uintptr_t>(scales2) & 1u))
+        return fail(SLIMK_ERR_MISALIGNED, "quantize_weight4: w 16-byte aligned, ldw %% 8 == 0, planes / ldp / scales2 2-byte aligned");
+    return hip_result(w2a8::launch_quantize_weight4(w, ldw, w_dtype == SLIMK_BF16, N, K, group_size, mode == SLIMK_QUANT_ASYM,
+                                                    planes, ldp, scales2, zp2, (hipStream_t)stream),
+                      "quantize_weight4");
+}
+
 int slimk_w2a8_act_quant_rep(const void* x, int ldx, int x_dtype, int M, int K, int group_size, int copies,
                              int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, void* stream) {
     if (!x || !q || !s_a) return fail(SLIMK_ERR_NULL_POINTER, "act_quant: NULL buffer");

@@ -330,6 +330,84 @@ hipError_t launch_quantize_weight(const void* w, int ldw, bool w_bf16, int N, in
     return hipGetLastError();
 }
 
+// 4-bit weights as two 2-bit planes over 2K (the operand the W2 kernels take for W4): thread = 8 elements of a
+// row as above; codes 0..15 with s = max(absmax, 1e-9) / 8, zero 8 (asym false) or s = max(max - min, 1e-9) / 15,
+// zero = clip(rne(-min / s), 0, 15) (asym true).  The hi digits (code >> 2) go to bytes 0 .. K/4-1 of the row
+// with scales fp16(4 * fp16(s)) and zero-points zero >> 2 in rows 0 .. G-1; the lo digits (code & 3) to bytes
+// K/4 .. 2K/4-1 with scales fp16(s) and zero-points zero & 3 in rows G .. 2G-1.
+template <bool BF16>
+__global__ __launch_bounds__(256) void quantize_weight4_kernel(const uint16_t* __restrict__ w, int ldw, int N, int K,
+                                                               int group_size, int asym, uint8_t* __restrict__ packed,
+                                                               int ldp, uint16_t* __restrict__ scales,
+                                                               uint8_t* __restrict__ zp) {
+    const int n = blockIdx.y;
+    const int v = blockIdx.x * 256 + threadIdx.x;
+    const bool on = v < K / 8;
+    float f[8];
+    if (on) {
+        load8<BF16>(w + (size_t)n * ldw + (size_t)v * 8, f);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = 0.0f;
+    }
+    float hi = f[0], lo = f[0], amax = fabsf(f[0]);
+#pragma unroll
+    for (int i = 1; i < 8; ++i) {
+        hi = fmaxf(hi, f[i]);
+        lo = fminf(lo, f[i]);
+        amax = fmaxf(amax, fabsf(f[i]));
+    }
+    const int tpg = group_size / 8;
+    for (int off = 1; off < tpg; off <<= 1) {
+        hi = fmaxf(hi, __shfl_xor(hi, off, 64));
+        lo = fminf(lo, __shfl_xor(lo, off, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    }
+    const float tiny = 1e-9f;
+    float s, zero;
+    if (!asym) {
+        s = fmaxf(amax, tiny) / 8.0f;
+        zero = 8.0f;
+    } else {
+        s = fmaxf(hi - lo, tiny) / 15.0f;
+        zero = fminf(fmaxf(rintf(-lo / s), 0.0f), 15.0f);
+    }
+    if (!on) return;
+    uint32_t hi_bytes = 0, lo_bytes = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float level = fminf(fmaxf(rintf(f[i] / s) + zero, 0.0f), 15.0f);
+        const uint32_t code = (uint32_t)(int)level;
+        const int at = (i >> 2) * 8 + 6 - 2 * (i & 3);  // byte i / 4, first code of a byte in bits 7:6
+        hi_bytes |= (code >> 2) << at;
+        lo_bytes |= (code & 3u) << at;
+    }
+    uint8_t* row = packed + (size_t)n * ldp;
+    *reinterpret_cast<uint16_t*>(row + (size_t)v * 2) = (uint16_t)hi_bytes;
+    *reinterpret_cast<uint16_t*>(row + (size_t)(K / 4) + (size_t)v * 2) = (uint16_t)lo_bytes;
+    if (v % tpg == 0) {
+        const size_t g = (size_t)(v / tpg), G = (size_t)(K / group_size);
+        const _Float16 s16 = (_Float16)s;
+        scales[g * N + n] = __builtin_bit_cast(uint16_t, (_Float16)((float)s16 * 4.0f));
+        scales[(G + g) * N + n] = __builtin_bit_cast(uint16_t, s16);
+        const uint32_t z = (uint32_t)(int)zero;
+        zp[g * N + n] = (uint8_t)(z >> 2);
+        zp[(G + g) * N + n] = (uint8_t)(z & 3u);
+    }
+}
+
+hipError_t launch_quantize_weight4(const void* w, int ldw, bool w_bf16, int N, int K, int group_size, bool asym,
+                                   uint8_t* packed, int ldp, uint16_t* scales, uint8_t* zp, hipStream_t stream) {
+    const dim3 grid((unsigned)((K / 8 + 255) / 256), (unsigned)N), block(256);
+    if (w_bf16)
+        quantize_weight4_kernel<true><<<grid, block, 0, stream>>>((const uint16_t*)w, ldw, N, K, group_size, asym ? 1 : 0,
+                                                                 packed, ldp, scales, zp);
+    else
+        quantize_weight4_kernel<false><<<grid, block, 0, stream>>>((const uint16_t*)w, ldw, N, K, group_size, asym ? 1 : 0,
+                                                                  packed, ldp, scales, zp);
+    return hipGetLastError();
+}
+
 // ------------------------------------------------------------------ fill / probe
 __global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t* p, size_t n_dwords) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n_dwords; i += (size_t)gridDim.x * 256) p[i] = 0u;

@@ -20,6 +20,11 @@ hipError_t launch_act_quant(const void* x, int ldx, bool x_bf16, int M, int K, i
 hipError_t launch_quantize_weight(const void* w, int ldw, bool w_bf16, int N, int K, int group_size, int mode,
                                   uint8_t* packed, int ldp, uint16_t* scales, uint8_t* zp, hipStream_t stream);
 
+// 4-bit codes written as the two 2-bit planes over 2K that the W2 kernels take (packed [N][ldp >= 2K/4],
+// scales and zp [2G][N]); asym false: levels -8..7, true: per-group zero-points
+hipError_t launch_quantize_weight4(const void* w, int ldw, bool w_bf16, int N, int K, int group_size, bool asym,
+                                   uint8_t* packed, int ldp, uint16_t* scales, uint8_t* zp, hipStream_t stream);
+
 hipError_t launch_fill_zero(void* p, size_t bytes, hipStream_t stream);
 
 hipError_t launch_read_probe(const void* src, size_t bytes, uint32_t* sink, hipStream_t stream);

@@ -11,7 +11,8 @@ import numpy as np
 import torch
 
 from .. import w4 as host_w4
-from .ops import (QuantizedActivation, W2A8Weight, _DT, _require_cuda, fused_applies, quantize_act_int8, repack_w2,
+from .. import _lib
+from .ops import (QuantizedActivation, W2A8Weight, _DT, _require_cuda, _stream_ptr, fused_applies, quantize_act_int8, repack_w2,
                   w2a8_gemm, w2a8_linear_fused)
 
 
@@ -46,6 +47,36 @@ def repack_w4(packed4, scales, zp=None, group_size: int = 128, zp_const: int = 8
         zp = zp.cpu().numpy() if isinstance(zp, torch.Tensor) else np.asarray(zp)
     packed2, scales2, zp2 = host_w4.split_planes(host_w4.unpack_w4(packed4), scales, zp)
     return W4A8Weight(repack_w2(packed2, scales2, zp2, group_size, device=device), N, K, group_size)
+
+
+def quantize_weight4_gpu(weight_nk: torch.Tensor, group_size: int = 128, mode: str = "sym"):
+    """Group-wise 4-bit quantisation of an fp16 / bf16 weight [N, K] on the GPU, as the two 2-bit planes over 2K:
+    the same numbers as ``split_planes(unpack_w4(...prepare_w4(weight)))`` on the host.  Returns (planes uint8
+    [N, 2K/4], scales float16 [2G, N], zero-points uint8 [2G, N]) as device tensors, the inputs of repack_w2."""
+    L = _lib.lib()
+    _require_cuda(weight_nk, "weight")
+    if weight_nk.dim() != 2 or weight_nk.dtype not in _DT:
+        raise ValueError("weight must be a 2-D float16 or bfloat16 tensor [N, K]")
+    modes = {"sym": _lib.QUANT_SYM, "asym": _lib.QUANT_ASYM}
+    if mode not in modes:
+        raise ValueError(f"unknown quantizer mode {mode!r} (expected 'sym' or 'asym')")
+    w = weight_nk if weight_nk.stride(1) == 1 and weight_nk.stride(0) % 8 == 0 and weight_nk.data_ptr() % 16 == 0 \
+        else weight_nk.contiguous()
+    N, K = w.shape
+    if group_size not in (64, 128, 256) or K % group_size != 0:
+        raise ValueError(f"unsupported K={K}, group_size={group_size} (group_size in (64, 128, 256), K % group_size == 0)")
+    dev = w.device
+    G = K // group_size
+    planes = torch.empty((N, K // 2), dtype=torch.uint8, device=dev)
+    scales2 = torch.empty((2 * G, N), dtype=torch.float16, device=dev)
+    zp2 = torch.empty((2 * G, N), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(L.slimk_w2a8_quantize_weight4(w.data_ptr(), w.stride(0), _DT[w.dtype], N, K, group_size, modes[mode],
+                                                 planes.data_ptr(), planes.stride(0), scales2.data_ptr(), zp2.data_ptr(),
+                                                 _stream_ptr(dev)))
+        if w is not weight_nk:
+            torch.cuda.current_stream(dev).synchronize()  # the contiguous copy is consumed by the enqueued kernel
+    return planes, scales2, zp2
 
 
 def save_w4(path, packed4, scales, zp=None, group_size: int = 128, zp_const: int = 8):
@@ -127,6 +158,14 @@ class W4A8Linear(torch.nn.Module):
 
     @classmethod
     def from_float(cls, weight_nk, group_size=128, mode="sym", bias=None, out_dtype=torch.float16, device="cuda"):
+        if isinstance(weight_nk, torch.Tensor) and weight_nk.is_cuda and weight_nk.dtype in _DT:
+            # quantise where the weight already is (same numbers as the host path)
+            planes, scales2, zp2 = quantize_weight4_gpu(weight_nk.detach(), group_size, mode)
+            if not bool(torch.isfinite(scales2).all()):
+                raise ValueError("4 * scale overflows float16")
+            N, K = weight_nk.shape
+            return cls(W4A8Weight(repack_w2(planes, scales2, zp2, group_size, device=weight_nk.device), N, K, group_size),
+                       bias, out_dtype)
         w_np = weight_nk.detach().float().cpu().numpy() if isinstance(weight_nk, torch.Tensor) else np.asarray(weight_nk)
         packed4, scales, zero = host_w4.prepare_w4(w_np, group_size, mode)
         return cls(repack_w4(packed4, scales, zero, group_size, device=device), bias, out_dtype)

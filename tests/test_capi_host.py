@@ -136,6 +136,12 @@ def test_repack_and_act_quant_validation(L):
     assert qw(FAKE, 4096, 0, 64, 4096, 128, 3, FAKE, 1024, FAKE, None, None) == 4      # mode
     assert qw(FAKE, 4100, 0, 64, 4096, 128, 1, FAKE, 1024, FAKE, None, None) == 3      # ldw % 8
     assert qw(FAKE, 4096, 0, 64, 4096, 128, 1, FAKE + 1, 1024, FAKE, None, None) == 3
+    q4 = L.slimk_w2a8_quantize_weight4  # (w, ldw, dtype, N, K, group, mode, planes, ldp, scales2, zp2, stream)
+    assert q4(FAKE, 4096, 0, 64, 4096, 128, 1, FAKE, 2048, FAKE, None, None) == 1       # zero-points are always written
+    assert q4(FAKE, 4096, 0, 64, 4096, 128, 0, FAKE, 2048, FAKE, FAKE, None) == 4       # no REF mode at four bits
+    assert q4(FAKE, 4096, 0, 64, 4096, 128, 1, FAKE, 1024, FAKE, FAKE, None) == 2       # ldp < K/2
+    assert q4(FAKE, 4096, 0, 70000, 4096, 128, 1, FAKE, 2048, FAKE, FAKE, None) == 2
+    assert q4(FAKE, 4100, 0, 64, 4096, 128, 2, FAKE, 2048, FAKE, FAKE, None) == 3
     # (x, ldx, dtype, w_r, s_r, zp_r, zp_const, M, N, K, group, out, ldo, out_dtype, ws, ws_bytes, split, stream)
     gf = L.slimk_w2a8_gemm_fused
     assert gf(None, 4096, 0, FAKE, FAKE, None, 2, 1, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 0, None) == 1

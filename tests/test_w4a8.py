@@ -258,3 +258,37 @@ def test_w4a8_grouped_launch(gpu_ops, oracle):
     torch.cuda.synchronize()
     for (_, _, out), (ref, bound) in zip(probs, refs):
         pu.assert_out_close(pu.out_tensor_bits(out), ref["out_bits"], False, bound, "W4A8 grouped")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N,K,g,mode,bf16", [(64, 256, 64, "sym", False), (200, 1024, 128, "asym", False),
+                                             (96, 2048, 256, "sym", True), (33, 4096, 128, "asym", True)])
+def test_w4_quantisation_on_gpu_bit_exact(gpu_ops, N, K, g, mode, bf16):
+    """The GPU 4-bit quantiser writes the two planes, their scales and zero-points exactly as the host functions
+    do (prepare_w4 + split_planes); a group of equal values and an all-zero group are in the draw."""
+    print(f"W4 quantise on GPU: N={N} K={K} g={g} {mode} bf16={bf16}", flush=True)
+    rng = np.random.default_rng(N + K)
+    wt = torch.from_numpy((rng.standard_normal((N, K)) * 0.05).astype(np.float32))
+    wt[1, :g] = 0.0
+    wt[2, g:2 * g] = 0.03125
+    wt = wt.to(torch.bfloat16 if bf16 else torch.float16)
+    planes, scales2, zp2 = gpu_ops.quantize_weight4_gpu(wt.cuda(), g, mode)
+    packed4, scales, zero = w4.prepare_w4(wt.float().numpy(), g, mode)
+    want_planes, want_scales, want_zp = w4.split_planes(w4.unpack_w4(packed4), scales, zero)
+    assert np.array_equal(planes.cpu().numpy(), want_planes)
+    assert np.array_equal(scales2.cpu().numpy().view(np.uint16), want_scales.view(np.uint16))
+    assert np.array_equal(zp2.cpu().numpy(), want_zp)
+
+
+@pytest.mark.gpu
+def test_w4a8_linear_from_a_gpu_weight(gpu_ops):
+    """from_float on a CUDA fp16 weight quantises on the GPU: same layer as from the host path, bit for bit."""
+    from slimkernels_amd.torch import w4 as tw4
+    w, x = _w4_case(5, 192, 512, 128, "asym", seed=4)
+    w16 = torch.from_numpy(w).half()
+    a = tw4.W4A8Linear.from_float(w16.cuda(), 128, "asym")
+    b = tw4.W4A8Linear.from_float(w16.float().numpy(), 128, "asym")
+    assert torch.equal(a.weight.planes.w_r, b.weight.planes.w_r) and torch.equal(a.weight.planes.s_r, b.weight.planes.s_r)
+    assert torch.equal(a.weight.planes.zp_r, b.weight.planes.zp_r)
+    xd = torch.from_numpy(x).cuda()
+    assert torch.equal(a(xd), b(xd))
