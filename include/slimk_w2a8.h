@@ -37,7 +37,13 @@
  * a code c = 4 * hi + lo is two 2-bit digits, and a W4 GEMM over K with G groups
  * is these calls over K' = 2K with 2G groups -- columns 0..K-1 the hi digits with
  * scales 4 * s and zero-points zp >> 2, columns K..2K-1 the lo digits with scales
- * s and zero-points zp & 3 -- against q and its row sums laid down twice.
+ * s and zero-points zp & 3 -- against q and its row sums laid down twice
+ * (slimk_w2a8_act_quant_rep writes them so; slimk_w2a8_quantize_weight4 quantises
+ * a weight straight into the two planes).
+ *
+ * The weight-only form (fp16 activations as they are, upstream's notebook kernel
+ * w2matmul) is slimk_w2a16_gemm at the end of this file; it takes the same
+ * repacked weights.
  */
 #ifndef SLIMK_W2A8_H
 #define SLIMK_W2A8_H
