@@ -226,7 +226,12 @@ def main():
             "steps": steps1, "GBps": round(step_bytes * steps1 / wall1 / 1e9, 2), "ms_per_step": round(wall1 * 1e3 / steps1, 5),
             "avg_launch_us": round(us1, 3),
             "frac_hbm": round(step_bytes / len(cases) / (us1 * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
-        detail.update(collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, dev))
+        try:
+            detail.update(collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, dev))
+        except Exception as e:  # the side rows must not take the headline line down with them; say what happened
+            import traceback
+            traceback.print_exc(file=sys.stderr)
+            detail["detail_error"] = repr(e)
         result["cpu_baseline"] = cpu_baseline(np, workloads, shapes)
     else:
         result["cpu_baseline"] = None
