@@ -402,9 +402,18 @@ def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, d
             G = K // g
             nb = N * K // 2 + 2 * N * G + N * G // 2 + M * K + 4 * M + 2 * M * N
             nops = 2 * M * N * K
-            w4rows.append({"shape": f"{N}x{K}", "M": M, "group": g, "weights": "cold" if cold else "warm", "us": round(us, 2),
+            w4rows.append({"shape": f"{N}x{K}", "M": M, "group": g, "weights": "cold" if cold else "warm", "kernel": "two planes over 2K",
+                           "us": round(us, 2),
                            "GBps": round(nb / (us * 1e-6) / 1e9, 1), "frac_hbm": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
                            "TOPS": round(nops / (us * 1e-6) / 1e12, 1), "frac_int8_mfma": round(nops / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4)})
+            if not cold:
+                # symmetric weights, many rows: the digits joined in front of the matrix core, one pass over K
+                w1 = tw4.W4A8Weight(use[0].planes, N, K, g, uniform_zp8=True)
+                tw4.w4a8_gemm_one_pass(qa, w1, torch.float16, out=out)
+                us = time_graph(torch, lambda: [tw4.w4a8_gemm_one_pass(qa, w1, torch.float16, out=out) for _ in range(4)], 4, replays=4)
+                w4rows.append({"shape": f"{N}x{K}", "M": M, "group": g, "weights": "warm", "kernel": "one pass (zero-point 8)",
+                               "us": round(us, 2), "TOPS": round(nops / (us * 1e-6) / 1e12, 1),
+                               "frac_int8_mfma": round(nops / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4)})
         del ws4
     detail["w4a8"] = w4rows
 

@@ -253,6 +253,22 @@ typedef struct slimk_w2a8_problem {
 int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int group_size, int out_dtype,
                             void* stream);
 
+/* 4-bit weights with the uniform zero-point 8 (levels -8..7) in ONE pass over K, for many token rows: the tiled
+ * kernel fetches the hi and the lo digit of every weight and puts them together in front of the matrix core
+ * (the int8 operand is 16 * (code - 8)), instead of running the two planes as a reduction over 2K.
+ *   q [M][ldq], s_a [M]   : slimk_w2a8_act_quant over K (laid down once; no row sums are needed)
+ *   w_r, s_r              : slimk_w2a8_repack of the two planes with K' = 2K (hi digits first) and their scales
+ *                           [2G][N] (4 * s, then s), e.g. the outputs of slimk_w2a8_quantize_weight4 in mode SYM;
+ *                           the planes' zero-points must be 2 (hi) and 0 (lo) -- they are not read here
+ *   M, N, K, group_size   : K is the reduction length of the 4-bit matrix (not 2K); K % 128 == 0, group_size 64 or 128
+ * int32 sums per group are exact; the result differs from the two-plane route only in fp32 summation order (G terms
+ * instead of 2G).  Any M works; few token rows are better served by slimk_w2a8_gemm over the planes.
+ * Replaces upstream's w4matmul_splitk (slimkernels/triton/gemm_splitk.ipynb cell 0) for the many-rows regime. */
+int slimk_w4a8_gemm(const int8_t* q, int ldq, const float* s_a,
+                    const uint32_t* w_r, const uint16_t* s_r,
+                    int M, int N, int K, int group_size,
+                    void* out, int ldo, int out_dtype, void* stream);
+
 /* Weight-only form: x [M][ldx] fp16 activations are NOT quantised; the 2-bit codes are widened to fp16 in
  * front of the fp16 matrix cores and every scale group's fp32 sum is scaled into the fp32 result:
  *   out[m][n] = cast( sum_g scales[g][n] * sum_{k in g} x[m][k] * (code[n][k] - zp[g][n]) ).

@@ -518,6 +518,28 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
                       "grouped skinny gemm");
 }
 
+int slimk_w4a8_gemm(const int8_t* q, int ldq, const float* s_a,
+                    const uint32_t* w_r, const uint16_t* s_r,
+                    int M, int N, int K, int group_size,
+                    void* out, int ldo, int out_dtype, void* stream) {
+    if (!q || !s_a || !w_r || !s_r || !out) return fail(SLIMK_ERR_NULL_POINTER, "w4a8_gemm: NULL buffer");
+    if (M <= 0 || N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "M=%d, N=%d must be positive", M, N);
+    if (int rc = check_kg(K, group_size)) return rc;
+    if (K % 128 != 0 || group_size > 128)
+        return fail(SLIMK_ERR_UNSUPPORTED, "w4a8_gemm: K=%d must be a multiple of 128 and group_size=%d 64 or 128", K, group_size);
+    if (out_dtype != SLIMK_F16 && out_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "out_dtype=%d", out_dtype);
+    if (ldq < K || ldo < N) return fail(SLIMK_ERR_BAD_SHAPE, "ldq=%d / ldo=%d too small for K=%d / N=%d", ldq, ldo, K, N);
+    if (2LL * K > 0x7fffffff) return fail(SLIMK_ERR_UNSUPPORTED, "K=%d too long", K);
+    if (int rc = check_extent(M, N, 2 * K, ldq)) return rc;
+    if (!aligned16(q) || ldq % 16 != 0 || !aligned16(w_r) || !aligned16(s_r) || (reinterpret_cast<uintptr_t>(out) & 1u))
+        return fail(SLIMK_ERR_MISALIGNED, "w4a8_gemm: q, w_r, s_r must be 16-byte aligned; ldq %% 16 == 0; out 2-byte aligned");
+    w2a8::GemmParams p{};
+    p.q = q; p.s_a = s_a; p.w_r = w_r; p.s_r = s_r; p.out = out; p.ldq = ldq; p.ldo = ldo;
+    p.M = M; p.N = N; p.K = K; p.G = K / group_size; p.steps = K / w2a8::kStepK; p.strips = strips_of(N);
+    p.zp_const = 2; p.split = 1; p.groups_per_split = p.G;
+    return hip_result(w2a8::launch_tiled_w4(p, group_size / w2a8::kStepK, out_dtype == SLIMK_BF16, (hipStream_t)stream), "w4a8_gemm");
+}
+
 int slimk_w2a16_gemm_auto_split_k(int M, int N, int K, int group_size) {
     if (M <= 0 || N <= 0 || !shape_ok(K, group_size) || K % 128 != 0) return 0;
     return w2a8::w2a16_auto_split(M, strips_of(N), K / w2a8::kStepK, group_size / w2a8::kStepK);

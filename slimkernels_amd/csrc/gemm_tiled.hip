@@ -39,7 +39,11 @@ constexpr int kAQueue = 4;                                 // activation fragmen
 
 // BM = token rows of the workgroup tile: 128, or 64 when 128-row tiles would leave CUs idle
 // (fewer tiles than CUs, or a single workgroup per CU with nothing to hide its latencies behind).
-template <int BM, int GS, bool SPLIT, bool ZP, typename OutT>
+// W4: 4-bit weights held as two 2-bit planes (hi digits in steps 0 .. steps-1 of w_r, lo digits in steps
+// steps .. 2*steps-1; s_r rows 0 .. G-1 = 4 * scale) with the uniform zero-point 8.  Both digits of a step are fetched
+// and put together before the MFMA: the operand byte 64 * (hi - 2) | 16 * lo is 16 * (code - 8), and the hi plane's
+// scale times the 1/64 of the 2-bit path is scale / 16: one pass over K instead of two over 2K.
+template <int BM, int GS, bool SPLIT, bool ZP, typename OutT, bool W4 = false>
 __device__ __forceinline__ void tiled_body(const GemmParams& p) {
     using namespace fast;
     constexpr int kBM = BM;
@@ -47,7 +51,8 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
     constexpr int kABlocks = kMB * kStageSteps;    // activation blocks per stage (16 or 8)
     constexpr int kStageDwords = kABlocks * 256;   // 16 or 8 KiB of activations per stage
     constexpr int kALoads = kABlocks / 4;          // LDS-direct activation block loads per wave and stage
-    constexpr int kWDwords = kStrips * kStageSteps * 256;  // the four waves' weight units of a stage: 8 KiB
+    constexpr int kWPlanes = W4 ? 2 : 1;
+    constexpr int kWDwords = kStrips * kStageSteps * 256 * kWPlanes;  // the four waves' weight units of a stage: 8 KiB a plane
     constexpr int kBufDwords = kStageDwords + kWDwords;
     constexpr int kBufs = 3;                       // stage s+2 is in flight while stage s is consumed
     __shared__ __attribute__((aligned(16))) uint32_t lds[kBufs][kBufDwords];
@@ -96,7 +101,7 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
     const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<int8_t*>(p.q), 0, (int)min((size_t)p.M * p.ldq, (size_t)0x7fffffff), 0x00020000);
     const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint32_t*>(p.w_r), 0, (int)min((size_t)p.strips * p.steps * (kUnitDwords * 4), (size_t)0x7fffffff), 0x00020000);
+        const_cast<uint32_t*>(p.w_r), 0, (int)min((size_t)p.strips * p.steps * (kUnitDwords * 4) * kWPlanes, (size_t)0x7fffffff), 0x00020000);
     const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(p.s_r), 0, (int)min((size_t)p.strips * p.G * 128, (size_t)0x7fffffff), 0x00020000);
     uint32_t a_off[kALoads];
@@ -114,7 +119,7 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
     v2u sraw[kGroupsPerStage];
     // Activations and this wave's weight units go straight from global memory into LDS (no registers
     // held while in flight), two stages ahead; the scales, a few bytes, go to registers one stage ahead.
-    constexpr int kLdsLoads = kALoads + kStageSteps;  // LDS-direct loads a wave issues per stage
+    constexpr int kLdsLoads = kALoads + kStageSteps * kWPlanes;  // LDS-direct loads a wave issues per stage
     auto fetch = [&](int stage, int buf) {
 #pragma unroll
         for (int i = 0; i < kALoads; ++i)
@@ -126,6 +131,13 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
                 w_rsrc, (__attribute__((address_space(3))) void*)&lds[buf][kStageDwords + (wave * kStageSteps + s) * 256], 16,
                 lane * 16, ((stage0 + stage) * kStageSteps + s) * b_step_stride + b_strip_off, 0, 0);
+        if constexpr (W4) {
+#pragma unroll
+            for (int s = 0; s < kStageSteps; ++s)   // the lo digits of the same steps: p.steps units further on
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                    w_rsrc, (__attribute__((address_space(3))) void*)&lds[buf][kStageDwords + kWDwords / 2 + (wave * kStageSteps + s) * 256], 16,
+                    lane * 16, ((stage0 + stage) * kStageSteps + s + p.steps) * b_step_stride + b_strip_off, 0, 0);
+        }
     };
     auto fetch_scales = [&](int stage) {
 #pragma unroll
@@ -244,6 +256,14 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
 #pragma unroll
             for (int pp = 0; pp < 3; ++pp) b[s][pp] = (wf << (6 - 2 * pp)) & (int)0xc0c0c0c0u;
             b[s][3] = w & (int)0xc0c0c0c0u;  // field 3 is stored already flipped
+            if constexpr (W4) {
+                typedef unsigned v4w __attribute__((ext_vector_type(4)));
+                const v4w wl = __builtin_bit_cast(v4w, *reinterpret_cast<const v4i*>(la + kStageDwords + kWDwords / 2 + (wave * kStageSteps + s) * 256));
+                b[s][0] |= __builtin_bit_cast(v4i, (wl << 4) & 0x30303030u);
+                b[s][1] |= __builtin_bit_cast(v4i, (wl << 2) & 0x30303030u);
+                b[s][2] |= __builtin_bit_cast(v4i, wl & 0x30303030u);
+                b[s][3] |= __builtin_bit_cast(v4i, ((wl ^ 0x80808080u) >> 2) & 0x30303030u);  // stored flipped: back to the code
+            }
         }
 
         // the scales of the next stage first, then the stage after next into the buffer that stage - 1 used
@@ -431,6 +451,26 @@ __global__ __launch_bounds__(256, 2) void tiled_kernel(const GemmParams p) {
 template <int GS, bool SPLIT, bool ZP, typename OutT>
 __global__ __launch_bounds__(256, 3) void tiled_kernel_bm64(const GemmParams p) {
     tiled_body<64, GS, SPLIT, ZP, OutT>(p);
+}
+
+// 4-bit weights, one pass (64-row tiles: three stage buffers of 24 KiB leave room for two workgroups on a CU)
+template <int GS, typename OutT>
+__global__ __launch_bounds__(256, 2) void tiled_kernel_w4(const GemmParams p) {
+    tiled_body<64, GS, false, false, OutT, true>(p);
+}
+
+hipError_t launch_tiled_w4(const GemmParams& p, int gs, bool out_bf16, hipStream_t stream) {
+    const int tiles_n = (p.strips + fast::kStrips - 1) / fast::kStrips;
+    const int tiles = tiles_n * ((p.M + 63) / 64);
+    const dim3 grid((tiles + 7) / 8 * 8, 1), block(256);
+    if (gs == 1) {
+        if (out_bf16) tiled_kernel_w4<1, OutBF16><<<grid, block, 0, stream>>>(p);
+        else tiled_kernel_w4<1, OutF16><<<grid, block, 0, stream>>>(p);
+    } else {
+        if (out_bf16) tiled_kernel_w4<2, OutBF16><<<grid, block, 0, stream>>>(p);
+        else tiled_kernel_w4<2, OutF16><<<grid, block, 0, stream>>>(p);
+    }
+    return hipGetLastError();
 }
 
 bool tiled_fast_supported(const GemmParams& p, int gs, bool asym) {

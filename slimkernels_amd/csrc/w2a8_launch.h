@@ -69,6 +69,9 @@ struct W2A16Params {
 int w2a16_auto_split(int M, int strips, int steps, int gs);
 hipError_t launch_w2a16(const W2A16Params& p, int gs, bool out_bf16, hipStream_t stream);
 
+// 4-bit weights as two planes (w_r over 2 * p.steps steps, s_r over 2 * p.G groups), uniform zero-point 8, one pass
+// over K: p.K / p.steps / p.G describe K, not 2K; gs 1 or 2; p.steps even
+hipError_t launch_tiled_w4(const GemmParams& p, int gs, bool out_bf16, hipStream_t stream);
 hipError_t launch_tiled_generic(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
 
 }  // namespace w2a8

@@ -23,6 +23,7 @@ class W4A8Weight:
     N: int
     K: int
     group_size: int
+    uniform_zp8: bool = False   # every zero-point is 8 (the symmetric levels): the one-pass kernel applies
 
     @property
     def device(self):
@@ -46,7 +47,8 @@ def repack_w4(packed4, scales, zp=None, group_size: int = 128, zp_const: int = 8
     else:
         zp = zp.cpu().numpy() if isinstance(zp, torch.Tensor) else np.asarray(zp)
     packed2, scales2, zp2 = host_w4.split_planes(host_w4.unpack_w4(packed4), scales, zp)
-    return W4A8Weight(repack_w2(packed2, scales2, zp2, group_size, device=device), N, K, group_size)
+    return W4A8Weight(repack_w2(packed2, scales2, zp2, group_size, device=device), N, K, group_size,
+                      uniform_zp8=bool((zp == 8).all()))
 
 
 def quantize_weight4_gpu(weight_nk: torch.Tensor, group_size: int = 128, mode: str = "sym"):
@@ -98,7 +100,10 @@ def load_w4_weight(path, device="cuda", mmap=True) -> W4A8Weight:
     if d["mode"] != "w4planes" or d["zp"] is None or d["K"] % 2 != 0:
         raise ValueError(f"{path}: not a two-plane W4 file (mode {d['mode']!r})")
     planes = repack_w2(d["packed"], d["scales"], d["zp"], d["group_size"], device=device)
-    return W4A8Weight(planes, d["N"], d["K"] // 2, d["group_size"])
+    G = d["K"] // 2 // d["group_size"]
+    zp = np.asarray(d["zp"])
+    return W4A8Weight(planes, d["N"], d["K"] // 2, d["group_size"],
+                      uniform_zp8=bool((zp[:G] == 2).all() and (zp[G:] == 0).all()))
 
 
 def activation_twice(qa: QuantizedActivation) -> QuantizedActivation:
@@ -124,6 +129,34 @@ def w4a8_gemm(qa: QuantizedActivation, w: W4A8Weight, out_dtype=torch.float16, *
     return y, acc[:, :, :G] * 4 + acc[:, :, G:]
 
 
+ONE_PASS_MIN_ROWS = 64   # from here on the matrix cores bound the time and one pass over K beats two planes over 2K
+
+
+def one_pass_applies(M: int, w: W4A8Weight) -> bool:
+    return w.uniform_zp8 and M >= ONE_PASS_MIN_ROWS and w.K % 128 == 0 and w.group_size in (64, 128)
+
+
+def w4a8_gemm_one_pass(qa: QuantizedActivation, w: W4A8Weight, out_dtype=torch.float16,
+                       out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The many-rows kernel for 4-bit weights with zero-point 8: hi and lo digit are put together in front of the
+    matrix core, one pass over K.  ``qa`` = quantize_act_int8(x) over K (laid down once)."""
+    M, K = qa.q.shape
+    if K != w.K or qa.group_size != w.group_size:
+        raise ValueError(f"activation K={K}/group {qa.group_size} does not match weight K={w.K}/group {w.group_size}")
+    if not w.uniform_zp8:
+        raise ValueError("the one-pass kernel needs the uniform zero-point 8 (symmetric levels)")
+    if out_dtype not in _DT:
+        raise ValueError("out_dtype must be torch.float16 or torch.bfloat16")
+    dev = qa.q.device
+    if out is None:
+        out = torch.empty((M, w.N), dtype=out_dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().slimk_w4a8_gemm(qa.q.data_ptr(), qa.q.stride(0), qa.s_a.data_ptr(), w.planes.w_r.data_ptr(),
+                                              w.planes.s_r.data_ptr(), M, w.N, K, w.group_size, out.data_ptr(),
+                                              out.stride(0), _DT[out.dtype], _stream_ptr(dev)))
+    return out
+
+
 def w4a8_gemm_grouped(problems, out_dtype=torch.float16):
     """Several independent W4A8 GEMMs of at most 32 token rows in ONE launch (the grouped kernel of the W2 path):
     ``problems`` is a list of (qa, w4, out) with ``qa`` = quantize_act_int8(x) over K, ``w4`` a W4A8Weight and
@@ -142,6 +175,8 @@ def w4a8_linear(x: torch.Tensor, w: W4A8Weight, out_dtype=torch.float16) -> torc
         raise ValueError(f"activation K={x.shape[1]} does not match weight K={w.K}")
     if x.shape[0] == 1 and fused_applies(1, 2 * w.K):
         return w2a8_linear_fused(torch.cat([x, x], dim=1), w.planes, out_dtype)
+    if one_pass_applies(x.shape[0], w):
+        return w4a8_gemm_one_pass(quantize_act_int8(x, w.group_size), w, out_dtype)
     # one quantisation launch writes the row and its group sums twice: the operand over 2K
     return w2a8_gemm(quantize_act_int8(x, w.group_size, copies=2), w.planes, out_dtype)
 
@@ -164,8 +199,8 @@ class W4A8Linear(torch.nn.Module):
             if not bool(torch.isfinite(scales2).all()):
                 raise ValueError("4 * scale overflows float16")
             N, K = weight_nk.shape
-            return cls(W4A8Weight(repack_w2(planes, scales2, zp2, group_size, device=weight_nk.device), N, K, group_size),
-                       bias, out_dtype)
+            return cls(W4A8Weight(repack_w2(planes, scales2, zp2, group_size, device=weight_nk.device), N, K, group_size,
+                                  uniform_zp8=mode == "sym"), bias, out_dtype)
         w_np = weight_nk.detach().float().cpu().numpy() if isinstance(weight_nk, torch.Tensor) else np.asarray(weight_nk)
         packed4, scales, zero = host_w4.prepare_w4(w_np, group_size, mode)
         return cls(repack_w4(packed4, scales, zero, group_size, device=device), bias, out_dtype)

@@ -23,7 +23,7 @@ def L():
 def declared_symbols():
     text = open(HEADER, encoding="utf-8").read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(slimk_w2a(?:8|16)_\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(slimk_w(?:2a8|2a16|4a8)_\w+)\s*\(", text)))
 
 
 def test_every_declared_symbol_is_exported_and_bound(L):
@@ -136,6 +136,13 @@ def test_repack_and_act_quant_validation(L):
     assert qw(FAKE, 4096, 0, 64, 4096, 128, 3, FAKE, 1024, FAKE, None, None) == 4      # mode
     assert qw(FAKE, 4100, 0, 64, 4096, 128, 1, FAKE, 1024, FAKE, None, None) == 3      # ldw % 8
     assert qw(FAKE, 4096, 0, 64, 4096, 128, 1, FAKE + 1, 1024, FAKE, None, None) == 3
+    g4 = L.slimk_w4a8_gemm  # (q, ldq, s_a, w_r, s_r, M, N, K, group, out, ldo, out_dtype, stream)
+    assert g4(None, 4096, FAKE, FAKE, FAKE, 64, 4096, 4096, 128, FAKE, 4096, 0, None) == 1
+    assert g4(FAKE, 4096, FAKE, FAKE, FAKE, 64, 4096, 4096, 256, FAKE, 4096, 0, None) == 7   # group 256
+    assert g4(FAKE, 4160, FAKE, FAKE, FAKE, 64, 4096, 4160, 64, FAKE, 4096, 0, None) == 7    # K % 128
+    assert g4(FAKE, 4000, FAKE, FAKE, FAKE, 64, 4096, 4096, 128, FAKE, 4096, 0, None) == 2   # ldq < K
+    assert g4(FAKE, 4096, FAKE, FAKE, FAKE, 64, 4096, 4096, 128, FAKE, 4096, 3, None) == 4
+    assert g4(FAKE, 4100, FAKE, FAKE, FAKE, 64, 4096, 4096, 128, FAKE, 4096, 0, None) == 3
     q4 = L.slimk_w2a8_quantize_weight4  # (w, ldw, dtype, N, K, group, mode, planes, ldp, scales2, zp2, stream)
     assert q4(FAKE, 4096, 0, 64, 4096, 128, 1, FAKE, 2048, FAKE, None, None) == 1       # zero-points are always written
     assert q4(FAKE, 4096, 0, 64, 4096, 128, 0, FAKE, 2048, FAKE, FAKE, None) == 4       # no REF mode at four bits

@@ -292,3 +292,43 @@ def test_w4a8_linear_from_a_gpu_weight(gpu_ops):
     assert torch.equal(a.weight.planes.zp_r, b.weight.planes.zp_r)
     xd = torch.from_numpy(x).cuda()
     assert torch.equal(a(xd), b(xd))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K,g,out", [(64, 256, 512, 128, "float16"), (200, 320, 1024, 64, "float16"),
+                                         (5, 100, 256, 128, "bfloat16"), (300, 1100, 2048, 128, "bfloat16"),
+                                         (129, 64, 128, 64, "float16")])
+def test_w4a8_one_pass_kernel(gpu_ops, oracle, M, N, K, g, out):
+    """Symmetric 4-bit weights through the kernel that joins the two digits in front of the matrix core: against the
+    oracle (exact int32 sums, fp32 epilogue over G groups) to the output criterion of the path, ragged M and N."""
+    from slimkernels_amd.torch import w4 as tw4
+    print(f"W4A8 one pass M={M} N={N} K={K} g={g} {out}", flush=True)
+    w, x = _w4_case(M, N, K, g, "sym", seed=M + K)
+    packed4, scales, zp = w4.prepare_w4(w, g, "sym")
+    codes = w4.unpack_w4(packed4)
+    bf16 = out == "bfloat16"
+    ref = oracle.w4_reference_forward(x, codes, scales, zp, g, out_bf16=bf16)
+    w4d = tw4.repack_w4(packed4, scales, zp, g)
+    assert w4d.uniform_zp8
+    qa = gpu_ops.quantize_act_int8(torch.from_numpy(x).cuda(), g)
+    dt = torch.bfloat16 if bf16 else torch.float16
+    y = tw4.w4a8_gemm_one_pass(qa, w4d, dt)
+    same = pu.assert_out_close(pu.out_tensor_bits(y), ref["out_bits"], bf16, pu.reorder_bound(ref["acc"], scales, ref["s_a"]),
+                               "W4A8 one pass")
+    print(f"  bit-identical with the oracle on {100 * same:.1f} % of the outputs", flush=True)
+    bound = _plane_bound(oracle, ref, codes, scales, zp, g)
+    # and the layer takes this road from 64 token rows on
+    lin = tw4.W4A8Linear(w4d, None, dt)
+    y2 = lin(torch.from_numpy(x).cuda())
+    if M >= tw4.ONE_PASS_MIN_ROWS:
+        assert torch.equal(y2.view(torch.int16), y.view(torch.int16))
+    pu.assert_out_close(pu.out_tensor_bits(y2), ref["out_bits"], bf16, bound, "W4A8Linear")
+
+
+def test_one_pass_needs_symmetric_weights():
+    from slimkernels_amd.torch import w4 as tw4
+    fake = tw4.W4A8Weight(None, 64, 256, 128, uniform_zp8=False)
+    assert not tw4.one_pass_applies(512, fake)
+    assert tw4.one_pass_applies(512, tw4.W4A8Weight(None, 64, 256, 128, uniform_zp8=True))
+    assert not tw4.one_pass_applies(8, tw4.W4A8Weight(None, 64, 256, 128, uniform_zp8=True))
+    assert not tw4.one_pass_applies(512, tw4.W4A8Weight(None, 64, 256, 256, uniform_zp8=True))
