@@ -262,7 +262,8 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
  *                           the planes' zero-points must be 2 (hi) and 0 (lo) -- they are not read here
  *   M, N, K, group_size   : K is the reduction length of the 4-bit matrix (not 2K); K % 128 == 0, group_size 64 or 128
  * int32 sums per group are exact; the result differs from the two-plane route only in fp32 summation order (G terms
- * instead of 2G).  Any M works; few token rows are better served by slimk_w2a8_gemm over the planes.
+ * instead of 2G).  Any M works, but K is not split: a problem of fewer than about 200 tiles of 64 rows x 256 channels
+ * is better served by slimk_w2a8_gemm over the planes (which splits K and has the few-rows kernels).
  * Replaces upstream's w4matmul_splitk (slimkernels/triton/gemm_splitk.ipynb cell 0) for the many-rows regime. */
 int slimk_w4a8_gemm(const int8_t* q, int ldq, const float* s_a,
                     const uint32_t* w_r, const uint16_t* s_r,

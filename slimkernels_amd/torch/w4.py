@@ -129,17 +129,22 @@ def w4a8_gemm(qa: QuantizedActivation, w: W4A8Weight, out_dtype=torch.float16, *
     return y, acc[:, :, :G] * 4 + acc[:, :, G:]
 
 
-ONE_PASS_MIN_ROWS = 64   # from here on the matrix cores bound the time and one pass over K beats two planes over 2K
+# The one-pass kernel has no split over K: it pays once its 64 x 256 tiles cover the chip.  Measured against the
+# two-plane route (which splits K when tiles are few): 14336 x 4096 at 112 tiles 33.8 / 34.5 us, at 224 tiles
+# 34.8 / 55.8 us, at 1792 tiles 161 / 294 us; 4096 x 14336 at 64 tiles 109 / 54 us.
+ONE_PASS_MIN_TILES = 192
 
 
 def one_pass_applies(M: int, w: W4A8Weight) -> bool:
-    return w.uniform_zp8 and M >= ONE_PASS_MIN_ROWS and w.K % 128 == 0 and w.group_size in (64, 128)
+    tiles = -(-w.N // 256) * -(-M // 64)
+    return w.uniform_zp8 and tiles >= ONE_PASS_MIN_TILES and w.K % 128 == 0 and w.group_size in (64, 128)
 
 
 def w4a8_gemm_one_pass(qa: QuantizedActivation, w: W4A8Weight, out_dtype=torch.float16,
                        out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The many-rows kernel for 4-bit weights with zero-point 8: hi and lo digit are put together in front of the
-    matrix core, one pass over K.  ``qa`` = quantize_act_int8(x) over K (laid down once)."""
+    matrix core, one pass over K, no split of K (meant for problems of a few hundred 64 x 256 tiles or more).
+    ``qa`` = quantize_act_int8(x) over K (laid down once)."""
     M, K = qa.q.shape
     if K != w.K or qa.group_size != w.group_size:
         raise ValueError(f"activation K={K}/group {qa.group_size} does not match weight K={w.K}/group {w.group_size}")

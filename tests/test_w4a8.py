@@ -298,7 +298,7 @@ def test_w4a8_linear_from_a_gpu_weight(gpu_ops):
 @pytest.mark.parametrize("M,N,K,g,out", [(64, 256, 512, 128, "float16"), (200, 320, 1024, 64, "float16"),
                                          (5, 100, 256, 128, "bfloat16"), (300, 1100, 2048, 128, "bfloat16"),
                                          (129, 64, 128, 64, "float16")])
-def test_w4a8_one_pass_kernel(gpu_ops, oracle, M, N, K, g, out):
+def test_w4a8_one_pass_kernel(gpu_ops, oracle, monkeypatch, M, N, K, g, out):
     """Symmetric 4-bit weights through the kernel that joins the two digits in front of the matrix core: against the
     oracle (exact int32 sums, fp32 epilogue over G groups) to the output criterion of the path, ragged M and N."""
     from slimkernels_amd.torch import w4 as tw4
@@ -317,18 +317,22 @@ def test_w4a8_one_pass_kernel(gpu_ops, oracle, M, N, K, g, out):
                                "W4A8 one pass")
     print(f"  bit-identical with the oracle on {100 * same:.1f} % of the outputs", flush=True)
     bound = _plane_bound(oracle, ref, codes, scales, zp, g)
-    # and the layer takes this road from 64 token rows on
+    # the layer takes this road once the problem has enough tiles (threshold lowered here to reach it) and the
+    # two-plane road otherwise
     lin = tw4.W4A8Linear(w4d, None, dt)
     y2 = lin(torch.from_numpy(x).cuda())
-    if M >= tw4.ONE_PASS_MIN_ROWS:
-        assert torch.equal(y2.view(torch.int16), y.view(torch.int16))
     pu.assert_out_close(pu.out_tensor_bits(y2), ref["out_bits"], bf16, bound, "W4A8Linear")
+    monkeypatch.setattr(tw4, "ONE_PASS_MIN_TILES", 1)
+    assert tw4.one_pass_applies(M, w4d)
+    y3 = lin(torch.from_numpy(x).cuda())
+    assert torch.equal(y3.view(torch.int16), y.view(torch.int16))
 
 
-def test_one_pass_needs_symmetric_weights():
+def test_one_pass_needs_symmetric_weights_and_enough_tiles():
     from slimkernels_amd.torch import w4 as tw4
-    fake = tw4.W4A8Weight(None, 64, 256, 128, uniform_zp8=False)
-    assert not tw4.one_pass_applies(512, fake)
-    assert tw4.one_pass_applies(512, tw4.W4A8Weight(None, 64, 256, 128, uniform_zp8=True))
-    assert not tw4.one_pass_applies(8, tw4.W4A8Weight(None, 64, 256, 128, uniform_zp8=True))
-    assert not tw4.one_pass_applies(512, tw4.W4A8Weight(None, 64, 256, 256, uniform_zp8=True))
+    big = dict(N=14336, K=4096, group_size=128)
+    assert tw4.one_pass_applies(512, tw4.W4A8Weight(None, uniform_zp8=True, **big))          # 56 x 8 tiles
+    assert not tw4.one_pass_applies(512, tw4.W4A8Weight(None, uniform_zp8=False, **big))
+    assert not tw4.one_pass_applies(64, tw4.W4A8Weight(None, uniform_zp8=True, **big))       # 56 tiles
+    assert not tw4.one_pass_applies(4096, tw4.W4A8Weight(None, 14336, 4096, 256, uniform_zp8=True))
+    assert not tw4.one_pass_applies(256, tw4.W4A8Weight(None, 4096, 14336, 128, uniform_zp8=True))   # 64 tiles
