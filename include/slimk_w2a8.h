@@ -262,13 +262,21 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
  *                           the planes' zero-points must be 2 (hi) and 0 (lo) -- they are not read here
  *   M, N, K, group_size   : K is the reduction length of the 4-bit matrix (not 2K); K % 128 == 0, group_size 64 or 128
  * int32 sums per group are exact; the result differs from the two-plane route only in fp32 summation order (G terms
- * instead of 2G).  Any M works, but K is not split: a problem of fewer than about 200 tiles of 64 rows x 256 channels
- * is better served by slimk_w2a8_gemm over the planes (which splits K and has the few-rows kernels).
- * Replaces upstream's w4matmul_splitk (slimkernels/triton/gemm_splitk.ipynb cell 0) for the many-rows regime. */
+ * instead of 2G).  Any M works (64-row tiles); up to 32 token rows are better served by slimk_w2a8_gemm over the
+ * planes (the few-rows kernels).
+ *   workspace, split_k    : as for slimk_w2a8_gemm with the tiled kernel (K split over several workgroups per tile when
+ *                           the tiles alone leave CUs idle; 0 = choose): slimk_w4a8_gemm_workspace_bytes(...) bytes,
+ *                           zero-initialised once with slimk_w2a8_workspace_init, left zero by every call; may be
+ *                           the workspace of the slimk_w2a8_gemm calls on the same stream
+ * Replaces upstream's w4matmul_splitk (slimkernels/triton/gemm_splitk.ipynb cell 0: SPLIT_K = 4 with atomic adds; here
+ * the partial tiles meet in the workspace and are summed in split order, so results do not depend on timing). */
+int slimk_w4a8_gemm_auto_split_k(int M, int N, int K, int group_size);
+size_t slimk_w4a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int split_k);
 int slimk_w4a8_gemm(const int8_t* q, int ldq, const float* s_a,
                     const uint32_t* w_r, const uint16_t* s_r,
                     int M, int N, int K, int group_size,
-                    void* out, int ldo, int out_dtype, void* stream);
+                    void* out, int ldo, int out_dtype,
+                    void* workspace, size_t workspace_bytes, int split_k, void* stream);
 
 /* Weight-only form: x [M][ldx] fp16 activations are NOT quantised; the 2-bit codes are widened to fp16 in
  * front of the fp16 matrix cores and every scale group's fp32 sum is scaled into the fp32 result:

@@ -518,10 +518,23 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
                       "grouped skinny gemm");
 }
 
+int slimk_w4a8_gemm_auto_split_k(int M, int N, int K, int group_size) {
+    if (M <= 0 || N <= 0 || !shape_ok(K, group_size) || K % 128 != 0 || group_size > 128) return 0;
+    return w2a8::tiled_w4_auto_split(M, strips_of(N), K / w2a8::kStepK);
+}
+
+size_t slimk_w4a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int split_k) {
+    if (split_k <= 0) split_k = slimk_w4a8_gemm_auto_split_k(M, N, K, group_size);
+    if (split_k <= 1 || M <= 0 || N <= 0) return 0;
+    const size_t tiles = w2a8::tiled_w4_tiles(M, strips_of(N));
+    return counter_bytes((int)tiles) + (size_t)split_k * tiles * 64 * 256 * sizeof(float);
+}
+
 int slimk_w4a8_gemm(const int8_t* q, int ldq, const float* s_a,
                     const uint32_t* w_r, const uint16_t* s_r,
                     int M, int N, int K, int group_size,
-                    void* out, int ldo, int out_dtype, void* stream) {
+                    void* out, int ldo, int out_dtype,
+                    void* workspace, size_t workspace_bytes, int split_k, void* stream) {
     if (!q || !s_a || !w_r || !s_r || !out) return fail(SLIMK_ERR_NULL_POINTER, "w4a8_gemm: NULL buffer");
     if (M <= 0 || N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "M=%d, N=%d must be positive", M, N);
     if (int rc = check_kg(K, group_size)) return rc;
@@ -533,10 +546,28 @@ int slimk_w4a8_gemm(const int8_t* q, int ldq, const float* s_a,
     if (int rc = check_extent(M, N, 2 * K, ldq)) return rc;
     if (!aligned16(q) || ldq % 16 != 0 || !aligned16(w_r) || !aligned16(s_r) || (reinterpret_cast<uintptr_t>(out) & 1u))
         return fail(SLIMK_ERR_MISALIGNED, "w4a8_gemm: q, w_r, s_r must be 16-byte aligned; ldq %% 16 == 0; out 2-byte aligned");
+    const int stages = K / (2 * w2a8::kStepK);
+    if (split_k <= 0) split_k = w2a8::tiled_w4_auto_split(M, strips_of(N), K / w2a8::kStepK);
+    if (split_k > stages) return fail(SLIMK_ERR_BAD_SHAPE, "split_k=%d exceeds the %d stages of 128 reduction elements", split_k, stages);
+    const size_t tiles = w2a8::tiled_w4_tiles(M, strips_of(N));
+    if (split_k > 1 && (size_t)split_k * tiles * 64 * 256 * 4 >= 0x7fffffffu)
+        return fail(SLIMK_ERR_UNSUPPORTED, "w4a8_gemm: split_k=%d over %zu tiles needs more than 2 GiB of partial sums", split_k, tiles);
+    const int sps = split_k > 1 ? (stages + split_k - 1) / split_k : stages;
+    if (split_k > 1) split_k = (stages + sps - 1) / sps;   // effective split: whole stages per split
+
     w2a8::GemmParams p{};
     p.q = q; p.s_a = s_a; p.w_r = w_r; p.s_r = s_r; p.out = out; p.ldq = ldq; p.ldo = ldo;
     p.M = M; p.N = N; p.K = K; p.G = K / group_size; p.steps = K / w2a8::kStepK; p.strips = strips_of(N);
-    p.zp_const = 2; p.split = 1; p.groups_per_split = p.G;
+    p.zp_const = 2; p.split = split_k; p.groups_per_split = split_k > 1 ? sps * (128 / group_size) : p.G;
+    if (split_k > 1) {
+        const size_t need = counter_bytes((int)tiles) + (size_t)split_k * tiles * 64 * 256 * sizeof(float);
+        if (!workspace) return fail(SLIMK_ERR_WORKSPACE, "split_k=%d needs a workspace of %zu bytes", split_k, need);
+        if (workspace_bytes < need)
+            return fail(SLIMK_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, need);
+        if (!aligned16(workspace)) return fail(SLIMK_ERR_MISALIGNED, "workspace must be 16-byte aligned");
+        p.ws_counter = reinterpret_cast<unsigned*>(workspace);
+        p.ws_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counter_bytes((int)tiles));
+    }
     return hip_result(w2a8::launch_tiled_w4(p, group_size / w2a8::kStepK, out_dtype == SLIMK_BF16, (hipStream_t)stream), "w4a8_gemm");
 }
 

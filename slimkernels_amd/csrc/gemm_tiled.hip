@@ -454,22 +454,45 @@ __global__ __launch_bounds__(256, 3) void tiled_kernel_bm64(const GemmParams p) 
 }
 
 // 4-bit weights, one pass (64-row tiles: three stage buffers of 24 KiB leave room for two workgroups on a CU)
-template <int GS, typename OutT>
+template <int GS, bool SPLIT, typename OutT>
 __global__ __launch_bounds__(256, 2) void tiled_kernel_w4(const GemmParams p) {
-    tiled_body<64, GS, false, false, OutT, true>(p);
+    tiled_body<64, GS, SPLIT, false, OutT, true>(p);
+}
+
+size_t tiled_w4_tiles(int M, int strips) {
+    return (size_t)((strips + fast::kStrips - 1) / fast::kStrips) * (size_t)((M + 63) / 64);
+}
+
+// K splits of the one-pass W4 kernel: the rule of the 64-row W2 tiles (about two workgroups per CU, every split at
+// least eight stages long; two halves for a long reduction with one workgroup on most CUs)
+int tiled_w4_auto_split(int M, int strips, int steps) {
+    const int tiles = (int)tiled_w4_tiles(M, strips);
+    const int stages = steps / fast::kStageSteps;
+    if (tiles > 128) return tiles <= 256 && stages >= 64 ? 2 : 1;
+    int split = 512 / tiles;
+    if (split > 8) split = 8;
+    if (split > stages / 8) split = stages / 8;
+    if (split < 1) split = 1;
+    const int sps = (stages + split - 1) / split;
+    return (stages + sps - 1) / sps;
 }
 
 hipError_t launch_tiled_w4(const GemmParams& p, int gs, bool out_bf16, hipStream_t stream) {
-    const int tiles_n = (p.strips + fast::kStrips - 1) / fast::kStrips;
-    const int tiles = tiles_n * ((p.M + 63) / 64);
-    const dim3 grid((tiles + 7) / 8 * 8, 1), block(256);
-    if (gs == 1) {
-        if (out_bf16) tiled_kernel_w4<1, OutBF16><<<grid, block, 0, stream>>>(p);
-        else tiled_kernel_w4<1, OutF16><<<grid, block, 0, stream>>>(p);
-    } else {
-        if (out_bf16) tiled_kernel_w4<2, OutBF16><<<grid, block, 0, stream>>>(p);
-        else tiled_kernel_w4<2, OutF16><<<grid, block, 0, stream>>>(p);
-    }
+    const int tiles = (int)tiled_w4_tiles(p.M, p.strips);
+    const dim3 grid((tiles + 7) / 8 * 8, p.split > 1 ? p.split : 1), block(256);
+#define SLIMK_W4_LAUNCH(GSV)                                                                              \
+    do {                                                                                                  \
+        if (p.split > 1) {                                                                                \
+            if (out_bf16) tiled_kernel_w4<GSV, true, OutBF16><<<grid, block, 0, stream>>>(p);             \
+            else tiled_kernel_w4<GSV, true, OutF16><<<grid, block, 0, stream>>>(p);                       \
+        } else {                                                                                          \
+            if (out_bf16) tiled_kernel_w4<GSV, false, OutBF16><<<grid, block, 0, stream>>>(p);            \
+            else tiled_kernel_w4<GSV, false, OutF16><<<grid, block, 0, stream>>>(p);                      \
+        }                                                                                                 \
+    } while (0)
+    if (gs == 1) SLIMK_W4_LAUNCH(1);
+    else SLIMK_W4_LAUNCH(2);
+#undef SLIMK_W4_LAUNCH
     return hipGetLastError();
 }
 

@@ -71,7 +71,11 @@ hipError_t launch_w2a16(const W2A16Params& p, int gs, bool out_bf16, hipStream_t
 
 // 4-bit weights as two planes (w_r over 2 * p.steps steps, s_r over 2 * p.G groups), uniform zero-point 8, one pass
 // over K: p.K / p.steps / p.G describe K, not 2K; gs 1 or 2; p.steps even
+// p.split > 1: K split over blockIdx.y in whole 128-element stages (p.groups_per_split), workspace = one arrival
+// counter and p.split fp32 tiles of 64 x 256 per tile (tiled_w4_tiles)
 hipError_t launch_tiled_w4(const GemmParams& p, int gs, bool out_bf16, hipStream_t stream);
+size_t tiled_w4_tiles(int M, int strips);
+int tiled_w4_auto_split(int M, int strips, int steps);
 hipError_t launch_tiled_generic(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
 
 }  // namespace w2a8

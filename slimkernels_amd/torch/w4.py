@@ -12,7 +12,7 @@ import torch
 
 from .. import w4 as host_w4
 from .. import _lib
-from .ops import (QuantizedActivation, W2A8Weight, _DT, _require_cuda, _stream_ptr, fused_applies, quantize_act_int8, repack_w2,
+from .ops import (QuantizedActivation, W2A8Weight, _DT, _require_cuda, _stream_ptr, _workspace, fused_applies, quantize_act_int8, repack_w2,
                   w2a8_gemm, w2a8_linear_fused)
 
 
@@ -129,21 +129,20 @@ def w4a8_gemm(qa: QuantizedActivation, w: W4A8Weight, out_dtype=torch.float16, *
     return y, acc[:, :, :G] * 4 + acc[:, :, G:]
 
 
-# The one-pass kernel has no split over K: it pays once its 64 x 256 tiles cover the chip.  Measured against the
-# two-plane route (which splits K when tiles are few): 14336 x 4096 at 112 tiles 33.8 / 34.5 us, at 224 tiles
-# 34.8 / 55.8 us, at 1792 tiles 161 / 294 us; 4096 x 14336 at 64 tiles 109 / 54 us.
-ONE_PASS_MIN_TILES = 192
+# Up to 32 token rows the few-rows kernels over the two planes are faster; beyond, the one-pass kernel is (measured
+# at M = 33 / 64 / 256: 14336 x 4096 18.5 / 19.1 / 34.6 us against 26.8 / 27.6 / 55.4 us over two planes,
+# 4096 x 14336 25.3 / 25.9 / 36.1 us against 36.0 / 36.1 / 53.5 us; at M = 24 it loses, 18.5 us against 15.6 us).
+ONE_PASS_MIN_ROWS = 33
 
 
 def one_pass_applies(M: int, w: W4A8Weight) -> bool:
-    tiles = -(-w.N // 256) * -(-M // 64)
-    return w.uniform_zp8 and tiles >= ONE_PASS_MIN_TILES and w.K % 128 == 0 and w.group_size in (64, 128)
+    return w.uniform_zp8 and M >= ONE_PASS_MIN_ROWS and w.K % 128 == 0 and w.group_size in (64, 128)
 
 
 def w4a8_gemm_one_pass(qa: QuantizedActivation, w: W4A8Weight, out_dtype=torch.float16,
-                       out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                       out: Optional[torch.Tensor] = None, split_k: int = 0) -> torch.Tensor:
     """The many-rows kernel for 4-bit weights with zero-point 8: hi and lo digit are put together in front of the
-    matrix core, one pass over K, no split of K (meant for problems of a few hundred 64 x 256 tiles or more).
+    matrix core, one pass over K (split over several workgroups per tile when the tiles are few; 0 = choose).
     ``qa`` = quantize_act_int8(x) over K (laid down once)."""
     M, K = qa.q.shape
     if K != w.K or qa.group_size != w.group_size:
@@ -155,10 +154,13 @@ def w4a8_gemm_one_pass(qa: QuantizedActivation, w: W4A8Weight, out_dtype=torch.f
     dev = qa.q.device
     if out is None:
         out = torch.empty((M, w.N), dtype=out_dtype, device=dev)
+    L = _lib.lib()
     with torch.cuda.device(dev):
-        _lib.check(_lib.lib().slimk_w4a8_gemm(qa.q.data_ptr(), qa.q.stride(0), qa.s_a.data_ptr(), w.planes.w_r.data_ptr(),
-                                              w.planes.s_r.data_ptr(), M, w.N, K, w.group_size, out.data_ptr(),
-                                              out.stride(0), _DT[out.dtype], _stream_ptr(dev)))
+        ws = _workspace(w.planes, L.slimk_w4a8_gemm_workspace_bytes(M, w.N, K, w.group_size, split_k))
+        _lib.check(L.slimk_w4a8_gemm(qa.q.data_ptr(), qa.q.stride(0), qa.s_a.data_ptr(), w.planes.w_r.data_ptr(),
+                                     w.planes.s_r.data_ptr(), M, w.N, K, w.group_size, out.data_ptr(),
+                                     out.stride(0), _DT[out.dtype], ws.data_ptr() if ws is not None else None,
+                                     ws.numel() if ws is not None else 0, split_k, _stream_ptr(dev)))
     return out
 
 

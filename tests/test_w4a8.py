@@ -298,7 +298,7 @@ def test_w4a8_linear_from_a_gpu_weight(gpu_ops):
 @pytest.mark.parametrize("M,N,K,g,out", [(64, 256, 512, 128, "float16"), (200, 320, 1024, 64, "float16"),
                                          (5, 100, 256, 128, "bfloat16"), (300, 1100, 2048, 128, "bfloat16"),
                                          (129, 64, 128, 64, "float16")])
-def test_w4a8_one_pass_kernel(gpu_ops, oracle, monkeypatch, M, N, K, g, out):
+def test_w4a8_one_pass_kernel(gpu_ops, oracle, M, N, K, g, out):
     """Symmetric 4-bit weights through the kernel that joins the two digits in front of the matrix core: against the
     oracle (exact int32 sums, fp32 epilogue over G groups) to the output criterion of the path, ragged M and N."""
     from slimkernels_amd.torch import w4 as tw4
@@ -316,23 +316,33 @@ def test_w4a8_one_pass_kernel(gpu_ops, oracle, monkeypatch, M, N, K, g, out):
     same = pu.assert_out_close(pu.out_tensor_bits(y), ref["out_bits"], bf16, pu.reorder_bound(ref["acc"], scales, ref["s_a"]),
                                "W4A8 one pass")
     print(f"  bit-identical with the oracle on {100 * same:.1f} % of the outputs", flush=True)
+    # K split over several workgroups per tile: partial sums meet in the workspace in split order, so the result
+    # is the same on every call and within the re-association bound of the oracle's
+    for split in (2, 3):
+        if split <= K // 128:
+            ys = tw4.w4a8_gemm_one_pass(qa, w4d, dt, split_k=split)
+            pu.assert_out_close(pu.out_tensor_bits(ys), ref["out_bits"], bf16, pu.reorder_bound(ref["acc"], scales, ref["s_a"]),
+                                f"W4A8 one pass, split {split}")
+            again = tw4.w4a8_gemm_one_pass(qa, w4d, dt, split_k=split)
+            assert torch.equal(ys.view(torch.int16), again.view(torch.int16))
+    y_after = tw4.w4a8_gemm_one_pass(qa, w4d, dt)          # the counters were left at zero
+    assert torch.equal(y_after.view(torch.int16), y.view(torch.int16))
     bound = _plane_bound(oracle, ref, codes, scales, zp, g)
-    # the layer takes this road once the problem has enough tiles (threshold lowered here to reach it) and the
-    # two-plane road otherwise
+    # the layer takes this road from 33 token rows on and the two-plane road below
     lin = tw4.W4A8Linear(w4d, None, dt)
     y2 = lin(torch.from_numpy(x).cuda())
     pu.assert_out_close(pu.out_tensor_bits(y2), ref["out_bits"], bf16, bound, "W4A8Linear")
-    monkeypatch.setattr(tw4, "ONE_PASS_MIN_TILES", 1)
-    assert tw4.one_pass_applies(M, w4d)
-    y3 = lin(torch.from_numpy(x).cuda())
-    assert torch.equal(y3.view(torch.int16), y.view(torch.int16))
+    assert tw4.one_pass_applies(M, w4d) == (M >= 33)
+    if M >= 33:
+        assert torch.equal(y2.view(torch.int16), y.view(torch.int16))
 
 
-def test_one_pass_needs_symmetric_weights_and_enough_tiles():
+def test_one_pass_needs_symmetric_weights_and_more_than_32_rows():
     from slimkernels_amd.torch import w4 as tw4
     big = dict(N=14336, K=4096, group_size=128)
-    assert tw4.one_pass_applies(512, tw4.W4A8Weight(None, uniform_zp8=True, **big))          # 56 x 8 tiles
+    assert tw4.one_pass_applies(512, tw4.W4A8Weight(None, uniform_zp8=True, **big))
+    assert tw4.one_pass_applies(33, tw4.W4A8Weight(None, uniform_zp8=True, **big))
+    assert not tw4.one_pass_applies(32, tw4.W4A8Weight(None, uniform_zp8=True, **big))
     assert not tw4.one_pass_applies(512, tw4.W4A8Weight(None, uniform_zp8=False, **big))
-    assert not tw4.one_pass_applies(64, tw4.W4A8Weight(None, uniform_zp8=True, **big))       # 56 tiles
     assert not tw4.one_pass_applies(4096, tw4.W4A8Weight(None, 14336, 4096, 256, uniform_zp8=True))
-    assert not tw4.one_pass_applies(256, tw4.W4A8Weight(None, 4096, 14336, 128, uniform_zp8=True))   # 64 tiles
+    assert not tw4.one_pass_applies(512, tw4.W4A8Weight(None, 4096, 4160, 64, uniform_zp8=True))      # K % 128
