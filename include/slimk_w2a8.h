@@ -253,16 +253,18 @@ typedef struct slimk_w2a8_problem {
 int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int group_size, int out_dtype,
                             void* stream);
 
-/* 4-bit weights with the uniform zero-point 8 (levels -8..7) in ONE pass over K, for many token rows: the tiled
- * kernel fetches the hi and the lo digit of every weight and puts them together in front of the matrix core
- * (the int8 operand is 16 * (code - 8)), instead of running the two planes as a reduction over 2K.
- *   q [M][ldq], s_a [M]   : slimk_w2a8_act_quant over K (laid down once; no row sums are needed)
+/* 4-bit weights in ONE pass over K, for more than 32 token rows: the tiled kernel fetches the hi and the lo digit of
+ * every weight and puts them together in front of the matrix core (the int8 operand is 16 * (code - 8)), instead of
+ * running the two planes as a reduction over 2K.
+ *   q [M][ldq], s_a [M]   : slimk_w2a8_act_quant over K (laid down once)
+ *   rowsum [G][ldr]       : its per-group row sums; read only with zp_r
  *   w_r, s_r              : slimk_w2a8_repack of the two planes with K' = 2K (hi digits first) and their scales
- *                           [2G][N] (4 * s, then s), e.g. the outputs of slimk_w2a8_quantize_weight4 in mode SYM;
- *                           the planes' zero-points must be 2 (hi) and 0 (lo) -- they are not read here
+ *                           [2G][N] (4 * s, then s), e.g. the outputs of slimk_w2a8_quantize_weight4
+ *   zp_r                  : NULL: every zero-point is 8 (the planes' are 2 and 0; mode SYM); else the planes'
+ *                           repacked zero-points (rows 0..G-1 zp >> 2, rows G..2G-1 zp & 3): the difference from 8
+ *                           enters through the row sums, (8 - zp) * scale * rowsum per group
  *   M, N, K, group_size   : K is the reduction length of the 4-bit matrix (not 2K); K % 128 == 0, group_size 64 or 128
- * int32 sums per group are exact; the result differs from the two-plane route only in fp32 summation order (G terms
- * instead of 2G).  Any M works (64-row tiles); up to 32 token rows are better served by slimk_w2a8_gemm over the
+ * int32 sums per group are exact; the result differs from the two-plane route only in fp32 summation order.  Any M works (64-row tiles); up to 32 token rows are better served by slimk_w2a8_gemm over the
  * planes (the few-rows kernels).
  *   workspace, split_k    : as for slimk_w2a8_gemm with the tiled kernel (K split over several workgroups per tile when
  *                           the tiles alone leave CUs idle; 0 = choose): slimk_w4a8_gemm_workspace_bytes(...) bytes,
@@ -272,8 +274,8 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
  * the partial tiles meet in the workspace and are summed in split order, so results do not depend on timing). */
 int slimk_w4a8_gemm_auto_split_k(int M, int N, int K, int group_size);
 size_t slimk_w4a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int split_k);
-int slimk_w4a8_gemm(const int8_t* q, int ldq, const float* s_a,
-                    const uint32_t* w_r, const uint16_t* s_r,
+int slimk_w4a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,
+                    const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r,
                     int M, int N, int K, int group_size,
                     void* out, int ldo, int out_dtype,
                     void* workspace, size_t workspace_bytes, int split_k, void* stream);

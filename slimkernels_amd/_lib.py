@@ -39,7 +39,7 @@ SIGNATURES = {
     "slimk_w2a8_gemm_grouped": (_i, [_vp, _i, _i, _i, _vp]),
     "slimk_w4a8_gemm_auto_split_k": (_i, [_i, _i, _i, _i]),
     "slimk_w4a8_gemm_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
-    "slimk_w4a8_gemm": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _i, _vp, _sz, _i, _vp]),
+    "slimk_w4a8_gemm": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _i, _vp, _sz, _i, _vp]),
     "slimk_w2a16_gemm_auto_split_k": (_i, [_i, _i, _i, _i]),
     "slimk_w2a16_gemm_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "slimk_w2a16_gemm": (_i, [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _i, _vp, _sz, _i, _vp]),

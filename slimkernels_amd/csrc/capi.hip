@@ -530,14 +530,18 @@ size_t slimk_w4a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int 
     return counter_bytes((int)tiles) + (size_t)split_k * tiles * 64 * 256 * sizeof(float);
 }
 
-int slimk_w4a8_gemm(const int8_t* q, int ldq, const float* s_a,
-                    const uint32_t* w_r, const uint16_t* s_r,
+int slimk_w4a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,
+                    const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r,
                     int M, int N, int K, int group_size,
                     void* out, int ldo, int out_dtype,
                     void* workspace, size_t workspace_bytes, int split_k, void* stream) {
     if (!q || !s_a || !w_r || !s_r || !out) return fail(SLIMK_ERR_NULL_POINTER, "w4a8_gemm: NULL buffer");
+    if (zp_r && !rowsum) return fail(SLIMK_ERR_NULL_POINTER, "w4a8_gemm: per-group zero-points need the row sums");
     if (M <= 0 || N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "M=%d, N=%d must be positive", M, N);
     if (int rc = check_kg(K, group_size)) return rc;
+    if (zp_r && ldr < M) return fail(SLIMK_ERR_BAD_SHAPE, "ldr=%d smaller than M=%d", ldr, M);
+    if (zp_r && (!aligned16(zp_r) || !aligned16(rowsum) || ldr % 4 != 0))
+        return fail(SLIMK_ERR_MISALIGNED, "w4a8_gemm: zp_r and rowsum must be 16-byte aligned and ldr %% 4 == 0");
     if (K % 128 != 0 || group_size > 128)
         return fail(SLIMK_ERR_UNSUPPORTED, "w4a8_gemm: K=%d must be a multiple of 128 and group_size=%d 64 or 128", K, group_size);
     if (out_dtype != SLIMK_F16 && out_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "out_dtype=%d", out_dtype);
@@ -557,6 +561,7 @@ int slimk_w4a8_gemm(const int8_t* q, int ldq, const float* s_a,
 
     w2a8::GemmParams p{};
     p.q = q; p.s_a = s_a; p.w_r = w_r; p.s_r = s_r; p.out = out; p.ldq = ldq; p.ldo = ldo;
+    p.zp_r = zp_r; p.rowsum = zp_r ? rowsum : nullptr; p.ldr = ldr;
     p.M = M; p.N = N; p.K = K; p.G = K / group_size; p.steps = K / w2a8::kStepK; p.strips = strips_of(N);
     p.zp_const = 2; p.split = split_k; p.groups_per_split = split_k > 1 ? sps * (128 / group_size) : p.G;
     if (split_k > 1) {

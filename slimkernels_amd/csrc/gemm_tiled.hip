@@ -183,12 +183,14 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
         for (int gb = 0; gb < g_cnt; gb += 4 * kRound) {
             v2u zs[kRound];
             uint32_t zz[kRound];
+            uint32_t zl[W4 ? kRound : 1];  // W4: the zero-points of the lo plane (rows G .. 2G-1)
             int rs[kRound][kMB];
 #pragma unroll
             for (int b = 0; b < kRound; ++b) {
                 const int g = g_lo + min(gb + 4 * b + quad, g_cnt - 1);  // clamped; masked below
                 zs[b] = __builtin_amdgcn_raw_buffer_load_b64(s_rsrc, s_lane_off, g * s_group_stride, 0);
                 zz[b] = p.zp_r ? zp32[((size_t)g * p.strips + strip) * 16 + col] : (uint32_t)p.zp_const * 0x01010101u;
+                if constexpr (W4) zl[b] = zp32[((size_t)(g + p.G) * p.strips + strip) * 16 + col];
 #pragma unroll
                 for (int mb = 0; mb < kMB; ++mb) rs[b][mb] = p.rowsum[(size_t)g * p.ldr + rrow[mb]];
             }
@@ -199,7 +201,12 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
                 float zb[4];
 #pragma unroll
                 for (int pp = 0; pp < 4; ++pp)
-                    zb[pp] = on ? (2.0f - (float)((zz[b] >> (8 * pp)) & 0xffu)) * (float)sh[pp] : 0.0f;
+                    // W4: sh is 4 * scale and the operand bytes are centred on 8 = 4 * 2 + 0: what is missing is
+                    // (8 - 4 * zp_hi - zp_lo) * scale = (2 - zp_hi - zp_lo / 4) * sh
+                    if constexpr (W4)
+                        zb[pp] = on ? (2.0f - (float)((zz[b] >> (8 * pp)) & 0xffu) - 0.25f * (float)((zl[b] >> (8 * pp)) & 0xffu)) * (float)sh[pp] : 0.0f;
+                    else
+                        zb[pp] = on ? (2.0f - (float)((zz[b] >> (8 * pp)) & 0xffu)) * (float)sh[pp] : 0.0f;
 #pragma unroll
                 for (int mb = 0; mb < kMB; ++mb) {
                     const float rsf = (float)rs[b][mb];
@@ -454,9 +461,9 @@ __global__ __launch_bounds__(256, 3) void tiled_kernel_bm64(const GemmParams p) 
 }
 
 // 4-bit weights, one pass (64-row tiles: three stage buffers of 24 KiB leave room for two workgroups on a CU)
-template <int GS, bool SPLIT, typename OutT>
+template <int GS, bool SPLIT, bool ZP, typename OutT>
 __global__ __launch_bounds__(256, 2) void tiled_kernel_w4(const GemmParams p) {
-    tiled_body<64, GS, SPLIT, false, OutT, true>(p);
+    tiled_body<64, GS, SPLIT, ZP, OutT, true>(p);
 }
 
 size_t tiled_w4_tiles(int M, int strips) {
@@ -480,18 +487,24 @@ int tiled_w4_auto_split(int M, int strips, int steps) {
 hipError_t launch_tiled_w4(const GemmParams& p, int gs, bool out_bf16, hipStream_t stream) {
     const int tiles = (int)tiled_w4_tiles(p.M, p.strips);
     const dim3 grid((tiles + 7) / 8 * 8, p.split > 1 ? p.split : 1), block(256);
-#define SLIMK_W4_LAUNCH(GSV)                                                                              \
+#define SLIMK_W4_LAUNCH(GSV, ZPV)                                                                         \
     do {                                                                                                  \
         if (p.split > 1) {                                                                                \
-            if (out_bf16) tiled_kernel_w4<GSV, true, OutBF16><<<grid, block, 0, stream>>>(p);             \
-            else tiled_kernel_w4<GSV, true, OutF16><<<grid, block, 0, stream>>>(p);                       \
+            if (out_bf16) tiled_kernel_w4<GSV, true, ZPV, OutBF16><<<grid, block, 0, stream>>>(p);        \
+            else tiled_kernel_w4<GSV, true, ZPV, OutF16><<<grid, block, 0, stream>>>(p);                  \
         } else {                                                                                          \
-            if (out_bf16) tiled_kernel_w4<GSV, false, OutBF16><<<grid, block, 0, stream>>>(p);            \
-            else tiled_kernel_w4<GSV, false, OutF16><<<grid, block, 0, stream>>>(p);                      \
+            if (out_bf16) tiled_kernel_w4<GSV, false, ZPV, OutBF16><<<grid, block, 0, stream>>>(p);       \
+            else tiled_kernel_w4<GSV, false, ZPV, OutF16><<<grid, block, 0, stream>>>(p);                 \
         }                                                                                                 \
     } while (0)
-    if (gs == 1) SLIMK_W4_LAUNCH(1);
-    else SLIMK_W4_LAUNCH(2);
+    const bool zp = p.zp_r != nullptr;   // per-group zero-points: the planes' (rows 0..G-1 hi, G..2G-1 lo) and p.rowsum
+    if (gs == 1) {
+        if (zp) SLIMK_W4_LAUNCH(1, true);
+        else SLIMK_W4_LAUNCH(1, false);
+    } else {
+        if (zp) SLIMK_W4_LAUNCH(2, true);
+        else SLIMK_W4_LAUNCH(2, false);
+    }
 #undef SLIMK_W4_LAUNCH
     return hipGetLastError();
 }

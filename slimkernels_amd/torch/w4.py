@@ -23,7 +23,7 @@ class W4A8Weight:
     N: int
     K: int
     group_size: int
-    uniform_zp8: bool = False   # every zero-point is 8 (the symmetric levels): the one-pass kernel applies
+    uniform_zp8: bool = False   # every zero-point is 8 (the symmetric levels): the one-pass kernel needs no row sums
 
     @property
     def device(self):
@@ -136,19 +136,17 @@ ONE_PASS_MIN_ROWS = 33
 
 
 def one_pass_applies(M: int, w: W4A8Weight) -> bool:
-    return w.uniform_zp8 and M >= ONE_PASS_MIN_ROWS and w.K % 128 == 0 and w.group_size in (64, 128)
+    return M >= ONE_PASS_MIN_ROWS and w.K % 128 == 0 and w.group_size in (64, 128)
 
 
 def w4a8_gemm_one_pass(qa: QuantizedActivation, w: W4A8Weight, out_dtype=torch.float16,
                        out: Optional[torch.Tensor] = None, split_k: int = 0) -> torch.Tensor:
-    """The many-rows kernel for 4-bit weights with zero-point 8: hi and lo digit are put together in front of the
+    """The many-rows kernel for 4-bit weights: hi and lo digit are put together in front of the
     matrix core, one pass over K (split over several workgroups per tile when the tiles are few; 0 = choose).
     ``qa`` = quantize_act_int8(x) over K (laid down once)."""
     M, K = qa.q.shape
     if K != w.K or qa.group_size != w.group_size:
         raise ValueError(f"activation K={K}/group {qa.group_size} does not match weight K={w.K}/group {w.group_size}")
-    if not w.uniform_zp8:
-        raise ValueError("the one-pass kernel needs the uniform zero-point 8 (symmetric levels)")
     if out_dtype not in _DT:
         raise ValueError("out_dtype must be torch.float16 or torch.bfloat16")
     dev = qa.q.device
@@ -157,8 +155,12 @@ def w4a8_gemm_one_pass(qa: QuantizedActivation, w: W4A8Weight, out_dtype=torch.f
     L = _lib.lib()
     with torch.cuda.device(dev):
         ws = _workspace(w.planes, L.slimk_w4a8_gemm_workspace_bytes(M, w.N, K, w.group_size, split_k))
-        _lib.check(L.slimk_w4a8_gemm(qa.q.data_ptr(), qa.q.stride(0), qa.s_a.data_ptr(), w.planes.w_r.data_ptr(),
-                                     w.planes.s_r.data_ptr(), M, w.N, K, w.group_size, out.data_ptr(),
+        # zero-points other than 8 enter through the row sums of the activations
+        zp_r = None if w.uniform_zp8 else w.planes.zp_r
+        _lib.check(L.slimk_w4a8_gemm(qa.q.data_ptr(), qa.q.stride(0), qa.s_a.data_ptr(),
+                                     qa.rowsum.data_ptr() if zp_r is not None else None, qa.rowsum.stride(0),
+                                     w.planes.w_r.data_ptr(), w.planes.s_r.data_ptr(),
+                                     zp_r.data_ptr() if zp_r is not None else None, M, w.N, K, w.group_size, out.data_ptr(),
                                      out.stride(0), _DT[out.dtype], ws.data_ptr() if ws is not None else None,
                                      ws.numel() if ws is not None else 0, split_k, _stream_ptr(dev)))
     return out

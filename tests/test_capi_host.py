@@ -136,16 +136,20 @@ def test_repack_and_act_quant_validation(L):
     assert qw(FAKE, 4096, 0, 64, 4096, 128, 3, FAKE, 1024, FAKE, None, None) == 4      # mode
     assert qw(FAKE, 4100, 0, 64, 4096, 128, 1, FAKE, 1024, FAKE, None, None) == 3      # ldw % 8
     assert qw(FAKE, 4096, 0, 64, 4096, 128, 1, FAKE + 1, 1024, FAKE, None, None) == 3
-    g4 = L.slimk_w4a8_gemm  # (q, ldq, s_a, w_r, s_r, M, N, K, group, out, ldo, out_dtype, ws, ws_bytes, split, stream)
-    assert g4(None, 4096, FAKE, FAKE, FAKE, 64, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 1, None) == 1
-    assert g4(FAKE, 4096, FAKE, FAKE, FAKE, 64, 4096, 4096, 256, FAKE, 4096, 0, None, 0, 1, None) == 7   # group 256
-    assert g4(FAKE, 4160, FAKE, FAKE, FAKE, 64, 4096, 4160, 64, FAKE, 4096, 0, None, 0, 1, None) == 7    # K % 128
-    assert g4(FAKE, 4000, FAKE, FAKE, FAKE, 64, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 1, None) == 2   # ldq < K
-    assert g4(FAKE, 4096, FAKE, FAKE, FAKE, 64, 4096, 4096, 128, FAKE, 4096, 3, None, 0, 1, None) == 4
-    assert g4(FAKE, 4100, FAKE, FAKE, FAKE, 64, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 1, None) == 3
-    assert g4(FAKE, 4096, FAKE, FAKE, FAKE, 64, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 4, None) == 5   # split without workspace
-    assert g4(FAKE, 4096, FAKE, FAKE, FAKE, 64, 4096, 4096, 128, FAKE, 4096, 0, FAKE, 1024, 4, None) == 5
-    assert g4(FAKE, 4096, FAKE, FAKE, FAKE, 64, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 33, None) == 2  # more splits than stages
+    # (q, ldq, s_a, rowsum, ldr, w_r, s_r, zp_r, M, N, K, group, out, ldo, out_dtype, ws, ws_bytes, split, stream)
+    g4 = L.slimk_w4a8_gemm
+    assert g4(None, 4096, FAKE, None, 0, FAKE, FAKE, None, 64, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 1, None) == 1
+    assert g4(FAKE, 4096, FAKE, None, 64, FAKE, FAKE, FAKE, 64, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 1, None) == 1   # zp_r without row sums
+    assert g4(FAKE, 4096, FAKE, FAKE, 60, FAKE, FAKE, FAKE, 64, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 1, None) == 2   # ldr < M
+    assert g4(FAKE, 4096, FAKE, FAKE, 66, FAKE, FAKE, FAKE, 64, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 1, None) == 3   # ldr % 4
+    assert g4(FAKE, 4096, FAKE, None, 0, FAKE, FAKE, None, 64, 4096, 4096, 256, FAKE, 4096, 0, None, 0, 1, None) == 7    # group 256
+    assert g4(FAKE, 4160, FAKE, None, 0, FAKE, FAKE, None, 64, 4096, 4160, 64, FAKE, 4096, 0, None, 0, 1, None) == 7     # K % 128
+    assert g4(FAKE, 4000, FAKE, None, 0, FAKE, FAKE, None, 64, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 1, None) == 2    # ldq < K
+    assert g4(FAKE, 4096, FAKE, None, 0, FAKE, FAKE, None, 64, 4096, 4096, 128, FAKE, 4096, 3, None, 0, 1, None) == 4
+    assert g4(FAKE, 4100, FAKE, None, 0, FAKE, FAKE, None, 64, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 1, None) == 3
+    assert g4(FAKE, 4096, FAKE, None, 0, FAKE, FAKE, None, 64, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 4, None) == 5    # split without workspace
+    assert g4(FAKE, 4096, FAKE, None, 0, FAKE, FAKE, None, 64, 4096, 4096, 128, FAKE, 4096, 0, FAKE, 1024, 4, None) == 5
+    assert g4(FAKE, 4096, FAKE, None, 0, FAKE, FAKE, None, 64, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 33, None) == 2   # more splits than stages
     s4 = L.slimk_w4a8_gemm_auto_split_k(64, 4096, 4096, 128)           # 16 tiles, 32 stages: 4 splits of 8 stages
     assert s4 == 4
     assert L.slimk_w4a8_gemm_workspace_bytes(64, 4096, 4096, 128, 0) == 256 + 4 * 16 * 64 * 256 * 4
