@@ -112,8 +112,11 @@ size_t slimk_w2a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int 
 /* ---- device work ------------------------------------------------------------------------ */
 
 /* Zero a split-K workspace once after allocating it (a fill kernel, safe under graph capture).
- * The GEMM leaves the workspace's counters at zero again when it finishes, so one
- * initialisation serves any number of later calls that use the workspace one at a time. */
+ * A workspace is a block of arrival counters of fixed size (64 KiB, whatever the problem) followed by the fp32
+ * partial tiles.  Every GEMM leaves the counters it used at zero again when it finishes, and the counter block
+ * never moves, so one initialisation serves any number of later calls of any shapes and kernels (2-bit, 4-bit
+ * one-pass, fused) that use the workspace one at a time; calls that overlap in time (different streams) need
+ * a workspace each. */
 int slimk_w2a8_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 
 /* Re-lay the interchange format into the gfx950 streaming layout.
@@ -158,7 +161,7 @@ int slimk_w2a8_quantize_weight(const void* w, int ldw, int w_dtype, int N, int K
  * mode SLIMK_QUANT_SYM: levels -8..7, s = max(absmax, 1e-9) / 8, zp = 8; SLIMK_QUANT_ASYM: s = max(max - min, 1e-9) / 15,
  * zp = clip(rne(-min / s), 0, 15); binary32 arithmetic, IEEE division, round-half-even, s rounded to fp16 once: the
  * numbers of this package's host functions (slimkernels_amd/w4.py: prepare_w4 + split_planes).  The outputs go to
- * slimk_w2a8_repack with K' = 2K.  N <= 65535.  Alignment as for slimk_w2a8_quantize_weight.
+ * slimk_w2a8_repack with K' = 2K.  Alignment as for slimk_w2a8_quantize_weight.
  * Upstream has no 4-bit quantiser (its W4 kernel runs on random codes, gemm_splitk.ipynb cell 2). */
 int slimk_w2a8_quantize_weight4(const void* w, int ldw, int w_dtype, int N, int K, int group_size, int mode,
                                 uint8_t* planes, int ldp, uint16_t* scales2, uint8_t* zp2, void* stream);
@@ -190,8 +193,15 @@ int slimk_w2a8_act_quant_rep(const void* x, int ldx, int x_dtype, int M, int K, 
  *                              1 for the upstream quantizer)
  *   out [M][ldo]             : fp16 or bf16 (out_dtype), ldo in elements
  *   acc_dump, dump_mode      : optional int32 verification output (see slimk_dump); NULL/0
- *                              in production.  The dump path uses separate kernel
- *                              instantiations so the timed kernels carry no extra code.
+ *                              in production.  A call with a dump runs the verification instantiation of
+ *                              the very kernel body the same call without one runs (same kernel choice,
+ *                              tile shape, split and wave count; the accumulators are written out as the
+ *                              matrix core left them, before their conversion to fp32), so the production
+ *                              instantiations carry no extra code and the two calls' outputs are
+ *                              bit-identical.  Only shapes the fast tiled kernel does not take (group
+ *                              256, K % 128 == 64) run the generic tiled kernel with or without a dump.
+ *   rowsum                   : may be NULL for the tiled kernel with zp_r NULL, zp_const 2, group 64 / 128
+ *                              and K % 128 == 0 (it is not read there)
  *   workspace                : required when the effective split_k > 1
  *                              (slimk_w2a8_gemm_workspace_bytes), else may be NULL
  *   kernel, split_k          : SLIMK_KERNEL_* and the split-K factor; 0 = choose.  split_k is an upper
@@ -252,6 +262,14 @@ typedef struct slimk_w2a8_problem {
  * No upstream counterpart. */
 int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int group_size, int out_dtype,
                             void* stream);
+
+/* slimk_w2a8_gemm_grouped with the int32 verification output of slimk_w2a8_gemm: acc_dumps is a HOST array of
+ * `count` device pointers, acc_dumps[i] receiving problem i's accumulators ([M][N][G] for SLIMK_DUMP_GROUPS,
+ * [M][N] for SLIMK_DUMP_SUM).  Runs the verification instantiation of the grouped kernel (same bodies, same
+ * placement of the problems); the outputs are bit-identical with slimk_w2a8_gemm_grouped's.
+ * No upstream counterpart (test infrastructure of this library). */
+int slimk_w2a8_gemm_grouped_verify(const slimk_w2a8_problem* problems, int count, int group_size, int out_dtype,
+                                   int32_t* const* acc_dumps, int dump_mode, void* stream);
 
 /* 4-bit weights in ONE pass over K, for more than 32 token rows: the tiled kernel fetches the hi and the lo digit of
  * every weight and puts them together in front of the matrix core (the int8 operand is 16 * (code - 8)), instead of

@@ -57,12 +57,12 @@ bool shape_ok(int K, int group_size) {
 
 int strips_of(int N) { return (N + w2a8::kStripN - 1) / w2a8::kStripN; }
 
-constexpr size_t kCounterBytesAlign = 256;
-
-size_t counter_bytes(int strips) {
-    size_t b = (size_t)strips * sizeof(unsigned);
-    return (b + kCounterBytesAlign - 1) / kCounterBytesAlign * kCounterBytesAlign;
-}
+// A split-K workspace starts with a block of arrival counters of FIXED size, whatever the problem, followed by the
+// fp32 partial tiles.  Every kernel leaves the counters it used at zero, and because the block does not move
+// with the shape, a workspace zeroed once stays valid for any sequence of problems (a counter block sized by the
+// problem would let a later, larger block overlap an earlier call's partial sums).
+constexpr size_t kCounterBlockBytes = 64 << 10;
+constexpr int kMaxCounters = (int)(kCounterBlockBytes / sizeof(unsigned));
 
 int resolve_kernel(int M, int kernel) {
     if (kernel == SLIMK_KERNEL_AUTO) return M <= 32 ? SLIMK_KERNEL_SKINNY : SLIMK_KERNEL_TILED;
@@ -176,11 +176,11 @@ size_t slimk_w2a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int 
     const int strips = strips_of(N);
     if (kern != SLIMK_KERNEL_SKINNY) {  // one arrival counter and `split_k` fp32 tiles of 64 x 256 per 64-row tile
         const size_t tiles = w2a8::tiled_fast_workspace_tiles(M, strips);
-        return counter_bytes((int)tiles) + (size_t)split_k * tiles * 64 * 256 * sizeof(float);
+        return kCounterBlockBytes + (size_t)split_k * tiles * 64 * 256 * sizeof(float);
     }
     const int mblocks = (M + 15) / 16;  // one tile and one arrival counter per (strip, block of 16 rows)
     const size_t tile = (size_t)16 * w2a8::kStripN;
-    return counter_bytes(strips * mblocks) + (size_t)split_k * strips * mblocks * tile * sizeof(float);
+    return kCounterBlockBytes + (size_t)split_k * strips * mblocks * tile * sizeof(float);
 }
 
 int slimk_w2a8_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
@@ -215,6 +215,7 @@ int slimk_w2a8_quantize_weight(const void* w, int ldw, int w_dtype, int N, int K
     if (mode < SLIMK_QUANT_REF || mode > SLIMK_QUANT_ASYM) return fail(SLIMK_ERR_BAD_ENUM, "mode=%d", mode);
     if (mode == SLIMK_QUANT_ASYM && !zp) return fail(SLIMK_ERR_NULL_POINTER, "quantize_weight: per-group zero-points need zp");
     if (ldw < K || ldp < K / 4) return fail(SLIMK_ERR_BAD_SHAPE, "ldw=%d / ldp=%d too small for K=%d", ldw, ldp, K);
+    if (K / 8 > 65535 * 256) return fail(SLIMK_ERR_UNSUPPORTED, "K=%d too long", K);
     if (!aligned16(w) || ldw % 8 != 0 || (reinterpret_cast<uintptr_t>(packed) & 1u) || ldp % 2 != 0 ||
         (reinterpret_cast<uintptr_t>(scales) & 1u))
         return fail(SLIMK_ERR_MISALIGNED, "quantize_weight: w 16-byte aligned, ldw %% 8 == 0, packed / ldp / scales 2-byte aligned");
@@ -226,7 +227,7 @@ int slimk_w2a8_quantize_weight(const void* w, int ldw, int w_dtype, int N, int K
 int slimk_w2a8_quantize_weight4(const void* w, int ldw, int w_dtype, int N, int K, int group_size, int mode,
                                 uint8_t* planes, int ldp, uint16_t* scales2, uint8_t* zp2, void* stream) {
     if (!w || !planes || !scales2 || !zp2) return fail(SLIMK_ERR_NULL_POINTER, "quantize_weight4: NULL buffer");
-    if (N <= 0 || N > 65535) return fail(SLIMK_ERR_BAD_SHAPE, "N=%d must be in 1..65535", N);
+    if (N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "N=%d must be positive", N);
     if (int rc = check_kg(K, group_size)) return rc;
     if (w_dtype != SLIMK_F16 && w_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "w_dtype=%d", w_dtype);
     if (mode != SLIMK_QUANT_SYM && mode != SLIMK_QUANT_ASYM) return fail(SLIMK_ERR_BAD_ENUM, "mode=%d (SYM or ASYM)", mode);
@@ -263,16 +264,28 @@ int slimk_w2a8_act_quant(const void* x, int ldx, int x_dtype, int M, int K, int 
     return slimk_w2a8_act_quant_rep(x, ldx, x_dtype, M, K, group_size, 1, q, ldq, s_a, rowsum, ldr, stream);
 }
 
-int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,
-                    const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
-                    int M, int N, int K, int group_size,
-                    void* out, int ldo, int out_dtype,
-                    int32_t* acc_dump, int dump_mode,
-                    void* workspace, size_t workspace_bytes,
-                    int kernel, int split_k, void* stream) {
-    if (!q || !s_a || !rowsum || !w_r || !s_r || !out) return fail(SLIMK_ERR_NULL_POINTER, "gemm: NULL buffer");
+}  // extern "C"
+
+namespace {
+
+// fit_split: a split factor chosen here (split_k <= 0) is lowered until its workspace fits workspace_bytes;
+// a caller's explicit split never is.
+int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,
+              const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
+              int M, int N, int K, int group_size,
+              void* out, int ldo, int out_dtype,
+              int32_t* acc_dump, int dump_mode,
+              void* workspace, size_t workspace_bytes,
+              int kernel, int split_k, void* stream, bool fit_split) {
+    if (!q || !s_a || !w_r || !s_r || !out) return fail(SLIMK_ERR_NULL_POINTER, "gemm: NULL buffer");
     if (M <= 0 || N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "M=%d, N=%d must be positive", M, N);
     if (int rc = check_kg(K, group_size)) return rc;
+    // the row sums fold zero-points; the fast tiled kernel centres its operand bytes on 2 and reads none for that value
+    const bool rowsum_unused = !zp_r && zp_const == 2 && resolve_kernel(M, kernel) == SLIMK_KERNEL_TILED &&
+                               group_size <= 128 && K % 128 == 0;
+    if (!rowsum && !rowsum_unused)
+        return fail(SLIMK_ERR_NULL_POINTER, "gemm: rowsum is NULL (only the tiled kernel with the uniform zero-point 2, group 64 / 128 and K %% 128 == 0 does without)");
+    if (!rowsum) ldr = (M + 3) / 4 * 4;
     if (out_dtype != SLIMK_F16 && out_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "out_dtype=%d", out_dtype);
     if (kernel < SLIMK_KERNEL_AUTO || kernel > SLIMK_KERNEL_TILED) return fail(SLIMK_ERR_BAD_ENUM, "kernel=%d", kernel);
     if (dump_mode < SLIMK_DUMP_NONE || dump_mode > SLIMK_DUMP_SUM) return fail(SLIMK_ERR_BAD_ENUM, "dump_mode=%d", dump_mode);
@@ -280,7 +293,7 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
     if (ldq < K || ldo < N || ldr < M) return fail(SLIMK_ERR_BAD_SHAPE, "gemm: ldq=%d, ldo=%d or ldr=%d too small", ldq, ldo, ldr);
     if (zp_const < 0 || zp_const > 3) return fail(SLIMK_ERR_BAD_SHAPE, "zp_const=%d must be 0..3", zp_const);
     if (int rc = check_extent(M, N, K, ldq)) return rc;
-    if (!aligned16(q) || ldq % 16 != 0 || !aligned16(rowsum) || ldr % 4 != 0 || !aligned16(w_r) ||
+    if (!aligned16(q) || ldq % 16 != 0 || (rowsum && (!aligned16(rowsum) || ldr % 4 != 0)) || !aligned16(w_r) ||
         !aligned16(s_r) || (zp_r && !aligned16(zp_r)))
         return fail(SLIMK_ERR_MISALIGNED, "gemm: q, rowsum, w_r, s_r, zp_r must be 16-byte aligned; ldq %% 16 == 0; ldr %% 4 == 0");
     if ((reinterpret_cast<uintptr_t>(out) & 1u) != 0) return fail(SLIMK_ERR_MISALIGNED, "gemm: out must be 2-byte aligned");
@@ -290,7 +303,11 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
         return fail(SLIMK_ERR_UNSUPPORTED, "the skinny kernel handles M <= 32 (M=%d)", M);
     const int G = K / group_size;
     const bool split_chosen_here = split_k <= 0;
-    if (split_k <= 0) split_k = auto_split(M, N, K, group_size, kern);
+    if (split_k <= 0) {
+        split_k = auto_split(M, N, K, group_size, kern);
+        if (fit_split)
+            while (split_k > 1 && slimk_w2a8_gemm_workspace_bytes(M, N, K, group_size, kern, split_k) > workspace_bytes) --split_k;
+    }
     if (split_k > G) return fail(SLIMK_ERR_BAD_SHAPE, "split_k=%d exceeds the number of groups %d", split_k, G);
     int gps;
     if (kern == SLIMK_KERNEL_TILED) {
@@ -332,7 +349,9 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
         p.ws_counter = reinterpret_cast<unsigned*>(workspace);
         const int counters = kern == SLIMK_KERNEL_SKINNY ? p.strips * ((M + 15) / 16)
                                                          : (int)w2a8::tiled_fast_workspace_tiles(M, p.strips);
-        p.ws_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counter_bytes(counters));
+        if (counters > kMaxCounters)
+            return fail(SLIMK_ERR_UNSUPPORTED, "split_k over %d output tiles (at most %d arrival counters)", counters, kMaxCounters);
+        p.ws_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBlockBytes);
     }
 
     hipStream_t st = (hipStream_t)stream;
@@ -342,11 +361,30 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
     const int gs = group_size / w2a8::kStepK;
     const bool asym = zp_r != nullptr;
     const bool out_bf16 = out_dtype == SLIMK_BF16;
-    if (kern == SLIMK_KERNEL_SKINNY && p.acc_dump == nullptr && skinny_shared_applies(M, N, K))
-        return hip_result(w2a8::launch_skinny_shared(p, gs, asym, out_bf16, st), "shared skinny gemm");
+    // a call with a dump runs the verification instantiation of the kernel the same call without one would run
+    const bool dump = p.acc_dump != nullptr;
+    if (kern == SLIMK_KERNEL_SKINNY && skinny_shared_applies(M, N, K))
+        return hip_result(dump ? w2a8::launch_skinny_shared_verify(p, gs, asym, out_bf16, st)
+                               : w2a8::launch_skinny_shared(p, gs, asym, out_bf16, st), "shared skinny gemm");
     if (kern == SLIMK_KERNEL_SKINNY)
-        return hip_result(w2a8::launch_skinny(p, gs, skinny_waves(M, N, K, split_k), asym, out_bf16, st), "skinny gemm");
+        return hip_result(dump ? w2a8::launch_skinny_verify(p, gs, skinny_waves(M, N, K, split_k), asym, out_bf16, st)
+                               : w2a8::launch_skinny(p, gs, skinny_waves(M, N, K, split_k), asym, out_bf16, st), "skinny gemm");
     return hip_result(w2a8::launch_tiled(p, gs, asym, out_bf16, st), "tiled gemm");
+}
+
+}  // namespace
+
+extern "C" {
+
+int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,
+                    const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
+                    int M, int N, int K, int group_size,
+                    void* out, int ldo, int out_dtype,
+                    int32_t* acc_dump, int dump_mode,
+                    void* workspace, size_t workspace_bytes,
+                    int kernel, int split_k, void* stream) {
+    return gemm_impl(q, ldq, s_a, rowsum, ldr, w_r, s_r, zp_r, zp_const, M, N, K, group_size, out, ldo, out_dtype,
+                     acc_dump, dump_mode, workspace, workspace_bytes, kernel, split_k, stream, false);
 }
 
 int slimk_w2a8_gemm_fused(const void* x, int ldx, int x_dtype,
@@ -386,16 +424,28 @@ int slimk_w2a8_gemm_fused(const void* x, int ldx, int x_dtype,
             return fail(SLIMK_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, need);
         if (!aligned16(workspace)) return fail(SLIMK_ERR_MISALIGNED, "workspace must be 16-byte aligned");
         p.ws_counter = reinterpret_cast<unsigned*>(workspace);
-        p.ws_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counter_bytes(p.strips));
+        if (p.strips > kMaxCounters)
+            return fail(SLIMK_ERR_UNSUPPORTED, "split_k over %d output tiles (at most %d arrival counters)", p.strips, kMaxCounters);
+        p.ws_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBlockBytes);
     }
     return hip_result(w2a8::launch_skinny_fused(p, group_size / w2a8::kStepK, skinny_waves(M, N, K, split_k), zp_r != nullptr,
                                                 out_dtype == SLIMK_BF16, (hipStream_t)stream),
                       "fused skinny gemm");
 }
 
-int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int group_size, int out_dtype,
-                            void* stream) {
+}  // extern "C"
+
+namespace {
+
+int gemm_grouped_impl(const slimk_w2a8_problem* problems, int count, int group_size, int out_dtype,
+                      int32_t* const* acc_dumps, int dump_mode, void* stream) {
     if (!problems) return fail(SLIMK_ERR_NULL_POINTER, "gemm_grouped: problems is NULL");
+    if (dump_mode != SLIMK_DUMP_NONE) {
+        if (dump_mode != SLIMK_DUMP_GROUPS && dump_mode != SLIMK_DUMP_SUM) return fail(SLIMK_ERR_BAD_ENUM, "dump_mode=%d", dump_mode);
+        if (!acc_dumps) return fail(SLIMK_ERR_NULL_POINTER, "gemm_grouped: dump_mode set but acc_dumps is NULL");
+        for (int i = 0; i < count && i < SLIMK_W2A8_MAX_GROUP; ++i)
+            if (!acc_dumps[i]) return fail(SLIMK_ERR_NULL_POINTER, "gemm_grouped: acc_dumps[%d] is NULL", i);
+    }
     if (count < 1 || count > SLIMK_W2A8_MAX_GROUP)
         return fail(SLIMK_ERR_BAD_SHAPE, "gemm_grouped: count=%d must be 1..%d", count, SLIMK_W2A8_MAX_GROUP);
     if (out_dtype != SLIMK_F16 && out_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "out_dtype=%d", out_dtype);
@@ -481,6 +531,7 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
         g.M = pr.M; g.N = pr.N; g.K = pr.K; g.G = pr.K / group_size; g.steps = pr.K / w2a8::kStepK;
         g.strips = strips_of(pr.N); g.zp_const = pr.zp_const;
         g.split = 1; g.groups_per_split = groups_per_split(g.G, group_size, 1);
+        if (dump_mode != SLIMK_DUMP_NONE) { g.acc_dump = acc_dumps[order[i]]; g.dump_mode = dump_mode; }
         gp.wg_begin[i] = wgs;
         gp.kparts[i] = kparts[order[i]];
         // units (sets of 8, 4 or 2 strips) in whole sets of eight, times the row blocks of 16 tokens
@@ -510,12 +561,33 @@ int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int g
     if (count == 1 && auto_split(problems[0].M, problems[0].N, problems[0].K, group_size, SLIMK_KERNEL_SKINNY) == 1) {
         const slimk_w2a8_problem& pr = problems[0];
         return slimk_w2a8_gemm(pr.q, pr.ldq, pr.s_a, pr.rowsum, pr.ldr, pr.w_r, pr.s_r, pr.zp_r, pr.zp_const, pr.M, pr.N, pr.K,
-                               group_size, pr.out, pr.ldo, out_dtype, nullptr, SLIMK_DUMP_NONE, nullptr, 0,
-                               SLIMK_KERNEL_SKINNY, 1, stream);
+                               group_size, pr.out, pr.ldo, out_dtype, dump_mode != SLIMK_DUMP_NONE ? acc_dumps[0] : nullptr, dump_mode,
+                               nullptr, 0, SLIMK_KERNEL_SKINNY, 1, stream);
     }
-    return hip_result(w2a8::launch_skinny_grouped(gp, group_size / w2a8::kStepK, zm == 1, out_dtype == SLIMK_BF16,
-                                                  (hipStream_t)stream),
+    hipStream_t st = (hipStream_t)stream;
+    if (dump_mode == SLIMK_DUMP_SUM)
+        for (int i = 0; i < count; ++i)
+            if (int rc = hip_result(w2a8::launch_fill_zero(acc_dumps[i], (size_t)problems[i].M * problems[i].N * sizeof(int32_t), st), "dump clear"))
+                return rc;
+    const int gs = group_size / w2a8::kStepK;
+    return hip_result(dump_mode != SLIMK_DUMP_NONE ? w2a8::launch_skinny_grouped_verify(gp, gs, zm == 1, out_dtype == SLIMK_BF16, st)
+                                                   : w2a8::launch_skinny_grouped(gp, gs, zm == 1, out_dtype == SLIMK_BF16, st),
                       "grouped skinny gemm");
+}
+
+}  // namespace
+
+extern "C" {
+
+int slimk_w2a8_gemm_grouped(const slimk_w2a8_problem* problems, int count, int group_size, int out_dtype,
+                            void* stream) {
+    return gemm_grouped_impl(problems, count, group_size, out_dtype, nullptr, SLIMK_DUMP_NONE, stream);
+}
+
+int slimk_w2a8_gemm_grouped_verify(const slimk_w2a8_problem* problems, int count, int group_size, int out_dtype,
+                                   int32_t* const* acc_dumps, int dump_mode, void* stream) {
+    if (dump_mode == SLIMK_DUMP_NONE) return fail(SLIMK_ERR_BAD_ENUM, "gemm_grouped_verify: dump_mode must be GROUPS or SUM");
+    return gemm_grouped_impl(problems, count, group_size, out_dtype, acc_dumps, dump_mode, stream);
 }
 
 int slimk_w4a8_gemm_auto_split_k(int M, int N, int K, int group_size) {
@@ -527,7 +599,7 @@ size_t slimk_w4a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int 
     if (split_k <= 0) split_k = slimk_w4a8_gemm_auto_split_k(M, N, K, group_size);
     if (split_k <= 1 || M <= 0 || N <= 0) return 0;
     const size_t tiles = w2a8::tiled_w4_tiles(M, strips_of(N));
-    return counter_bytes((int)tiles) + (size_t)split_k * tiles * 64 * 256 * sizeof(float);
+    return kCounterBlockBytes + (size_t)split_k * tiles * 64 * 256 * sizeof(float);
 }
 
 int slimk_w4a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,
@@ -565,13 +637,13 @@ int slimk_w4a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
     p.M = M; p.N = N; p.K = K; p.G = K / group_size; p.steps = K / w2a8::kStepK; p.strips = strips_of(N);
     p.zp_const = 2; p.split = split_k; p.groups_per_split = split_k > 1 ? sps * (128 / group_size) : p.G;
     if (split_k > 1) {
-        const size_t need = counter_bytes((int)tiles) + (size_t)split_k * tiles * 64 * 256 * sizeof(float);
+        const size_t need = kCounterBlockBytes + (size_t)split_k * tiles * 64 * 256 * sizeof(float);
         if (!workspace) return fail(SLIMK_ERR_WORKSPACE, "split_k=%d needs a workspace of %zu bytes", split_k, need);
         if (workspace_bytes < need)
             return fail(SLIMK_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, need);
         if (!aligned16(workspace)) return fail(SLIMK_ERR_MISALIGNED, "workspace must be 16-byte aligned");
         p.ws_counter = reinterpret_cast<unsigned*>(workspace);
-        p.ws_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counter_bytes((int)tiles));
+        p.ws_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBlockBytes);
     }
     return hip_result(w2a8::launch_tiled_w4(p, group_size / w2a8::kStepK, out_dtype == SLIMK_BF16, (hipStream_t)stream), "w4a8_gemm");
 }

@@ -1,0 +1,20 @@
+// Verification instantiations of the skinny-M kernels: the production bodies (skinny_bodies.h) with the int32 dump
+// switched on.  A verification launch takes the same instantiation choices as the production launch of the same
+// problem; its outputs are bit-identical with the production launch's.
+#include "skinny_bodies.h"
+
+namespace w2a8 {
+
+hipError_t launch_skinny_verify(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, hipStream_t stream) {
+    return launch_skinny_impl<true>(p, gs, waves, asym, out_bf16, stream);
+}
+
+hipError_t launch_skinny_shared_verify(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream) {
+    return launch_skinny_shared_impl<true>(p, gs, asym, out_bf16, stream);
+}
+
+hipError_t launch_skinny_grouped_verify(const GroupedParams& gp, int gs, bool asym, bool out_bf16, hipStream_t stream) {
+    return launch_skinny_grouped_impl<true>(gp, gs, asym, out_bf16, stream);
+}
+
+}  // namespace w2a8

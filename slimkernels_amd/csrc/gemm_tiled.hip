@@ -43,7 +43,10 @@ constexpr int kAQueue = 4;                                 // activation fragmen
 // steps .. 2*steps-1; s_r rows 0 .. G-1 = 4 * scale) with the uniform zero-point 8.  Both digits of a step are fetched
 // and put together before the MFMA: the operand byte 64 * (hi - 2) | 16 * lo is 16 * (code - 8), and the hi plane's
 // scale times the 1/64 of the 2-bit path is scale / 16: one pass over K instead of two over 2K.
-template <int BM, int GS, bool SPLIT, bool ZP, typename OutT, bool W4 = false>
+// DUMP: verification instantiation of the same body: every per-group int32 accumulator is also written out (exactly,
+// as the MFMA left it, before its conversion to fp32); nothing else changes, so the output bits are the production
+// instantiation's.
+template <int BM, int GS, bool SPLIT, bool ZP, typename OutT, bool W4 = false, bool DUMP = false>
 __device__ __forceinline__ void tiled_body(const GemmParams& p) {
     using namespace fast;
     constexpr int kBM = BM;
@@ -306,6 +309,12 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
                         const int e = (s * 4 + pp) * kDrainPerMfma + d;  // 0..15: sub-block e / 4, row e % 4
                         t[pmb][e / 4][e % 4] = __builtin_fmaf((float)acc[(u & 1) ^ 1][e / 4][e % 4],
                                                               u == 0 ? sc_prev[e / 4] : sc[pgi][e / 4], t[pmb][e / 4][e % 4]);
+                        if constexpr (DUMP) {  // the previous unit's group: for u == 0 the last group of the previous stage
+                            if ((u > 0 || stage > 0) && strip_ok)
+                                dump_group_sum<W4>(p, m_tile + pmb * 16 + quad * 4 + e % 4, strip * kStripN + (e / 4) * 16 + col,
+                                                   (stage0 + stage) * kGroupsPerStage + (u == 0 ? -1 : pgi),
+                                                   acc[(u & 1) ^ 1][e / 4][e % 4] >> (W4 ? 4 : 6), W4 ? 8 : 2);
+                        }
                     }
                     if (pp == 3 && r + kAQueue < kABlocks) aq[r % kAQueue] = lds_a(r + kAQueue);
                     __builtin_amdgcn_sched_barrier(0);
@@ -323,7 +332,14 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
     for (int pp = 0; pp < 4; ++pp)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
+        {
             t[kMB - 1][pp][j] = __builtin_fmaf((float)acc[1][pp][j], sc_prev[pp], t[kMB - 1][pp][j]);
+            if constexpr (DUMP) {
+                if (strip_ok)
+                    dump_group_sum<W4>(p, m_tile + (kMB - 1) * 16 + quad * 4 + j, strip * kStripN + pp * 16 + col,
+                                       (stage0 + n_stages) * kGroupsPerStage - 1, acc[1][pp][j] >> (W4 ? 4 : 6), W4 ? 8 : 2);
+            }
+        }
 
     uint16_t* out = reinterpret_cast<uint16_t*>(p.out);
     if (SPLIT) {
@@ -451,19 +467,19 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
 }
 
 // 128-row tiles: two workgroups (eight waves) per CU; 64-row tiles need fewer registers: three.
-template <int GS, bool ZP, typename OutT>
+template <int GS, bool ZP, typename OutT, bool DUMP = false>
 __global__ __launch_bounds__(256, 2) void tiled_kernel(const GemmParams p) {
-    tiled_body<128, GS, false, ZP, OutT>(p);
+    tiled_body<128, GS, false, ZP, OutT, false, DUMP>(p);
 }
-template <int GS, bool SPLIT, bool ZP, typename OutT>
-__global__ __launch_bounds__(256, 3) void tiled_kernel_bm64(const GemmParams p) {
-    tiled_body<64, GS, SPLIT, ZP, OutT>(p);
+template <int GS, bool SPLIT, bool ZP, typename OutT, bool DUMP = false>
+__global__ __launch_bounds__(256, DUMP ? 2 : 3) void tiled_kernel_bm64(const GemmParams p) {
+    tiled_body<64, GS, SPLIT, ZP, OutT, false, DUMP>(p);
 }
 
 // 4-bit weights, one pass (64-row tiles: three stage buffers of 24 KiB leave room for two workgroups on a CU)
-template <int GS, bool SPLIT, bool ZP, typename OutT>
+template <int GS, bool SPLIT, bool ZP, typename OutT, bool DUMP = false>
 __global__ __launch_bounds__(256, 2) void tiled_kernel_w4(const GemmParams p) {
-    tiled_body<64, GS, SPLIT, ZP, OutT, true>(p);
+    tiled_body<64, GS, SPLIT, ZP, OutT, true, DUMP>(p);
 }
 
 size_t tiled_w4_tiles(int M, int strips) {
@@ -487,9 +503,18 @@ int tiled_w4_auto_split(int M, int strips, int steps) {
 hipError_t launch_tiled_w4(const GemmParams& p, int gs, bool out_bf16, hipStream_t stream) {
     const int tiles = (int)tiled_w4_tiles(p.M, p.strips);
     const dim3 grid((tiles + 7) / 8 * 8, p.split > 1 ? p.split : 1), block(256);
+    const bool dump = p.acc_dump != nullptr && p.dump_mode != 0;
 #define SLIMK_W4_LAUNCH(GSV, ZPV)                                                                         \
     do {                                                                                                  \
-        if (p.split > 1) {                                                                                \
+        if (dump) {                                                                                       \
+            if (p.split > 1) {                                                                            \
+                if (out_bf16) tiled_kernel_w4<GSV, true, ZPV, OutBF16, true><<<grid, block, 0, stream>>>(p);  \
+                else tiled_kernel_w4<GSV, true, ZPV, OutF16, true><<<grid, block, 0, stream>>>(p);        \
+            } else {                                                                                      \
+                if (out_bf16) tiled_kernel_w4<GSV, false, ZPV, OutBF16, true><<<grid, block, 0, stream>>>(p); \
+                else tiled_kernel_w4<GSV, false, ZPV, OutF16, true><<<grid, block, 0, stream>>>(p);       \
+            }                                                                                             \
+        } else if (p.split > 1) {                                                                                \
             if (out_bf16) tiled_kernel_w4<GSV, true, ZPV, OutBF16><<<grid, block, 0, stream>>>(p);        \
             else tiled_kernel_w4<GSV, true, ZPV, OutF16><<<grid, block, 0, stream>>>(p);                  \
         } else {                                                                                          \
@@ -511,8 +536,7 @@ hipError_t launch_tiled_w4(const GemmParams& p, int gs, bool out_bf16, hipStream
 
 bool tiled_fast_supported(const GemmParams& p, int gs, bool asym) {
     (void)asym;
-    const bool dump = p.acc_dump != nullptr && p.dump_mode != 0;
-    return !dump && (gs == 1 || gs == 2) && p.steps % fast::kStageSteps == 0;
+    return (gs == 1 || gs == 2) && p.steps % fast::kStageSteps == 0;
 }
 
 // Tile height and tile count of the fast kernel for a problem: two workgroups fit a CU, so below
@@ -567,9 +591,20 @@ hipError_t launch_tiled(const GemmParams& p, int gs, bool asym, bool out_bf16, h
     const dim3 grid((tiles + 7) / 8 * 8, p.split > 1 ? p.split : 1), block(256);
     const bool zp = asym || p.zp_const != 2;
     const bool split = bm == 64 && p.split > 1;
+    const bool dump = p.acc_dump != nullptr && p.dump_mode != 0;
+    // a verification call runs the same body with the dump switched on (same tile height, same split)
 #define SLIMK_TILED_LAUNCH(GSV, ZPV)                                                                          \
     do {                                                                                                      \
-        if (bm == 128) {                                                                                      \
+        if (dump && bm == 128) {                                                                              \
+            if (out_bf16) tiled_kernel<GSV, ZPV, OutBF16, true><<<grid, block, 0, stream>>>(p);               \
+            else tiled_kernel<GSV, ZPV, OutF16, true><<<grid, block, 0, stream>>>(p);                         \
+        } else if (dump && split) {                                                                           \
+            if (out_bf16) tiled_kernel_bm64<GSV, true, ZPV, OutBF16, true><<<grid, block, 0, stream>>>(p);    \
+            else tiled_kernel_bm64<GSV, true, ZPV, OutF16, true><<<grid, block, 0, stream>>>(p);              \
+        } else if (dump) {                                                                                    \
+            if (out_bf16) tiled_kernel_bm64<GSV, false, ZPV, OutBF16, true><<<grid, block, 0, stream>>>(p);   \
+            else tiled_kernel_bm64<GSV, false, ZPV, OutF16, true><<<grid, block, 0, stream>>>(p);             \
+        } else if (bm == 128) {                                                                               \
             if (out_bf16) tiled_kernel<GSV, ZPV, OutBF16><<<grid, block, 0, stream>>>(p);                     \
             else tiled_kernel<GSV, ZPV, OutF16><<<grid, block, 0, stream>>>(p);                               \
         } else if (split) {                                                                                   \

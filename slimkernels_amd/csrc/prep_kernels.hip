@@ -267,8 +267,8 @@ __global__ __launch_bounds__(256) void quantize_weight_kernel(const uint16_t* __
                                                               int group_size, int mode, uint8_t* __restrict__ packed,
                                                               int ldp, uint16_t* __restrict__ scales,
                                                               uint8_t* __restrict__ zp) {
-    const int n = blockIdx.y;
-    const int v = blockIdx.x * 256 + threadIdx.x;  // 8-element vector of the row
+    const int n = blockIdx.x;                      // rows on grid.x: no 65535 limit on N
+    const int v = blockIdx.y * 256 + threadIdx.x;  // 8-element vector of the row
     const bool on = v < K / 8;                      // K / 8 is a multiple of a group's threads: whole groups on or off
     float f[8];
     if (on) {
@@ -320,7 +320,7 @@ __global__ __launch_bounds__(256) void quantize_weight_kernel(const uint16_t* __
 
 hipError_t launch_quantize_weight(const void* w, int ldw, bool w_bf16, int N, int K, int group_size, int mode,
                                   uint8_t* packed, int ldp, uint16_t* scales, uint8_t* zp, hipStream_t stream) {
-    const dim3 grid((unsigned)((K / 8 + 255) / 256), (unsigned)N), block(256);
+    const dim3 grid((unsigned)N, (unsigned)((K / 8 + 255) / 256)), block(256);
     if (w_bf16)
         quantize_weight_kernel<true><<<grid, block, 0, stream>>>((const uint16_t*)w, ldw, N, K, group_size, mode, packed,
                                                                 ldp, scales, zp);
@@ -340,8 +340,8 @@ __global__ __launch_bounds__(256) void quantize_weight4_kernel(const uint16_t* _
                                                                int group_size, int asym, uint8_t* __restrict__ packed,
                                                                int ldp, uint16_t* __restrict__ scales,
                                                                uint8_t* __restrict__ zp) {
-    const int n = blockIdx.y;
-    const int v = blockIdx.x * 256 + threadIdx.x;
+    const int n = blockIdx.x;
+    const int v = blockIdx.y * 256 + threadIdx.x;
     const bool on = v < K / 8;
     float f[8];
     if (on) {
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(256) void quantize_weight4_kernel(const uint16_t* _
 
 hipError_t launch_quantize_weight4(const void* w, int ldw, bool w_bf16, int N, int K, int group_size, bool asym,
                                    uint8_t* packed, int ldp, uint16_t* scales, uint8_t* zp, hipStream_t stream) {
-    const dim3 grid((unsigned)((K / 8 + 255) / 256), (unsigned)N), block(256);
+    const dim3 grid((unsigned)N, (unsigned)((K / 8 + 255) / 256)), block(256);
     if (w_bf16)
         quantize_weight4_kernel<true><<<grid, block, 0, stream>>>((const uint16_t*)w, ldw, N, K, group_size, asym ? 1 : 0,
                                                                  packed, ldp, scales, zp);

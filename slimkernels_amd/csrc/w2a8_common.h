@@ -86,6 +86,24 @@ __device__ __forceinline__ float half_bits_to_float(uint16_t h) {
     return (float)__builtin_bit_cast(_Float16, h);
 }
 
+// Verification instantiations only: record the exact int32 sum of one (token m, channel n, scale group g).
+// `value` is sum_k q * (code - c0) as the kernel's operand encoding yields it (c0 = 0 for the plain fields,
+// 2 for the bytes centred on the symmetric levels, 8 for the joined 4-bit digits); the true sum
+// sum_k q * (code - zp) follows in integers from the group's row sum.  W4: the zero-point is 4 * hi + lo of the two
+// planes (rows g and g + G of zp_r), 8 without zp_r.
+template <bool W4 = false>
+__device__ __forceinline__ void dump_group_sum(const GemmParams& p, int m, int n, int g, int value, int c0) {
+    if (m >= p.M || n >= p.N || g >= p.G) return;
+    const size_t zi = (size_t)(n >> 6) * 64 + (n & 15) * 4 + ((n >> 4) & 3);
+    int zp;
+    if (W4) zp = p.zp_r ? 4 * (int)p.zp_r[(size_t)g * p.strips * 64 + zi] + (int)p.zp_r[(size_t)(g + p.G) * p.strips * 64 + zi] : 8;
+    else zp = p.zp_r ? (int)p.zp_r[(size_t)g * p.strips * 64 + zi] : p.zp_const;
+    int v = value;
+    if (zp != c0) v += (c0 - zp) * p.rowsum[(size_t)g * p.ldr + m];
+    if (p.dump_mode == 1) p.acc_dump[((size_t)m * p.N + n) * p.G + g] = v;
+    else atomicAdd(p.acc_dump + (size_t)m * p.N + n, v);
+}
+
 // The output is defined as cast(fp32 product): the empty asm keeps the compiler from folding the
 // caller's fp32 multiply into a v_fma_mixlo_f16, which would round the exact product once.
 struct OutF16 {

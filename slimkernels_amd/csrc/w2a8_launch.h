@@ -43,8 +43,14 @@ hipError_t launch_skinny_shared(const GemmParams& p, int gs, bool asym, bool out
 // asym: every problem carries per-group zero-points (zp_r); otherwise each uses its uniform zp_const
 hipError_t launch_skinny_grouped(const GroupedParams& gp, int gs, bool asym, bool out_bf16, hipStream_t stream);
 
-// launch_tiled picks the fast kernel when it applies (uniform zero-point 2, group 64/128, K % 128 == 0,
-// no verification dump) and the generic one otherwise.
+// Verification instantiations of the three launches above (gemm_skinny_verify.hip): the same bodies with the int32
+// dump switched on (p.acc_dump / p.dump_mode, per problem in a grouped launch), same instantiation choices.
+hipError_t launch_skinny_verify(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, hipStream_t stream);
+hipError_t launch_skinny_shared_verify(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
+hipError_t launch_skinny_grouped_verify(const GroupedParams& gp, int gs, bool asym, bool out_bf16, hipStream_t stream);
+
+// launch_tiled picks the fast kernel when it applies (group 64/128, K % 128 == 0; with p.acc_dump its verification
+// instantiation) and the generic one otherwise.
 hipError_t launch_tiled(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
 // Split-K of the fast tiled kernel (64-row tiles only): the factor it would choose, the largest it
 // accepts, and the number of tiles a split workspace must hold (64 x 256 fp32 each, per split).

@@ -296,23 +296,27 @@ def w2a16_gemm(x: torch.Tensor, w: W2A8Weight, out_dtype=torch.float16, *, split
     return out
 
 
-def w2a8_gemm_grouped(problems, out_dtype=torch.float16):
+def w2a8_gemm_grouped(problems, out_dtype=torch.float16, *, dump: Optional[str] = None):
     """Several independent skinny (M <= 32) GEMMs in one kernel launch.
 
     ``problems`` is a sequence of (QuantizedActivation, W2A8Weight) or (qa, w, out) tuples that
     share group size and zero-point mode; returns the list of outputs.  More than 24 problems are
-    issued as several launches."""
+    issued as several launches.  With ``dump`` ("groups" or "sum") the verification instantiation of
+    the grouped kernel runs and (outputs, int32 accumulator tensors) is returned."""
     L = _lib.lib()
     probs = [(p[0], p[1], p[2] if len(p) > 2 else None) for p in problems]
     if not probs:
         return []
     dev = probs[0][0].q.device
     g = probs[0][1].group_size
-    outs = []
+    if dump not in (None, "groups", "sum"):
+        raise ValueError("dump must be None, 'groups' or 'sum'")
+    outs, accs = [], []
     with torch.cuda.device(dev):
         for lo in range(0, len(probs), _lib.MAX_GROUP):
             chunk = probs[lo:lo + _lib.MAX_GROUP]
             arr = (_lib.Problem * len(chunk))()
+            dumps = (ctypes.c_void_p * len(chunk))()
             for i, (qa, w, out) in enumerate(chunk):
                 M, K = qa.q.shape
                 if K != w.K or qa.group_size != w.group_size or w.group_size != g:
@@ -322,12 +326,21 @@ def w2a8_gemm_grouped(problems, out_dtype=torch.float16):
                 if out.dtype != out_dtype:
                     raise ValueError("every output must have dtype out_dtype")
                 outs.append(out)
+                if dump is not None:
+                    shape = (M, w.N, K // g) if dump == "groups" else (M, w.N)
+                    accs.append(torch.empty(shape, dtype=torch.int32, device=dev))
+                    dumps[i] = accs[-1].data_ptr()
                 arr[i] = _lib.Problem(qa.q.data_ptr(), qa.s_a.data_ptr(), qa.rowsum.data_ptr(), w.w_r.data_ptr(),
                                       w.s_r.data_ptr(), w.zp_r.data_ptr() if w.zp_r is not None else None,
                                       out.data_ptr(), qa.q.stride(0), qa.rowsum.stride(0), out.stride(0),
                                       M, w.N, K, w.zp_const)
-            _lib.check(L.slimk_w2a8_gemm_grouped(ctypes.byref(arr), len(chunk), g, _DT[out_dtype], _stream_ptr(dev)))
-    return outs
+            if dump is None:
+                _lib.check(L.slimk_w2a8_gemm_grouped(ctypes.byref(arr), len(chunk), g, _DT[out_dtype], _stream_ptr(dev)))
+            else:
+                _lib.check(L.slimk_w2a8_gemm_grouped_verify(
+                    ctypes.byref(arr), len(chunk), g, _DT[out_dtype], ctypes.byref(dumps),
+                    _lib.DUMP_GROUPS if dump == "groups" else _lib.DUMP_SUM, _stream_ptr(dev)))
+    return outs if dump is None else (outs, accs)
 
 
 def wint2_gemm(activation: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, zp=None,

@@ -56,14 +56,14 @@ def test_split_heuristic_and_workspace(L):
     s = L.slimk_w2a8_gemm_auto_split_k(16, 4096, 14336, 128, _lib.KERNEL_AUTO)
     assert s == 4
     ws = L.slimk_w2a8_gemm_workspace_bytes(16, 4096, 14336, 128, _lib.KERNEL_AUTO, 0)
-    assert ws == 256 + s * 64 * (16 * 64) * 4     # counters + split x strips x (16 x 64 fp32 tile)
+    assert ws == 65536 + s * 64 * (16 * 64) * 4     # fixed counter block + split x strips x (16 x 64 fp32 tile)
     # 17..32 tokens run as two blocks of 16 rows: one counter and one tile per (strip, block)
-    assert L.slimk_w2a8_gemm_workspace_bytes(32, 4096, 14336, 128, _lib.KERNEL_AUTO, 4) == 512 + 4 * 64 * 2 * (16 * 64) * 4
+    assert L.slimk_w2a8_gemm_workspace_bytes(32, 4096, 14336, 128, _lib.KERNEL_AUTO, 4) == 65536 + 4 * 64 * 2 * (16 * 64) * 4
     # the tiled kernel splits K only when its 64-row tiles would leave CUs idle
     assert L.slimk_w2a8_gemm_auto_split_k(4096, 14336, 4096, 128, _lib.KERNEL_AUTO) == 1
     s = L.slimk_w2a8_gemm_auto_split_k(512, 4096, 14336, 128, _lib.KERNEL_AUTO)      # 16 x 8 tiles, 112 stages
     assert s == 4
-    assert L.slimk_w2a8_gemm_workspace_bytes(512, 4096, 14336, 128, _lib.KERNEL_AUTO, 0) == 512 + s * 128 * (64 * 256) * 4
+    assert L.slimk_w2a8_gemm_workspace_bytes(512, 4096, 14336, 128, _lib.KERNEL_AUTO, 0) == 65536 + s * 128 * (64 * 256) * 4
     assert L.slimk_w2a8_gemm_auto_split_k(0, 4096, 4096, 128, 0) == 0
 
 
@@ -97,7 +97,12 @@ def test_gemm_argument_validation(L):
     assert _gemm(L, dump=1, acc=None) == 1
     assert _gemm(L, M=64, ldr=64, kernel=_lib.KERNEL_SKINNY) == 7
     assert _gemm(L, M=64, ldr=64, kernel=_lib.KERNEL_TILED, split=2) == 5       # valid, but needs a workspace
-    assert _gemm(L, M=64, ldr=64, kernel=_lib.KERNEL_TILED, split=2, dump=2, acc=FAKE) == 7   # the verification kernel cannot split
+    assert _gemm(L, M=64, ldr=64, kernel=_lib.KERNEL_TILED, split=2, dump=2, acc=FAKE) == 5   # the verification instantiation splits alike
+    # row sums fold zero-points: the tiled kernel with the uniform zero-point 2 reads none, everything else needs them
+    assert _gemm(L, rowsum=None) == 1 and b"rowsum" in L.slimk_w2a8_last_error()
+    assert _gemm(L, M=64, rowsum=None, kernel=_lib.KERNEL_TILED, zp_const=1) == 1
+    assert _gemm(L, M=64, rowsum=None, kernel=_lib.KERNEL_TILED, g=256) == 1
+    assert _gemm(L, M=64, rowsum=None, kernel=_lib.KERNEL_TILED, split=2) == 5                # accepted up to the workspace check
     # split-K without / with too small a workspace (N = 4096, K = 14336 wants split 4)
     assert _gemm(L, K=14336, ldq=14336) == 5 and b"workspace" in L.slimk_w2a8_last_error()
     assert _gemm(L, K=14336, ldq=14336, ws=FAKE, wsb=1024) == 5
@@ -152,14 +157,14 @@ def test_repack_and_act_quant_validation(L):
     assert g4(FAKE, 4096, FAKE, None, 0, FAKE, FAKE, None, 64, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 33, None) == 2   # more splits than stages
     s4 = L.slimk_w4a8_gemm_auto_split_k(64, 4096, 4096, 128)           # 16 tiles, 32 stages: 4 splits of 8 stages
     assert s4 == 4
-    assert L.slimk_w4a8_gemm_workspace_bytes(64, 4096, 4096, 128, 0) == 256 + 4 * 16 * 64 * 256 * 4
+    assert L.slimk_w4a8_gemm_workspace_bytes(64, 4096, 4096, 128, 0) == 65536 + 4 * 16 * 64 * 256 * 4
     assert L.slimk_w4a8_gemm_auto_split_k(2048, 14336, 4096, 128) == 1 and L.slimk_w4a8_gemm_workspace_bytes(2048, 14336, 4096, 128, 0) == 0
     assert L.slimk_w4a8_gemm_auto_split_k(64, 4096, 4096, 256) == 0
     q4 = L.slimk_w2a8_quantize_weight4  # (w, ldw, dtype, N, K, group, mode, planes, ldp, scales2, zp2, stream)
     assert q4(FAKE, 4096, 0, 64, 4096, 128, 1, FAKE, 2048, FAKE, None, None) == 1       # zero-points are always written
     assert q4(FAKE, 4096, 0, 64, 4096, 128, 0, FAKE, 2048, FAKE, FAKE, None) == 4       # no REF mode at four bits
     assert q4(FAKE, 4096, 0, 64, 4096, 128, 1, FAKE, 1024, FAKE, FAKE, None) == 2       # ldp < K/2
-    assert q4(FAKE, 4096, 0, 70000, 4096, 128, 1, FAKE, 2048, FAKE, FAKE, None) == 2
+    assert q4(FAKE, 4096, 0, 0, 4096, 128, 1, FAKE, 2048, FAKE, FAKE, None) == 2
     assert q4(FAKE, 4100, 0, 64, 4096, 128, 2, FAKE, 2048, FAKE, FAKE, None) == 3
     # (x, ldx, dtype, w_r, s_r, zp_r, zp_const, M, N, K, group, out, ldo, out_dtype, ws, ws_bytes, split, stream)
     gf = L.slimk_w2a8_gemm_fused

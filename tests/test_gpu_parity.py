@@ -39,7 +39,7 @@ def test_repack_matches_layout_definition(gpu_ops, N, K, g, with_zp):
 @pytest.mark.parametrize("N,K,g,mode,bf16", [(64, 256, 128, "sym", False), (100, 512, 64, "asym", False),
                                              (7, 768, 256, "ref", False), (130, 1024, 128, "asym", True),
                                              (33, 8192, 128, "sym", True), (256, 4096, 64, "ref", False)])
-def test_weight_quantisation_on_gpu_bit_exact(gpu_ops, N, K, g, mode, bf16):
+def test_weight_quantisation_on_gpu_bit_exact(gpu_ops, oracle, N, K, g, mode, bf16):
     """fp16 / bf16 weight -> packed codes, fp16 scales, zero-points: the host functions' numbers."""
     from slimkernels_amd import prepare_w2
     _say("quantize_weight", N, K, g, mode, bf16)
@@ -58,6 +58,13 @@ def test_weight_quantisation_on_gpu_bit_exact(gpu_ops, N, K, g, mode, bf16):
     host = prepare_w2(wt.float().numpy(), g, mode)
     packed, scales, zero = gpu_ops.quantize_weight_gpu(wt.cuda(), g, mode)
     torch.cuda.synchronize()
+    # against the oracle itself: its C quantiser on the [K, N] matrix, its packer on the transposed codes, its
+    # float32 scales rounded once to float16
+    o_codes, o_scales, o_zp = oracle.c_quantize_w2(np.ascontiguousarray(wt.float().numpy().T), g, mode)
+    np.testing.assert_array_equal(packed.cpu().numpy(), oracle.c_pack(np.ascontiguousarray(o_codes.T)))
+    np.testing.assert_array_equal(scales.cpu().numpy().view(np.uint16), o_scales.astype(np.float16).view(np.uint16))
+    np.testing.assert_array_equal(zero.cpu().numpy(), o_zp)
+    # and against the package's host functions
     np.testing.assert_array_equal(packed.cpu().numpy(), host[0])
     np.testing.assert_array_equal(scales.cpu().numpy().view(np.uint16), host[1].view(np.uint16))
     np.testing.assert_array_equal(zero.cpu().numpy(), host[2])
@@ -103,7 +110,11 @@ def test_act_quant_bit_exact(gpu_ops, oracle, M, K, g, bf16, outliers):
 
 
 # ------------------------------------------------------------------ GEMM on small and ragged shapes
-def _run_case(gpu_ops, oracle, case, kernel, split_k=0, dump="groups", exact_out=False, same_bits=True):
+def _run_case(gpu_ops, oracle, case, kernel, split_k=0, dump="groups", exact_out=False, same_bits=True, strict=False):
+    """One GEMM twice: with the int32 dump (the verification instantiation of the kernel body the call
+    selects) and without (the production instantiation of the same body).  int8 activations and int32
+    accumulators exact; outputs bit-identical with the oracle (exact_out), or within rtol 1e-3 / 1 ULP
+    (strict: kernels that sum in the oracle's order), or additionally within the re-association bound."""
     _say("gemm", case.name, kernel, "split", split_k, "dump", dump)
     packed, scales, zero = pu.quantized_weight(case)
     x = workloads.make_activation(case)
@@ -125,8 +136,8 @@ def _run_case(gpu_ops, oracle, case, kernel, split_k=0, dump="groups", exact_out
         if exact_out:
             np.testing.assert_array_equal(bits, ref["out_bits"])
         else:
-            pu.assert_out_close(bits, ref["out_bits"], bf16, bound, case.name)
-    if same_bits:  # the verification instantiation and the production one run the same kernel body
+            pu.assert_out_close(bits, ref["out_bits"], bf16, None if strict else bound, case.name)
+    if same_bits:  # the verification instantiation and the production one are the same kernel body
         np.testing.assert_array_equal(pu.out_tensor_bits(out), pu.out_tensor_bits(out2))
 
 
@@ -174,10 +185,9 @@ def test_skinny_wide_activation_fetch(gpu_ops, oracle, M, N, K, g, mode, out, sp
 ])
 def test_skinny_shared_one_problem(gpu_ops, oracle, M, N, K, g, mode, out, split):
     """17..32 token rows on a matrix of 24 MiB or more: one problem runs through the shared-activation
-    workgroups with K split across workgroups.  The int32 dump comes from the one-strip kernel's
-    verification build, so the two outputs are each held to the output criterion, not to each other."""
+    workgroups with K split across workgroups; the int32 dump comes from the same body."""
     case = pu.small_case(M, N, K, g, mode, seed=M + K, out_dtype=out)
-    _run_case(gpu_ops, oracle, case, "skinny", split_k=split, dump="sum", same_bits=False)
+    _run_case(gpu_ops, oracle, case, "skinny", split_k=split, dump="sum")
 
 
 @pytest.mark.parametrize("M,N,K,g,mode,out", SMALL + [
@@ -190,7 +200,7 @@ def test_tiled_small(gpu_ops, oracle, M, N, K, g, mode, out):
     # unsplit and with the zero-point the operand bytes are centred on (the symmetric levels), the tiled
     # kernels sum the groups in the oracle's order: bit-identical outputs.  Other zero-points add their
     # term through fp32 MFMAs first: the output criterion.
-    exact = mode == "sym"
+    exact = mode == "sym" and g <= 128 and K % 128 == 0   # (other shapes run the generic kernel: the output criterion)
     _run_case(gpu_ops, oracle, case, "tiled", split_k=1, dump="groups", exact_out=exact)
     _run_case(gpu_ops, oracle, case, "tiled", split_k=1, dump="sum", exact_out=exact)
     # whatever split the library picks by itself (K may be split when tiles are few): the output criterion
@@ -261,11 +271,58 @@ def test_config_c1(gpu_ops, oracle):
 
 
 @pytest.mark.parametrize("shape", ["qo", "kv", "gate_up", "down"])
-@pytest.mark.parametrize("M", [1, 8, 32])
+@pytest.mark.parametrize("M", list(workloads.DECODE_M))
 def test_config_c2_decode(gpu_ops, oracle, shape, M):
     N, K = workloads.LLAMA8B_LINEARS[shape]
     case = workloads.Case("c2", M, N, K, outliers=True)
     _run_case(gpu_ops, oracle, case, "auto")
+
+
+def test_config_c2_as_one_grouped_launch(gpu_ops, oracle):
+    """The benchmark's step: exactly the 24 GEMMs of the decode sweep (M in {1,2,4,8,16,32} x the four Llama-3-8B
+    linears, outlier channels) issued as ONE grouped launch.  The verification instantiation of the grouped kernel
+    gives every problem's int32 accumulators (exact against the oracle); the production launch's outputs are
+    bit-identical with the verification launch's and meet the output criterion against the oracle."""
+    cases = workloads.config_cases("c2")
+    assert len(cases) == 24
+    weights, probs, refs = {}, [], []
+    for c in cases:
+        if (c.N, c.K) not in weights:
+            packed, scales, zero = pu.quantized_weight(c)
+            weights[(c.N, c.K)] = (packed, scales, zero, gpu_ops.repack_w2(packed, scales, None, c.group_size, zp_const=2))
+        packed, scales, zero, w = weights[(c.N, c.K)]
+        x = workloads.make_activation(c)
+        probs.append((gpu_ops.quantize_act_int8(torch.from_numpy(x).cuda(), c.group_size), w))
+        refs.append((oracle.reference_forward(x, packed, scales, zero, c.group_size, want_acc=True), scales))
+    _say("grouped launch of the", len(probs), "c2 problems")
+    outs = gpu_ops.w2a8_gemm_grouped(probs)
+    outs_v, accs = gpu_ops.w2a8_gemm_grouped(probs, dump="groups")
+    torch.cuda.synchronize()
+    for c, o, ov, acc, (ref, scales) in zip(cases, outs, outs_v, accs, refs):
+        np.testing.assert_array_equal(acc.cpu().numpy(), ref["acc"], err_msg=c.name)
+        np.testing.assert_array_equal(pu.out_tensor_bits(o), pu.out_tensor_bits(ov), err_msg=c.name)
+        pu.assert_out_close(pu.out_tensor_bits(o), ref["out_bits"], False,
+                            pu.reorder_bound(ref["acc"], scales, ref["s_a"]), "c2 grouped " + c.name)
+
+
+def test_workspace_serves_changing_shapes(gpu_ops, oracle):
+    """One weight object, one lazily created split-K workspace, token counts that change from call to call (tiled
+    split 8 -> skinny split 4, and two tiled splits with different tile counts): the arrival counters sit in a block
+    of fixed size in front of the partial sums, so a later call's counters never land on an earlier call's partials."""
+    N, K, g = 4096, 14336, 128
+    base = pu.small_case(1, N, K, g, "sym", seed=21)
+    packed, scales, zero = pu.quantized_weight(base)
+    w = gpu_ops.repack_w2(packed, scales, None, g, zp_const=2)
+    for M in (64, 20, 256, 320, 20, 64):
+        case = pu.small_case(M, N, K, g, "sym", seed=100 + M)
+        x = workloads.make_activation(case)
+        ref = oracle.reference_forward(x, packed, scales, zero, g, want_acc=True)
+        out = gpu_ops.w2a8_gemm(gpu_ops.quantize_act_int8(torch.from_numpy(x).cuda(), g), w)
+        torch.cuda.synchronize()
+        _say("workspace reuse M", M, "workspace bytes", 0 if w.workspace is None else w.workspace.numel())
+        pu.assert_out_close(pu.out_tensor_bits(out), ref["out_bits"], False,
+                            pu.reorder_bound(ref["acc"], scales, ref["s_a"]), f"workspace reuse M={M}")
+    assert int(w.workspace[:65536].view(torch.int32).abs().max()) == 0   # the counter block is back at zero
 
 
 def test_config_c5_asym_ragged(gpu_ops, oracle):
