@@ -216,6 +216,28 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
                     void* workspace, size_t workspace_bytes,
                     int kernel, int split_k, void* stream);
 
+/* slimk_w2a8_gemm for callers that cannot allocate device memory and so cannot supply a split-K workspace: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart upstream (its
+ * launcher never splits K).  Same arguments and results as slimk_w2a8_gemm without acc_dump / dump_mode /
+ * workspace / workspace_bytes: the arrival counters and partial sums of a split-K launch live in a device array
+ * inside the library, SLIMK_W2A8_STATIC_WORKSPACE_BYTES per GPU the library is used on, held until the process
+ * ends.  The call allocates and frees nothing, on the device or through any library.
+ *  - split_k = 0: the library's choice, lowered until its workspace fits the array (bit-identical with
+ *    slimk_w2a8_gemm given the same effective split); an explicit split_k whose workspace
+ *    (slimk_w2a8_gemm_workspace_bytes) exceeds the array is refused with SLIMK_ERR_WORKSPACE before any launch.
+ *  - Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (different streams,
+ *    concurrent graph launches) race on it; calls ordered on one stream, of any shapes, are fine (each leaves
+ *    the counters at zero, the partial sums need no clearing).
+ *  - The first call on each GPU looks the array's address up and clears its counter block with a small kernel on
+ *    `stream`; make that call outside graph capture. */
+#define SLIMK_W2A8_STATIC_WORKSPACE_BYTES ((16u << 20) + (64u << 10))
+size_t slimk_w2a8_static_workspace_bytes(void);
+int slimk_w2a8_gemm_static(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,
+                           const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
+                           int M, int N, int K, int group_size,
+                           void* out, int ldo, int out_dtype,
+                           int kernel, int split_k, void* stream);
+
 /* The GEMM for at most four token rows with the activation quantisation inside: x [M][ldx] fp16 or
  * bf16 (x_dtype) takes the place of q, s_a and rowsum, and every workgroup quantises the rows itself
  * (same numbers as slimk_w2a8_act_quant) while its first weights are on the way - one launch

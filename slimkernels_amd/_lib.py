@@ -35,6 +35,8 @@ SIGNATURES = {
     "slimk_w2a8_act_quant_rep": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _vp]),
     "slimk_w2a8_gemm": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i,
                              _vp, _i, _i, _vp, _i, _vp, _sz, _i, _i, _vp]),
+    "slimk_w2a8_static_workspace_bytes": (_sz, []),
+    "slimk_w2a8_gemm_static": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _vp]),
     "slimk_w2a8_gemm_fused": (_i, [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _i, _vp, _sz, _i, _vp]),
     "slimk_w2a8_gemm_grouped": (_i, [_vp, _i, _i, _i, _vp]),
     "slimk_w2a8_gemm_grouped_verify": (_i, [_vp, _i, _i, _i, _vp, _i, _vp]),

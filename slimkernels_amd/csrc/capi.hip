@@ -4,10 +4,14 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include <mutex>
 #include <string>
 
 #include "../../include/slimk_w2a8.h"
 #include "w2a8_launch.h"
+
+// The library-owned split-K workspace of slimk_w2a8_gemm_static (see static_workspace() below).
+static __device__ __align__(256) unsigned char scratch[SLIMK_W2A8_STATIC_WORKSPACE_BYTES];
 
 namespace {
 
@@ -268,8 +272,8 @@ int slimk_w2a8_act_quant(const void* x, int ldx, int x_dtype, int M, int K, int 
 
 namespace {
 
-// fit_split: a split factor chosen here (split_k <= 0) is lowered until its workspace fits workspace_bytes;
-// a caller's explicit split never is.
+// fit_split: a split factor chosen here (split_k <= 0) is lowered until its workspace fits workspace_bytes
+// (the library-owned workspace of slimk_w2a8_gemm_static has a fixed size); a caller's explicit split never is.
 int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,
               const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
               int M, int N, int K, int group_size,
@@ -372,6 +376,35 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
     return hip_result(w2a8::launch_tiled(p, gs, asym, out_bf16, st), "tiled gemm");
 }
 
+// ---- the library-owned split-K workspace of slimk_w2a8_gemm_static: a device array of fixed size, one copy per GPU
+// the library runs on, held until the process ends.  Its name is a host-side stand-in, not a device address:
+// the address on the current device comes from hipGetSymbolAddress, once per device, and only that pointer is
+// ever handed to a kernel.
+constexpr size_t kStaticWorkspaceBytes = SLIMK_W2A8_STATIC_WORKSPACE_BYTES;
+static_assert(kStaticWorkspaceBytes > kCounterBlockBytes && kStaticWorkspaceBytes % 256 == 0, "static workspace size");
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices];   // per device: where that device's copy of `scratch` lives (nullptr: not asked yet)
+
+// The current device's copy of the array; on the first call on a device its counter block is cleared on `stream`
+// (the array starts as zeros and every GEMM leaves its counters at zero, so this only guards the very first use).
+int static_workspace(void** ptr, hipStream_t stream) {
+    int dev = -1;
+    if (hipError_t e = hipGetDevice(&dev)) return hip_result(e, "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return fail(SLIMK_ERR_UNSUPPORTED, "device ordinal %d (at most %d devices)", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) return hip_result(e, "hipGetSymbolAddress(scratch)");
+        if (!p || !aligned16(p)) return fail(SLIMK_ERR_HIP, "hipGetSymbolAddress(scratch) returned %p", p);
+        if (int rc = hip_result(w2a8::launch_fill_zero(p, kCounterBlockBytes, stream), "static workspace clear")) return rc;
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return SLIMK_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -385,6 +418,27 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
                     int kernel, int split_k, void* stream) {
     return gemm_impl(q, ldq, s_a, rowsum, ldr, w_r, s_r, zp_r, zp_const, M, N, K, group_size, out, ldo, out_dtype,
                      acc_dump, dump_mode, workspace, workspace_bytes, kernel, split_k, stream, false);
+}
+
+size_t slimk_w2a8_static_workspace_bytes(void) { return kStaticWorkspaceBytes; }
+
+int slimk_w2a8_gemm_static(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,
+                           const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
+                           int M, int N, int K, int group_size,
+                           void* out, int ldo, int out_dtype,
+                           int kernel, int split_k, void* stream) {
+    // an explicit split beyond the fixed workspace is an error here, before anything touches the GPU
+    if (split_k > 1 && M > 0 && N > 0 && shape_ok(K, group_size) && kernel >= SLIMK_KERNEL_AUTO && kernel <= SLIMK_KERNEL_TILED) {
+        const size_t need = slimk_w2a8_gemm_workspace_bytes(M, N, K, group_size, kernel, split_k);
+        if (need > kStaticWorkspaceBytes)
+            return fail(SLIMK_ERR_WORKSPACE, "gemm_static: split_k=%d needs %zu bytes of workspace, the library-owned one holds %zu "
+                        "(pass a smaller split_k, 0 to let the library choose one that fits, or use slimk_w2a8_gemm)",
+                        split_k, need, kStaticWorkspaceBytes);
+    }
+    void* ws = nullptr;
+    if (int rc = static_workspace(&ws, (hipStream_t)stream)) return rc;
+    return gemm_impl(q, ldq, s_a, rowsum, ldr, w_r, s_r, zp_r, zp_const, M, N, K, group_size, out, ldo, out_dtype,
+                     nullptr, SLIMK_DUMP_NONE, ws, kStaticWorkspaceBytes, kernel, split_k, stream, true);
 }
 
 int slimk_w2a8_gemm_fused(const void* x, int ldx, int x_dtype,

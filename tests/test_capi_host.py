@@ -111,6 +111,15 @@ def test_gemm_argument_validation(L):
     assert _gemm(L, N=1 << 19, ldo=1 << 19, K=1 << 16, ldq=1 << 16) == 7 and b"2 GiB" in L.slimk_w2a8_last_error()
 
 
+def test_gemm_static_refuses_an_oversized_split_on_the_host(L):
+    """The entry point that allocates nothing owns 16 MiB + 64 KiB of workspace: an explicit split beyond it is
+    refused before any GPU call (so this runs without a GPU)."""
+    assert L.slimk_w2a8_static_workspace_bytes() == (16 << 20) + (64 << 10)
+    rc = L.slimk_w2a8_gemm_static(FAKE, 14336, FAKE, FAKE, 512, FAKE, FAKE, None, 2, 512, 4096, 14336, 128,
+                                  FAKE, 4096, 0, _lib.KERNEL_TILED, 8, None)
+    assert rc == 5 and b"library-owned" in L.slimk_w2a8_last_error()
+
+
 def test_repack_and_act_quant_validation(L):
     r = L.slimk_w2a8_repack
     assert r(None, 1024, FAKE, None, 4096, 4096, 128, FAKE, FAKE, None, None) == 1
