@@ -41,8 +41,11 @@ COLD_FOOTPRINT = 640 << 20    # bytes of distinct weight copies between two uses
 # `python3 bench.py --skip-detail` (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same
 # counter reads for this file's 256 MiB calibration read (read_probe_kernel: 131080 -> x2.0) and
 # calibration fill (fill_zero_kernel: 262144 -> x1.0):  (115983 * 2.0 + 2898 * 1.0) KiB.
+# Counters cannot be read from inside a run: the figure is the one of the committed profile summary named in
+# TRAFFIC_SOURCE, taken on the same kernel code (the summary gives the command).
 CLOCK_WARMUP_MS = 150   # untimed run of the measured work before every timed region (see timed_run, time_graph)
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = int((115983 * 2.0 + 2898 * 1.0) * 1024)
+TRAFFIC_SOURCE = "profiles/skinny_grouped_kernel__c2_decode_sweep.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by the in-run 256 MiB read / fill calibration)"
 
 
 def main():
@@ -210,7 +213,7 @@ def main():
                    "clock_warmup_ms": CLOCK_WARMUP_MS},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "w2a8::skinny_grouped_kernel", "avg_launch_us": round(avg_launch_us, 3),
+                     "traffic_source": TRAFFIC_SOURCE, "kernel": "w2a8::skinny_grouped_kernel", "avg_launch_us": round(avg_launch_us, 3),
                      "algorithmic_bytes_per_launch": step_bytes},
     }
 
@@ -232,11 +235,43 @@ def main():
             import traceback
             traceback.print_exc(file=sys.stderr)
             detail["detail_error"] = repr(e)
+        result["roofline"]["also"] = also_rows(detail, step_bytes, len(cases))
         result["cpu_baseline"] = cpu_baseline(np, workloads, shapes)
     else:
         result["cpu_baseline"] = None
     result["detail"] = detail
     print(json.dumps(result))
+
+
+def also_rows(detail, step_bytes, n_gemms):
+    """The other half of the metric and the single-GEMM figures, lifted out of `detail` into the `roofline` object:
+    int8-MFMA fractions of the tiled kernel at M >= 2048 (c3, and c4 at its largest shapes), HBM fractions of single
+    decode GEMMs (c4 at M = 1 / 16, the c2 sweep as 24 launches) and of the grouped sweep restricted to M <= 16."""
+    rows = []
+    for r in detail.get("prefill", []):
+        if r["M"] >= 2048:
+            rows.append({"bound": "int8_mfma", "workload": f"c3 M={r['M']} {r['shape']} g128", "kernel": "w2a8::tiled_kernel",
+                         "avg_us": r["us"], "achieved": r["TOPS"], "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": r["frac_int8_mfma"]})
+    for r in detail.get("other_configs", []):
+        if r["config"] == "c4" and r["M"] >= 2048:
+            rows.append({"bound": "int8_mfma", "workload": f"c4 M={r['M']} {r['shape']} g64 bf16", "kernel": "w2a8::tiled_kernel",
+                         "avg_us": r["us"], "achieved": r["TOPS"], "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": r["frac_int8_mfma"]})
+        elif r["config"] == "c4" and r["M"] <= 16:
+            rows.append({"bound": "hbm", "workload": f"c4 M={r['M']} {r['shape']} g64 bf16, one GEMM per launch, cold", "kernel": "w2a8::skinny_kernel",
+                         "avg_us": r["us"], "achieved": r["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": r["frac_hbm"]})
+        elif r["config"] in ("c4", "c5"):
+            rows.append({"bound": "near the ridge (both given)", "workload": f"{r['config']} M={r['M']} {r['shape']} g{r['group']} {r['mode']}",
+                         "avg_us": r["us"], "frac_hbm": r["frac_hbm"], "frac_int8_mfma": r["frac_int8_mfma"]})
+    if "single_launch" in detail:
+        sl = detail["single_launch"]
+        rows.append({"bound": "hbm", "workload": "c2 sweep as 24 launches, one GEMM each (latency-bound)", "kernel": "w2a8::skinny_kernel",
+                     "avg_us": sl["avg_launch_us"], "achieved": sl["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": sl["frac_hbm"]})
+    if "decode_sweep_m_le_16" in detail:
+        r = detail["decode_sweep_m_le_16"]
+        rows.append({"bound": "hbm", "workload": "c2 sweep restricted to M <= 16 (20 GEMMs), one grouped launch, cold",
+                     "kernel": "w2a8::skinny_grouped_kernel", "avg_us": r["us"], "achieved": r["GBps"], "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": r["frac_hbm"]})
+    return rows
 
 
 def _lib_check(rc):
@@ -299,6 +334,23 @@ def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, d
         row["cold_frac_hbm"] = round(row["cold_GBps"] / HBM_PEAK_GBPS, 4)
         table.append(row)
     detail["decode"] = table
+
+    # ---- the grouped sweep restricted to M <= 16 (the rows the HBM target is worded on): 20 GEMMs, one launch, cold
+    small = [c for c in cases if c.M <= 16]
+    nb16 = sum(workloads.algorithmic_bytes(c) for c in small)
+    n_rot = max(len(sh.copies) for sh in shapes.values())
+
+    def sweep16():
+        for rot in range(n_rot):
+            probs = []
+            for i, c in enumerate(small):
+                sh = shapes[name_of[(c.N, c.K)]]
+                _, qa, out = acts[(c.N, c.K, c.M)]
+                probs.append((qa, sh.copies[(rot * 5 + i) % len(sh.copies)], out))
+            ops.w2a8_gemm_grouped(probs, torch.float16)
+    us = time_graph(torch, sweep16, n_rot, replays=6)
+    detail["decode_sweep_m_le_16"] = {"gemms": len(small), "bytes": nb16, "us": round(us, 2), "GBps": round(nb16 / (us * 1e-6) / 1e9, 1),
+                                      "frac_hbm": round(nb16 / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
 
     # ---- activation quantisation, timed on its own (bytes: 2MK read + MK + 4M + 4MG written)
     aq = []

@@ -68,8 +68,19 @@ int strips_of(int N) { return (N + w2a8::kStripN - 1) / w2a8::kStripN; }
 constexpr size_t kCounterBlockBytes = 64 << 10;
 constexpr int kMaxCounters = (int)(kCounterBlockBytes / sizeof(unsigned));
 
-int resolve_kernel(int M, int kernel) {
-    if (kernel == SLIMK_KERNEL_AUTO) return M <= 32 ? SLIMK_KERNEL_SKINNY : SLIMK_KERNEL_TILED;
+// The skinny kernel takes any number of token rows (16 or 32 at a time, each pass re-reading the weights, from the
+// second on out of L2).  Measured against the tiled kernel on 33..256 rows: it wins while the reduction is short
+// (K <= 4096: the tiled kernel's few stages do not amortise its start-up) and the passes over the weights stay under
+// about 100 MiB in all (14336 x 4096: up to 96 rows, 11008 x 4096: up to 160, 4096 x 4096: 15.9 -> 9.6 us at 128 rows).
+constexpr int kSkinnyMaxRows = 256;
+bool skinny_wins_mid(int M, int N, int K) {
+    if (M <= 32 || M > kSkinnyMaxRows || K > 4096) return false;
+    const size_t weight_bytes = (size_t)strips_of(N) * 64 * (K / 4);
+    return (size_t)((M + 15) / 16) * weight_bytes <= ((size_t)100 << 20);
+}
+
+int resolve_kernel(int M, int N, int K, int kernel) {
+    if (kernel == SLIMK_KERNEL_AUTO) return M <= 32 || skinny_wins_mid(M, N, K) ? SLIMK_KERNEL_SKINNY : SLIMK_KERNEL_TILED;
     return kernel;
 }
 
@@ -169,12 +180,12 @@ size_t slimk_w2a8_repacked_zp_bytes(int N, int K, int group_size) {
 
 int slimk_w2a8_gemm_auto_split_k(int M, int N, int K, int group_size, int kernel) {
     if (M <= 0 || N <= 0 || !shape_ok(K, group_size)) return 0;
-    return auto_split(M, N, K, group_size, resolve_kernel(M, kernel));
+    return auto_split(M, N, K, group_size, resolve_kernel(M, N, K, kernel));
 }
 
 size_t slimk_w2a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int kernel, int split_k) {
     if (M <= 0 || N <= 0 || !shape_ok(K, group_size)) return 0;
-    const int kern = resolve_kernel(M, kernel);
+    const int kern = resolve_kernel(M, N, K, kernel);
     if (split_k <= 0) split_k = auto_split(M, N, K, group_size, kern);
     if (split_k <= 1) return 0;
     const int strips = strips_of(N);
@@ -285,7 +296,7 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
     if (M <= 0 || N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "M=%d, N=%d must be positive", M, N);
     if (int rc = check_kg(K, group_size)) return rc;
     // the row sums fold zero-points; the fast tiled kernel centres its operand bytes on 2 and reads none for that value
-    const bool rowsum_unused = !zp_r && zp_const == 2 && resolve_kernel(M, kernel) == SLIMK_KERNEL_TILED &&
+    const bool rowsum_unused = !zp_r && zp_const == 2 && resolve_kernel(M, N, K, kernel) == SLIMK_KERNEL_TILED &&
                                group_size <= 128 && K % 128 == 0;
     if (!rowsum && !rowsum_unused)
         return fail(SLIMK_ERR_NULL_POINTER, "gemm: rowsum is NULL (only the tiled kernel with the uniform zero-point 2, group 64 / 128 and K %% 128 == 0 does without)");
@@ -302,9 +313,9 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
         return fail(SLIMK_ERR_MISALIGNED, "gemm: q, rowsum, w_r, s_r, zp_r must be 16-byte aligned; ldq %% 16 == 0; ldr %% 4 == 0");
     if ((reinterpret_cast<uintptr_t>(out) & 1u) != 0) return fail(SLIMK_ERR_MISALIGNED, "gemm: out must be 2-byte aligned");
 
-    const int kern = resolve_kernel(M, kernel);
-    if (kern == SLIMK_KERNEL_SKINNY && M > 32)
-        return fail(SLIMK_ERR_UNSUPPORTED, "the skinny kernel handles M <= 32 (M=%d)", M);
+    const int kern = resolve_kernel(M, N, K, kernel);
+    if (kern == SLIMK_KERNEL_SKINNY && M > kSkinnyMaxRows)
+        return fail(SLIMK_ERR_UNSUPPORTED, "the skinny kernel handles M <= %d (M=%d)", kSkinnyMaxRows, M);
     const int G = K / group_size;
     const bool split_chosen_here = split_k <= 0;
     if (split_k <= 0) {

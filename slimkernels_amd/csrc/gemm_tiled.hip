@@ -375,27 +375,32 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
         }
         __syncthreads();
         if (lds[0][0] == 0) return;
-        // one split at a time, all of its fragments in flight together (one memory latency per split)
+        // one split at a time, four token blocks' fragments in flight together (one memory latency per split and
+        // half tile; all eight blocks at once would not fit the registers next to the running sums)
+        constexpr int kChunk = 4;
 #pragma unroll
-        for (int mb = 0; mb < kMB; ++mb)
+        for (int mb0 = 0; mb0 < kMB; mb0 += kChunk) {
 #pragma unroll
-            for (int pp = 0; pp < 4; ++pp)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) t[mb][pp][j] = 0.0f;
-        for (int sp = 0; sp < n_split; ++sp) {
-            v4f v[kMB][4];
-#pragma unroll
-            for (int mb = 0; mb < kMB; ++mb)
-#pragma unroll
-                for (int pp = 0; pp < 4; ++pp)
-                    v[mb][pp] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
-                        ws_rsrc, ws_lane + (mb * 4 + pp) * 1024, sp * ws_split_pitch + ws_tile, kCoherent));
-#pragma unroll
-            for (int mb = 0; mb < kMB; ++mb)
+            for (int mb = 0; mb < kChunk; ++mb)
 #pragma unroll
                 for (int pp = 0; pp < 4; ++pp)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) t[mb][pp][j] += v[mb][pp][j];
+                    for (int j = 0; j < 4; ++j) t[mb0 + mb][pp][j] = 0.0f;
+            for (int sp = 0; sp < n_split; ++sp) {
+                v4f v[kChunk][4];
+#pragma unroll
+                for (int mb = 0; mb < kChunk; ++mb)
+#pragma unroll
+                    for (int pp = 0; pp < 4; ++pp)
+                        v[mb][pp] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
+                            ws_rsrc, ws_lane + ((mb0 + mb) * 4 + pp) * 1024, sp * ws_split_pitch + ws_tile, kCoherent));
+#pragma unroll
+                for (int mb = 0; mb < kChunk; ++mb)
+#pragma unroll
+                    for (int pp = 0; pp < 4; ++pp)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) t[mb0 + mb][pp][j] += v[mb][pp][j];
+            }
         }
         if (tid == 0) __hip_atomic_store(p.ws_counter + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -467,9 +472,9 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
 }
 
 // 128-row tiles: two workgroups (eight waves) per CU; 64-row tiles need fewer registers: three.
-template <int GS, bool ZP, typename OutT, bool DUMP = false>
+template <int GS, bool SPLIT, bool ZP, typename OutT, bool DUMP = false>
 __global__ __launch_bounds__(256, 2) void tiled_kernel(const GemmParams p) {
-    tiled_body<128, GS, false, ZP, OutT, false, DUMP>(p);
+    tiled_body<128, GS, SPLIT, ZP, OutT, false, DUMP>(p);
 }
 template <int GS, bool SPLIT, bool ZP, typename OutT, bool DUMP = false>
 __global__ __launch_bounds__(256, DUMP ? 2 : 3) void tiled_kernel_bm64(const GemmParams p) {
@@ -552,7 +557,7 @@ static void tiled_fast_tiles(int M, int strips, int* bm, int* tiles) {
 int tiled_fast_max_split(int M, int strips, int steps) {
     int bm, tiles;
     tiled_fast_tiles(M, strips, &bm, &tiles);
-    if (bm != 64 || steps % fast::kStageSteps != 0) return 1;
+    if (steps % fast::kStageSteps != 0) return 1;
     return steps / fast::kStageSteps;
 }
 
@@ -565,7 +570,7 @@ int tiled_fast_max_split(int M, int strips, int steps) {
 int tiled_fast_auto_split(int M, int strips, int steps) {
     int bm, tiles;
     tiled_fast_tiles(M, strips, &bm, &tiles);
-    if (bm != 64 || steps % fast::kStageSteps != 0) return 1;
+    if (steps % fast::kStageSteps != 0) return 1;
     const int stages = steps / fast::kStageSteps;
     // one workgroup per CU on most CUs and a long reduction: two halves (measured at 128 x 28672 x 8192,
     // 224 tiles of 64 stages: 67.5 -> 61.2 us; at 32 stages per tile the halves are slower: 28.1 -> 31.6 us)
@@ -578,10 +583,11 @@ int tiled_fast_auto_split(int M, int strips, int steps) {
     return (stages + sps - 1) / sps;
 }
 
+// in units of 64 x 256 tiles (a 128-row tile counts twice)
 size_t tiled_fast_workspace_tiles(int M, int strips) {
     int bm, tiles;
     tiled_fast_tiles(M, strips, &bm, &tiles);
-    return (size_t)tiles;
+    return (size_t)tiles * (bm / 64);
 }
 
 hipError_t launch_tiled(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream) {
@@ -590,23 +596,29 @@ hipError_t launch_tiled(const GemmParams& p, int gs, bool asym, bool out_bf16, h
     tiled_fast_tiles(p.M, p.strips, &bm, &tiles);
     const dim3 grid((tiles + 7) / 8 * 8, p.split > 1 ? p.split : 1), block(256);
     const bool zp = asym || p.zp_const != 2;
-    const bool split = bm == 64 && p.split > 1;
+    const bool split = p.split > 1;
     const bool dump = p.acc_dump != nullptr && p.dump_mode != 0;
     // a verification call runs the same body with the dump switched on (same tile height, same split)
 #define SLIMK_TILED_LAUNCH(GSV, ZPV)                                                                          \
     do {                                                                                                      \
-        if (dump && bm == 128) {                                                                              \
-            if (out_bf16) tiled_kernel<GSV, ZPV, OutBF16, true><<<grid, block, 0, stream>>>(p);               \
-            else tiled_kernel<GSV, ZPV, OutF16, true><<<grid, block, 0, stream>>>(p);                         \
+        if (dump && bm == 128 && split) {                                                                     \
+            if (out_bf16) tiled_kernel<GSV, true, ZPV, OutBF16, true><<<grid, block, 0, stream>>>(p);         \
+            else tiled_kernel<GSV, true, ZPV, OutF16, true><<<grid, block, 0, stream>>>(p);                   \
+        } else if (dump && bm == 128) {                                                                       \
+            if (out_bf16) tiled_kernel<GSV, false, ZPV, OutBF16, true><<<grid, block, 0, stream>>>(p);        \
+            else tiled_kernel<GSV, false, ZPV, OutF16, true><<<grid, block, 0, stream>>>(p);                  \
         } else if (dump && split) {                                                                           \
             if (out_bf16) tiled_kernel_bm64<GSV, true, ZPV, OutBF16, true><<<grid, block, 0, stream>>>(p);    \
             else tiled_kernel_bm64<GSV, true, ZPV, OutF16, true><<<grid, block, 0, stream>>>(p);              \
         } else if (dump) {                                                                                    \
             if (out_bf16) tiled_kernel_bm64<GSV, false, ZPV, OutBF16, true><<<grid, block, 0, stream>>>(p);   \
             else tiled_kernel_bm64<GSV, false, ZPV, OutF16, true><<<grid, block, 0, stream>>>(p);             \
+        } else if (bm == 128 && split) {                                                                      \
+            if (out_bf16) tiled_kernel<GSV, true, ZPV, OutBF16><<<grid, block, 0, stream>>>(p);               \
+            else tiled_kernel<GSV, true, ZPV, OutF16><<<grid, block, 0, stream>>>(p);                         \
         } else if (bm == 128) {                                                                               \
-            if (out_bf16) tiled_kernel<GSV, ZPV, OutBF16><<<grid, block, 0, stream>>>(p);                     \
-            else tiled_kernel<GSV, ZPV, OutF16><<<grid, block, 0, stream>>>(p);                               \
+            if (out_bf16) tiled_kernel<GSV, false, ZPV, OutBF16><<<grid, block, 0, stream>>>(p);              \
+            else tiled_kernel<GSV, false, ZPV, OutF16><<<grid, block, 0, stream>>>(p);                        \
         } else if (split) {                                                                                   \
             if (out_bf16) tiled_kernel_bm64<GSV, true, ZPV, OutBF16><<<grid, block, 0, stream>>>(p);          \
             else tiled_kernel_bm64<GSV, true, ZPV, OutF16><<<grid, block, 0, stream>>>(p);                    \

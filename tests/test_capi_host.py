@@ -95,7 +95,7 @@ def test_gemm_argument_validation(L):
     assert _gemm(L, kernel=9) == 4
     assert _gemm(L, dump=3) == 4
     assert _gemm(L, dump=1, acc=None) == 1
-    assert _gemm(L, M=64, ldr=64, kernel=_lib.KERNEL_SKINNY) == 7
+    assert _gemm(L, M=300, ldr=300, kernel=_lib.KERNEL_SKINNY) == 7                        # the skinny kernel stops at 256 rows
     assert _gemm(L, M=64, ldr=64, kernel=_lib.KERNEL_TILED, split=2) == 5       # valid, but needs a workspace
     assert _gemm(L, M=64, ldr=64, kernel=_lib.KERNEL_TILED, split=2, dump=2, acc=FAKE) == 5   # the verification instantiation splits alike
     # row sums fold zero-points: the tiled kernel with the uniform zero-point 2 reads none, everything else needs them

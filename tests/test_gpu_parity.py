@@ -95,6 +95,14 @@ def test_act_quant_bit_exact(gpu_ops, oracle, M, K, g, bf16, outliers):
     x[min(1, M - 1), : min(K, 70)] = 0.0
     if M > 2:
         x[2] = 0.0  # an all-zero token
+    if M > 4:
+        # exact and near ties of the rounding: a row whose scale is exactly 1 (absmax 127) holding k + 1/2, and one whose
+        # scale is a hair above 1, so that the same values land just below the tie points
+        ties = (np.arange(K) % 253 - 126).astype(np.float32) + 0.5
+        x[3] = ties.astype(np.float16)
+        x[3, 0] = 127.0
+        x[4] = ties.astype(np.float16)
+        x[4, 0] = 127.0625
     if bf16:
         xt = torch.from_numpy(x.astype(np.float32)).to(torch.bfloat16)
         bits = xt.view(torch.int16).numpy().view(np.uint16)
@@ -175,6 +183,22 @@ def test_skinny_wide_activation_fetch(gpu_ops, oracle, M, N, K, g, mode, out, sp
     case = pu.small_case(M, N, K, g, mode, seed=M + K, out_dtype=out)
     _run_case(gpu_ops, oracle, case, "skinny", split_k=split)
     _run_case(gpu_ops, oracle, case, "skinny", split_k=0, dump="sum")
+
+
+@pytest.mark.parametrize("M,N,K,g,mode,out,split", [
+    (33, 4096, 4096, 128, "sym", "float16", 0),     # the library's own choice for these rows and sizes
+    (77, 200, 512, 128, "asym", "float16", 1),      # five row blocks: two passes of two and one of one
+    (100, 130, 2048, 64, "sym", "bfloat16", 1),
+    (256, 64, 1024, 256, "ref", "float16", 1),
+    (64, 192, 4096, 128, "asym", "bfloat16", 1),    # eight waves per workgroup
+    (48, 128, 14336, 128, "sym", "float16", 4),     # K split across workgroups: sixteen-wave workgroups, one row block per wave
+])
+def test_skinny_more_than_32_rows(gpu_ops, oracle, M, N, K, g, mode, out, split):
+    """33..256 token rows through the weight-streaming kernel (two blocks of 16 rows per wave and pass over the
+    weights): int32 sums exact, the output criterion, verification and production instantiation bit-identical."""
+    case = pu.small_case(M, N, K, g, mode, seed=M + N + K, out_dtype=out)
+    _run_case(gpu_ops, oracle, case, "skinny", split_k=split)
+    _run_case(gpu_ops, oracle, case, "auto", split_k=0, dump="sum")
 
 
 @pytest.mark.parametrize("M,N,K,g,mode,out,split", [
