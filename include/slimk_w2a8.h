@@ -74,7 +74,7 @@ enum slimk_dtype { SLIMK_F16 = 0, SLIMK_BF16 = 1 };
 enum slimk_kernel {
     SLIMK_KERNEL_AUTO = 0,   /* skinny for M <= 32 and for 33..256 rows on short reductions (K <= 4096) over small and
                                 medium matrices (passes over the weights under 100 MiB in all), tiled otherwise */
-    SLIMK_KERNEL_SKINNY = 1, /* weight-streaming split-K kernel, M <= 256 (16 or 32 rows per pass over the weights) */
+    SLIMK_KERNEL_SKINNY = 1, /* weight-streaming split-K kernel, M <= 256 (16 rows per pass over the weights) */
     SLIMK_KERNEL_TILED = 2   /* LDS-pipelined MFMA tile kernel, any M */
 };
 

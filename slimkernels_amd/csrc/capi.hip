@@ -68,10 +68,11 @@ int strips_of(int N) { return (N + w2a8::kStripN - 1) / w2a8::kStripN; }
 constexpr size_t kCounterBlockBytes = 64 << 10;
 constexpr int kMaxCounters = (int)(kCounterBlockBytes / sizeof(unsigned));
 
-// The skinny kernel takes any number of token rows (16 or 32 at a time, each pass re-reading the weights, from the
-// second on out of L2).  Measured against the tiled kernel on 33..256 rows: it wins while the reduction is short
+// The skinny kernel takes any number of token rows (16 at a time, the passes side by side as workgroups of their
+// own, each re-reading the weights, all but the first out of L2).  Measured against the tiled kernel on 33..256 rows: it wins while the reduction is short
 // (K <= 4096: the tiled kernel's few stages do not amortise its start-up) and the passes over the weights stay under
-// about 100 MiB in all (14336 x 4096: up to 96 rows, 11008 x 4096: up to 160, 4096 x 4096: 15.9 -> 9.6 us at 128 rows).
+// about 100 MiB in all (14336 x 4096: up to 96 rows, 11008 x 4096: up to 160, 4096 x 4096: 15.1 -> 6.3 us at 33 rows, 15.9 -> 9.6 us at 128;
+// two row blocks per wave, which halve the passes, lose at the small sizes and gain under 10 % at the large ones).
 constexpr int kSkinnyMaxRows = 256;
 bool skinny_wins_mid(int M, int N, int K) {
     if (M <= 32 || M > kSkinnyMaxRows || K > 4096) return false;

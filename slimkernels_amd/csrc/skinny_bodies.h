@@ -38,7 +38,7 @@ typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 struct SkinnyMeta {
     uint16_t scale[kDepth][16][4];  // [group in chunk][col][sub-block]
     uint8_t zp[kDepth][16][4];
-    int32_t rowsum[kDepth][32];     // up to two blocks of 16 token rows per wave
+    int32_t rowsum[kDepth][16];
 };
 
 // FUSED: the workgroup quantises the (at most four) token rows itself before it needs them.
@@ -50,22 +50,20 @@ struct FusedRows {
 };
 struct NoFusedRows {};
 
-template <int NWP, bool WIDE, bool FUSED = false, int MB = 1>
+template <int NWP, bool WIDE, bool FUSED = false>
 struct SkinnySmem {
     union {
         SkinnyMeta meta[NWP];
-        float red[NWP][16 * MB][kStripN + 1];
+        float red[NWP][16][kStripN + 1];
     };
     v4u atile[WIDE ? NWP : 1][kDepth][64];  // WIDE: a wave's activation fragments of one chunk, in MFMA operand order
     int last;
     typename std::conditional<FUSED, FusedRows, NoFusedRows>::type fused;
 };
 
-// One wave's share of one strip and MB blocks of 16 token rows.  MB = 1 is the decode form (a problem with 17..32
-// rows is run as two row blocks by two sets of waves: the second read of the weights comes from L2, and the small
-// register footprint of a single block is what lets four waves share a SIMD).  MB = 2 serves 33 token rows and more on
-// matrices small enough that this weight-streaming kernel beats the tiled one: a wave unpacks a weight unit once for
-// two row blocks, which halves the passes over the weights and the vector work beside the matrix core.
+// One wave's share of one strip and one block of 16 token rows (a problem with 17..32 rows is
+// run as two row blocks by two sets of waves: the second read of the weights comes from L2, and
+// the small register footprint of a single block is what lets four waves share a SIMD).
 //   J     live rows per lane of a D fragment: 4 in general, 1 when M == 1 (only row 0 of the 16x16
 //         block is a real token, so three quarters of the drain arithmetic are dropped)
 //   GS    steps per scale group
@@ -87,11 +85,11 @@ struct SkinnySmem {
 // product over the groups (16 tokens x 16 channels x up to 4 groups of a chunk) and goes through
 // one v_mfma_f32_16x16x4_f32 per chunk and sub-block, accumulating straight into the fp32 running
 // sums (same D layout as the int8 MFMA).
-template <int J, int GS, int NWK, int NWP, bool ASYM, bool DUMP, bool NT, bool WIDE, bool FUSED, typename OutT, int MB = 1>
+template <int J, int GS, int NWK, int NWP, bool ASYM, bool DUMP, bool NT, bool WIDE, bool FUSED, typename OutT>
 __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip, const int split, const int mblk,
-                                            const int kwave, const int pwave, SkinnySmem<NWP, WIDE, FUSED, MB>& sm) {
+                                            const int kwave, const int pwave, SkinnySmem<NWP, WIDE, FUSED>& sm) {
     static_assert(!FUSED || (!WIDE && !DUMP && NWK == NWP), "fused activation quantisation: the plain production body");
-    static_assert(MB == 1 || (MB == 2 && !WIDE && !FUSED && J == 4), "two row blocks per wave: the plain body, all rows live");
+    constexpr int MB = 1;
     static_assert(NWK == 1 || NWK == NWP, "K is split over one wave or over the whole workgroup");
     constexpr int kThreads = NWP * 64;
     constexpr int kGroupsPerChunk = kDepth / GS;
@@ -105,14 +103,14 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     SkinnyMeta& meta = sm.meta[pwave];
 
     // this row block's view of the per-token operands
-    const int m0 = mblk * (16 * MB);
-    const int M = min(16 * MB, p.M - m0);
+    const int m0 = mblk * 16;
+    const int M = min(16, p.M - m0);
     const int8_t* const qp = p.q + (size_t)m0 * p.ldq;
     const float* const sap = p.s_a + m0;
     const int32_t* const rsp = p.rowsum + m0;
     const int ldr = p.ldr - m0;
     uint16_t* const out = reinterpret_cast<uint16_t*>(p.out) + (size_t)m0 * p.ldo;
-    const int mblocks = (p.M + 16 * MB - 1) / (16 * MB);
+    const int mblocks = (p.M + 15) >> 4;
     const int tile_id = strip * mblocks + mblk;  // index of this (strip, row block) in the split-K workspace
 
     // token scales for the epilogue, fetched first
@@ -574,11 +572,11 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     if (tid == 0) __hip_atomic_store(p.ws_counter + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int J, int GS, int NW, bool ASYM, bool DUMP, bool NT, bool WIDE, typename OutT, int MB = 1>
+template <int J, int GS, int NW, bool ASYM, bool DUMP, bool NT, bool WIDE, typename OutT>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const GemmParams p) {
-    __shared__ __attribute__((aligned(16))) SkinnySmem<NW, WIDE, false, MB> sm;
+    __shared__ __attribute__((aligned(16))) SkinnySmem<NW, WIDE> sm;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keeps ranges and bases in SGPRs
-    skinny_body<J, GS, NW, NW, ASYM, DUMP, NT, WIDE, false, OutT, MB>(p, blockIdx.x, blockIdx.y, blockIdx.z, wave, wave, sm);
+    skinny_body<J, GS, NW, NW, ASYM, DUMP, NT, WIDE, false, OutT>(p, blockIdx.x, blockIdx.y, blockIdx.z, wave, wave, sm);
 }
 
 // The same with the activation quantisation inside (at most four token rows, given as fp16 / bf16).
@@ -1049,19 +1047,19 @@ static hipError_t launch_skinny_shared_impl(const GemmParams& p, int gs, bool as
     return hipGetLastError();
 }
 
-template <int J, int GS, int NW, bool ASYM, bool DUMP, bool NT, bool WIDE, int MB = 1>
+template <int J, int GS, int NW, bool ASYM, bool DUMP, bool NT, bool WIDE>
 static void launch_out(const GemmParams& p, bool out_bf16, hipStream_t stream) {
-    const dim3 grid(p.strips, p.split, (p.M + 16 * MB - 1) / (16 * MB)), block(NW * 64);
+    const dim3 grid(p.strips, p.split, (p.M + 15) / 16), block(NW * 64);
     if (out_bf16)
-        skinny_kernel<J, GS, NW, ASYM, DUMP, NT, WIDE, OutBF16, MB><<<grid, block, 0, stream>>>(p);
+        skinny_kernel<J, GS, NW, ASYM, DUMP, NT, WIDE, OutBF16><<<grid, block, 0, stream>>>(p);
     else
-        skinny_kernel<J, GS, NW, ASYM, DUMP, NT, WIDE, OutF16, MB><<<grid, block, 0, stream>>>(p);
+        skinny_kernel<J, GS, NW, ASYM, DUMP, NT, WIDE, OutF16><<<grid, block, 0, stream>>>(p);
 }
 
-template <int J, int GS, int NW, bool DUMP, bool NT, bool WIDE, int MB = 1>
+template <int J, int GS, int NW, bool DUMP, bool NT, bool WIDE>
 static void launch_zm(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
-    if (asym) launch_out<J, GS, NW, true, DUMP, NT, WIDE, MB>(p, out_bf16, stream);
-    else launch_out<J, GS, NW, false, DUMP, NT, WIDE, MB>(p, out_bf16, stream);
+    if (asym) launch_out<J, GS, NW, true, DUMP, NT, WIDE>(p, out_bf16, stream);
+    else launch_out<J, GS, NW, false, DUMP, NT, WIDE>(p, out_bf16, stream);
 }
 
 // Two-steps-wide activation fetch pays from 16 token rows on when the reduction is long (measured:
@@ -1072,9 +1070,6 @@ constexpr int kWideRows = 16, kWideK = 8192;
 template <int GS, int NW, bool DUMP>
 static void launch_rows(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
     const bool wide = p.M >= kWideRows && p.K >= kWideK;
-    // more than 32 token rows (short reductions on small and medium matrices, where this kernel beats the tiled one):
-    // two row blocks per wave; sixteen-wave workgroups keep one (their LDS meeting area has no room for two)
-    if (p.M > 32 && NW <= 8) { launch_zm<4, GS, NW, DUMP, false, false, 2>(p, asym, out_bf16, stream); return; }
     if (p.M == 1) launch_zm<1, GS, NW, DUMP, true, false>(p, asym, out_bf16, stream);
     else if (p.M <= 16 && !wide) launch_zm<4, GS, NW, DUMP, true, false>(p, asym, out_bf16, stream);
     else if (p.M <= 16) launch_zm<4, GS, NW, DUMP, true, true>(p, asym, out_bf16, stream);

@@ -187,15 +187,16 @@ def test_skinny_wide_activation_fetch(gpu_ops, oracle, M, N, K, g, mode, out, sp
 
 @pytest.mark.parametrize("M,N,K,g,mode,out,split", [
     (33, 4096, 4096, 128, "sym", "float16", 0),     # the library's own choice for these rows and sizes
-    (77, 200, 512, 128, "asym", "float16", 1),      # five row blocks: two passes of two and one of one
+    (77, 200, 512, 128, "asym", "float16", 1),      # five row blocks, the last ragged
     (100, 130, 2048, 64, "sym", "bfloat16", 1),
     (256, 64, 1024, 256, "ref", "float16", 1),
     (64, 192, 4096, 128, "asym", "bfloat16", 1),    # eight waves per workgroup
-    (48, 128, 14336, 128, "sym", "float16", 4),     # K split across workgroups: sixteen-wave workgroups, one row block per wave
+    (48, 128, 14336, 128, "sym", "float16", 4),     # K split across workgroups: sixteen-wave workgroups
 ])
 def test_skinny_more_than_32_rows(gpu_ops, oracle, M, N, K, g, mode, out, split):
-    """33..256 token rows through the weight-streaming kernel (two blocks of 16 rows per wave and pass over the
-    weights): int32 sums exact, the output criterion, verification and production instantiation bit-identical."""
+    """33..256 token rows through the weight-streaming kernel (16 rows per workgroup and pass over the weights, the
+    passes side by side): int32 sums exact, the output criterion, verification and production instantiation
+    bit-identical."""
     case = pu.small_case(M, N, K, g, mode, seed=M + N + K, out_dtype=out)
     _run_case(gpu_ops, oracle, case, "skinny", split_k=split)
     _run_case(gpu_ops, oracle, case, "auto", split_k=0, dump="sum")
