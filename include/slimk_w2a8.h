@@ -199,10 +199,10 @@ int slimk_w2a8_act_quant_rep(const void* x, int ldx, int x_dtype, int M, int K, 
  *                              tile shape, split and wave count; the accumulators are written out as the
  *                              matrix core left them, before their conversion to fp32), so the production
  *                              instantiations carry no extra code and the two calls' outputs are
- *                              bit-identical.  Only shapes the fast tiled kernel does not take (group
- *                              256, K % 128 == 64) run the generic tiled kernel with or without a dump.
- *   rowsum                   : may be NULL for the tiled kernel with zp_r NULL, zp_const 2, group 64 / 128
- *                              and K % 128 == 0 (it is not read there)
+ *                              bit-identical.  The fast tiled kernel takes every supported group size and K
+ *                              (a group of 256 on 64-row tiles only).
+ *   rowsum                   : may be NULL for the tiled kernel with zp_r NULL and zp_const 2 (it is not
+ *                              read there)
  *   workspace                : required when the effective split_k > 1
  *                              (slimk_w2a8_gemm_workspace_bytes), else may be NULL
  *   kernel, split_k          : SLIMK_KERNEL_* and the split-K factor; 0 = choose.  split_k is an upper

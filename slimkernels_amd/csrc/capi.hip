@@ -127,9 +127,9 @@ int skinny_shared_split(int M, int N, int K, int group_size) {
 // 11.6 us at split 4).
 int auto_split(int M, int N, int K, int group_size, int kernel) {
     if (kernel != SLIMK_KERNEL_SKINNY) {
-        // the fast tiled kernel splits K when its tiles would leave CUs idle (group 64 / 128 only)
-        if (group_size > 128) return 1;
-        return w2a8::tiled_fast_auto_split(M, strips_of(N), K / w2a8::kStepK);
+        // the fast tiled kernel splits K when its tiles would leave CUs idle (groups of up to 256)
+        if (group_size > 256) return 1;
+        return w2a8::tiled_fast_auto_split(M, strips_of(N), K / w2a8::kStepK, group_size / w2a8::kStepK);
     }
     if (skinny_shared_applies(M, N, K)) return skinny_shared_split(M, N, K, group_size);
     const int strips = strips_of(N);
@@ -191,7 +191,7 @@ size_t slimk_w2a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int 
     if (split_k <= 1) return 0;
     const int strips = strips_of(N);
     if (kern != SLIMK_KERNEL_SKINNY) {  // one arrival counter and `split_k` fp32 tiles of 64 x 256 per 64-row tile
-        const size_t tiles = w2a8::tiled_fast_workspace_tiles(M, strips);
+        const size_t tiles = w2a8::tiled_fast_workspace_tiles(M, strips, group_size / w2a8::kStepK);
         return kCounterBlockBytes + (size_t)split_k * tiles * 64 * 256 * sizeof(float);
     }
     const int mblocks = (M + 15) / 16;  // one tile and one arrival counter per (strip, block of 16 rows)
@@ -298,9 +298,9 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
     if (int rc = check_kg(K, group_size)) return rc;
     // the row sums fold zero-points; the fast tiled kernel centres its operand bytes on 2 and reads none for that value
     const bool rowsum_unused = !zp_r && zp_const == 2 && resolve_kernel(M, N, K, kernel) == SLIMK_KERNEL_TILED &&
-                               group_size <= 128 && K % 128 == 0;
+                               group_size <= 256;
     if (!rowsum && !rowsum_unused)
-        return fail(SLIMK_ERR_NULL_POINTER, "gemm: rowsum is NULL (only the tiled kernel with the uniform zero-point 2, group 64 / 128 and K %% 128 == 0 does without)");
+        return fail(SLIMK_ERR_NULL_POINTER, "gemm: rowsum is NULL (only the tiled kernel with the uniform zero-point 2 and a group size of at most 256 does without)");
     if (!rowsum) ldr = (M + 3) / 4 * 4;
     if (out_dtype != SLIMK_F16 && out_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "out_dtype=%d", out_dtype);
     if (kernel < SLIMK_KERNEL_AUTO || kernel > SLIMK_KERNEL_TILED) return fail(SLIMK_ERR_BAD_ENUM, "kernel=%d", kernel);
@@ -327,22 +327,23 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
     if (split_k > G) return fail(SLIMK_ERR_BAD_SHAPE, "split_k=%d exceeds the number of groups %d", split_k, G);
     int gps;
     if (kern == SLIMK_KERNEL_TILED) {
-        // only the fast kernel (uniform zero-point 2, no dump, group 64 / 128) with 64-row tiles splits K
+        // only the fast kernel (groups of up to 256) splits K
         w2a8::GemmParams probe{};
         probe.acc_dump = dump_mode != SLIMK_DUMP_NONE ? acc_dump : nullptr; probe.dump_mode = dump_mode;
         probe.zp_const = zp_const; probe.steps = K / w2a8::kStepK;
-        const bool can = w2a8::tiled_fast_supported(probe, group_size / w2a8::kStepK, zp_r != nullptr) &&
-                         w2a8::tiled_fast_max_split(M, strips_of(N), K / w2a8::kStepK) > 1 &&
-                         (size_t)split_k * w2a8::tiled_fast_workspace_tiles(M, strips_of(N)) * 64 * 256 * 4 < 0x7fffffffu;
+        const int gs_t = group_size / w2a8::kStepK;
+        const bool can = w2a8::tiled_fast_supported(probe, gs_t, zp_r != nullptr) &&
+                         w2a8::tiled_fast_max_split(M, strips_of(N), K / w2a8::kStepK, gs_t) > 1 &&
+                         (size_t)split_k * w2a8::tiled_fast_workspace_tiles(M, strips_of(N), gs_t) * 64 * 256 * 4 < 0x7fffffffu;
         if (split_k > 1 && !can) {
             if (!split_chosen_here)
                 return fail(SLIMK_ERR_UNSUPPORTED, "this tiled GEMM cannot split K (split_k=%d)", split_k);
             split_k = 1;
         }
-        const int stages = K / (2 * w2a8::kStepK);
-        const int sps = split_k > 1 ? (stages + split_k - 1) / split_k : stages;
-        if (split_k > 1) split_k = (stages + sps - 1) / sps;  // effective split: whole 128-element stages per split
-        gps = split_k > 1 ? sps * (128 / group_size) : G;
+        gps = G;
+        if (split_k > 1)  // effective split: whole 128-element stages (256 with that group size) per split
+            split_k = w2a8::tiled_fast_effective_split(K / w2a8::kStepK, gs_t, split_k, &gps);
+        if (split_k <= 1) gps = G;
     } else {
         gps = groups_per_split(G, group_size, split_k);
         split_k = (G + gps - 1) / gps;  // effective split: the request is an upper bound (whole chunks per split)
@@ -364,7 +365,7 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
         if (!aligned16(workspace)) return fail(SLIMK_ERR_MISALIGNED, "workspace must be 16-byte aligned");
         p.ws_counter = reinterpret_cast<unsigned*>(workspace);
         const int counters = kern == SLIMK_KERNEL_SKINNY ? p.strips * ((M + 15) / 16)
-                                                         : (int)w2a8::tiled_fast_workspace_tiles(M, p.strips);
+                                                         : (int)w2a8::tiled_fast_workspace_tiles(M, p.strips, group_size / w2a8::kStepK);
         if (counters > kMaxCounters)
             return fail(SLIMK_ERR_UNSUPPORTED, "split_k over %d output tiles (at most %d arrival counters)", counters, kMaxCounters);
         p.ws_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBlockBytes);

@@ -49,15 +49,27 @@ hipError_t launch_skinny_verify(const GemmParams& p, int gs, int waves, bool asy
 hipError_t launch_skinny_shared_verify(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
 hipError_t launch_skinny_grouped_verify(const GroupedParams& gp, int gs, bool asym, bool out_bf16, hipStream_t stream);
 
-// launch_tiled picks the fast kernel when it applies (group 64/128, K % 128 == 0; with p.acc_dump its verification
-// instantiation) and the generic one otherwise.
+// 4-bit weights as two planes (w_r over 2 * p.steps steps, s_r over 2 * p.G groups), uniform zero-point 8, one pass
+// over K: p.K / p.steps / p.G describe K, not 2K; gs 1 or 2; p.steps even
+// p.split > 1: K split over blockIdx.y in whole 128-element stages (p.groups_per_split), workspace = one arrival
+// counter and p.split fp32 tiles of 64 x 256 per tile (tiled_w4_tiles)
+hipError_t launch_tiled_w4(const GemmParams& p, int gs, bool out_bf16, hipStream_t stream);
+hipError_t launch_tiled_w4_verify(const GemmParams& p, int gs, bool out_bf16, hipStream_t stream);
+size_t tiled_w4_tiles(int M, int strips);
+int tiled_w4_auto_split(int M, int strips, int steps);
+
+// The tiled kernel (group 64 / 128 / 256); with p.acc_dump launch_tiled hands over to the verification
+// instantiations (launch_tiled_verify, a translation unit of their own).
 hipError_t launch_tiled(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
-// Split-K of the fast tiled kernel (64-row tiles only): the factor it would choose, the largest it
-// accepts, and the number of tiles a split workspace must hold (64 x 256 fp32 each, per split).
+hipError_t launch_tiled_verify(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
+// Split-K of the fast tiled kernel (gs = 64-element steps per group): the factor it would choose, the largest it
+// accepts, what a requested factor comes to (whole stages per split; *groups_per_split = a split's length in groups),
+// and the number of tiles a split workspace must hold (64 x 256 fp32 each, per split).
 bool tiled_fast_supported(const GemmParams& p, int gs, bool asym);
-int tiled_fast_auto_split(int M, int strips, int steps);
-int tiled_fast_max_split(int M, int strips, int steps);
-size_t tiled_fast_workspace_tiles(int M, int strips);
+int tiled_fast_auto_split(int M, int strips, int steps, int gs);
+int tiled_fast_max_split(int M, int strips, int steps, int gs);
+int tiled_fast_effective_split(int steps, int gs, int split, int* groups_per_split);
+size_t tiled_fast_workspace_tiles(int M, int strips, int gs);
 // Weight-only form (fp16 activations on the fp16 matrix cores, gemm_w2a16.hip).
 struct W2A16Params {
     const uint16_t* x;      // [M][ldx] fp16 bits
@@ -74,14 +86,5 @@ struct W2A16Params {
 };
 int w2a16_auto_split(int M, int strips, int steps, int gs);
 hipError_t launch_w2a16(const W2A16Params& p, int gs, bool out_bf16, hipStream_t stream);
-
-// 4-bit weights as two planes (w_r over 2 * p.steps steps, s_r over 2 * p.G groups), uniform zero-point 8, one pass
-// over K: p.K / p.steps / p.G describe K, not 2K; gs 1 or 2; p.steps even
-// p.split > 1: K split over blockIdx.y in whole 128-element stages (p.groups_per_split), workspace = one arrival
-// counter and p.split fp32 tiles of 64 x 256 per tile (tiled_w4_tiles)
-hipError_t launch_tiled_w4(const GemmParams& p, int gs, bool out_bf16, hipStream_t stream);
-size_t tiled_w4_tiles(int M, int strips);
-int tiled_w4_auto_split(int M, int strips, int steps);
-hipError_t launch_tiled_generic(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
 
 }  // namespace w2a8

@@ -101,7 +101,7 @@ def test_gemm_argument_validation(L):
     # row sums fold zero-points: the tiled kernel with the uniform zero-point 2 reads none, everything else needs them
     assert _gemm(L, rowsum=None) == 1 and b"rowsum" in L.slimk_w2a8_last_error()
     assert _gemm(L, M=64, rowsum=None, kernel=_lib.KERNEL_TILED, zp_const=1) == 1
-    assert _gemm(L, M=64, rowsum=None, kernel=_lib.KERNEL_TILED, g=256) == 1
+    assert _gemm(L, M=64, rowsum=None, kernel=_lib.KERNEL_TILED, g=256, split=2) == 5         # any group size: accepted up to the workspace check
     assert _gemm(L, M=64, rowsum=None, kernel=_lib.KERNEL_TILED, split=2) == 5                # accepted up to the workspace check
     # split-K without / with too small a workspace (N = 4096, K = 14336 wants split 4)
     assert _gemm(L, K=14336, ldq=14336) == 5 and b"workspace" in L.slimk_w2a8_last_error()

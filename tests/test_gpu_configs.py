@@ -103,6 +103,11 @@ def test_config_c4_large(gpu_ops, oracle, N, K, M):
     (2100, 8192, 1024, 128, "asym", "float16"),
     # the upstream quantizer's uniform zero-point 1
     (4096, 4096, 256, 128, "ref", "float16"),
+    # groups of 256 (64-row tiles, a group spans two stages), with and without the zero-point prologue
+    (4100, 4096, 512, 256, "sym", "float16"),
+    (2100, 4100, 1024, 256, "asym", "bfloat16"),
+    # an odd number of 64-element steps at group 64: the last stage is half past the end of K
+    (4100, 4096, 320, 64, "sym", "bfloat16"),
 ])
 def test_tiled_kernel_chip_filling_shapes(gpu_ops, oracle, M, N, K, g, mode, out):
     """Problems of at least two 128 x 256 tiles per CU (the 128-row tiles of the fast tiled kernel) away from the

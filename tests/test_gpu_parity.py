@@ -219,13 +219,20 @@ def test_skinny_shared_one_problem(gpu_ops, oracle, M, N, K, g, mode, out, split
     (77, 200, 512, 128, "asym", "float16"),
     (129, 130, 320, 64, "sym", "float16"),
     (300, 64, 256, 128, "sym", "bfloat16"),
+    # groups of 256: a group spans two stages of the tiled kernel and its int32 sums stay in registers between them
+    (70, 130, 2560, 256, "sym", "float16"),
+    (100, 300, 1024, 256, "asym", "bfloat16"),
+    (64, 256, 256, 256, "ref", "float16"),
+    # an odd number of 64-element steps: the last stage's second step lies past the end of K
+    (200, 256, 64, 64, "sym", "float16"),
+    (77, 100, 448, 64, "asym", "float16"),
 ])
 def test_tiled_small(gpu_ops, oracle, M, N, K, g, mode, out):
     case = pu.small_case(M, N, K, g, mode, seed=M + N + 1, out_dtype=out)
     # unsplit and with the zero-point the operand bytes are centred on (the symmetric levels), the tiled
     # kernels sum the groups in the oracle's order: bit-identical outputs.  Other zero-points add their
     # term through fp32 MFMAs first: the output criterion.
-    exact = mode == "sym" and g <= 128 and K % 128 == 0   # (other shapes run the generic kernel: the output criterion)
+    exact = mode == "sym"
     _run_case(gpu_ops, oracle, case, "tiled", split_k=1, dump="groups", exact_out=exact)
     _run_case(gpu_ops, oracle, case, "tiled", split_k=1, dump="sum", exact_out=exact)
     # whatever split the library picks by itself (K may be split when tiles are few): the output criterion
@@ -259,7 +266,9 @@ def test_tiled_output_views(gpu_ops, oracle, M, N, K, g, out):
 
 
 @pytest.mark.parametrize("M,N,K,g,out,split", [(64, 256, 2048, 128, "float16", 2), (77, 300, 4096, 64, "bfloat16", 4),
-                                                 (130, 64, 3072, 128, "float16", 3), (40, 512, 8192, 128, "float16", 8)])
+                                                 (130, 64, 3072, 128, "float16", 3), (40, 512, 8192, 128, "float16", 8),
+                                                 (64, 256, 4096, 256, "float16", 3), (77, 300, 4160, 64, "bfloat16", 4),
+                                                 (50, 128, 2816, 256, "bfloat16", 11)])
 def test_tiled_split_k(gpu_ops, oracle, M, N, K, g, out, split):
     """Split-K of the fast tiled kernel: the output criterion, and run-to-run identical bits."""
     case = pu.small_case(M, N, K, g, "sym", seed=M + K, out_dtype=out)
