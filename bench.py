@@ -360,21 +360,24 @@ def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, d
         aq.append({"M": M, "K": K, "us": round(us, 2), "GBps": round((3 * M * K + 4 * M + 4 * M * (K // 128)) / (us * 1e-6) / 1e9, 1)})
     detail["act_quant"] = aq
 
-    # ---- one decode row end to end: act-quant + GEMM as two launches against the single launch with the
-    # quantisation inside the GEMM (fp16 activation row in, fp16 out), cold weights
+    # ---- decode rows end to end (fp16 activation rows in, fp16 out, cold weights): act-quant + GEMM as two launches
+    # against the single launch with the quantisation inside the GEMM, where that launch takes the shape
     fused = []
     for c in cases:
-        if c.M != 1:
+        if c.M not in (1, 2, 4, 16, 32):
             continue
         sh = shapes[name_of[(c.N, c.K)]]
-        x, _, out = acts[(c.N, c.K, 1)]
-        for w in sh.copies:
-            ops.w2a8_linear_fused(x, w, torch.float16, out=out)
+        x, _, out = acts[(c.N, c.K, c.M)]
         two = time_graph(torch, lambda: [ops.w2a8_gemm(ops.quantize_act_int8(x, 128), w, torch.float16, out=out) for w in sh.copies],
                          len(sh.copies), replays=3)
-        one = time_graph(torch, lambda: [ops.w2a8_linear_fused(x, w, torch.float16, out=out) for w in sh.copies],
-                         len(sh.copies), replays=3)
-        fused.append({"shape": f"{c.N}x{c.K}", "M": 1, "act_quant_then_gemm_us": round(two, 2), "fused_us": round(one, 2)})
+        row = {"shape": f"{c.N}x{c.K}", "M": c.M, "act_quant_then_gemm_us": round(two, 2), "fused_us": None}
+        if ops.fused_applies(c.M, c.K):
+            for w in sh.copies:
+                ops.w2a8_linear_fused(x, w, torch.float16, out=out)
+            one = time_graph(torch, lambda: [ops.w2a8_linear_fused(x, w, torch.float16, out=out) for w in sh.copies],
+                             len(sh.copies), replays=3)
+            row["fused_us"] = round(one, 2)
+        fused.append(row)
     detail["decode_row_end_to_end"] = fused
 
     # ---- prefill regime (c3): tiled int8-MFMA kernel
