@@ -239,19 +239,31 @@ int slimk_w2a8_gemm_static(const int8_t* q, int ldq, const float* s_a, const int
                            void* out, int ldo, int out_dtype,
                            int kernel, int split_k, void* stream);
 
-/* The GEMM for at most four token rows with the activation quantisation inside: x [M][ldx] fp16 or
- * bf16 (x_dtype) takes the place of q, s_a and rowsum, and every workgroup quantises the rows itself
- * (same numbers as slimk_w2a8_act_quant) while its first weights are on the way - one launch
- * instead of two on the latency-bound decode path.  M <= 4 and M * K <= 32768, else
- * SLIMK_ERR_UNSUPPORTED.  The result is bit-identical with slimk_w2a8_act_quant followed by
- * slimk_w2a8_gemm (skinny kernel, same split_k).  Workspace and split_k as for slimk_w2a8_gemm
- * with SLIMK_KERNEL_SKINNY.  x 16-byte aligned, ldx % 8 == 0.
- * No upstream counterpart (upstream feeds already quantised FP8, wgmma_sm90_W2A8.cu:533-536). */
+/* The GEMM for up to 32 token rows with the activation quantisation inside: x [M][ldx] fp16 or bf16 (x_dtype)
+ * takes the place of q, s_a and rowsum - one launch instead of two on the latency-bound decode path, the numbers of
+ * slimk_w2a8_act_quant, the result bit-identical with slimk_w2a8_act_quant followed by slimk_w2a8_gemm (skinny
+ * kernel, one strip per workgroup, same split_k).  Two forms, chosen by shape:
+ *  - M <= 4 and M * K <= 32768: every workgroup quantises the rows itself into LDS while its first weights are on
+ *    the way.  Workspace and split_k as for slimk_w2a8_gemm with SLIMK_KERNEL_SKINNY (none unless K is split).
+ *  - otherwise (M <= 32): the first M workgroups of the grid quantise one row each into the workspace and raise a
+ *    counter there; every workgroup starts its weight stream and then waits for the rows (a bounded wait: a workgroup
+ *    that does not see them arrive in time quantises them itself, so the kernel ends whatever happens).  This form
+ *    ALWAYS needs a workspace of slimk_w2a8_gemm_fused_workspace_bytes(...) bytes, zeroed once with
+ *    slimk_w2a8_workspace_init (the kernel leaves its counters at zero; calls that share a workspace must not overlap
+ *    in time).  A workspace of that size also serves slimk_w2a8_gemm calls of the same shape.
+ * M > 32: SLIMK_ERR_UNSUPPORTED.  x 16-byte aligned, ldx % 8 == 0.
+ * No upstream counterpart (upstream feeds already quantised FP8, wgmma_sm90_W2A8.cu:533-536; the model-level caller
+ * is llama.py:15-19). */
+size_t slimk_w2a8_gemm_fused_workspace_bytes(int M, int N, int K, int group_size, int split_k);
 int slimk_w2a8_gemm_fused(const void* x, int ldx, int x_dtype,
                           const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
                           int M, int N, int K, int group_size,
                           void* out, int ldo, int out_dtype,
                           void* workspace, size_t workspace_bytes, int split_k, void* stream);
+/* Test hook, no upstream counterpart: the number of polls (about a microsecond each) the second form above waits for
+ * the rows before a workgroup quantises them itself; returns the previous value (default 20000).  0 makes every
+ * workgroup take that road, which is how the tests reach it; results do not depend on the value. */
+int slimk_w2a8_set_fused_spin_limit(int polls);
 
 /* One problem of a grouped launch: the arguments of slimk_w2a8_gemm that describe data. */
 typedef struct slimk_w2a8_problem {

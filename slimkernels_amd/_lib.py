@@ -38,6 +38,8 @@ SIGNATURES = {
     "slimk_w2a8_static_workspace_bytes": (_sz, []),
     "slimk_w2a8_gemm_static": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _vp]),
     "slimk_w2a8_gemm_fused": (_i, [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _i, _vp, _sz, _i, _vp]),
+    "slimk_w2a8_gemm_fused_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "slimk_w2a8_set_fused_spin_limit": (_i, [_i]),
     "slimk_w2a8_gemm_grouped": (_i, [_vp, _i, _i, _i, _vp]),
     "slimk_w2a8_gemm_grouped_verify": (_i, [_vp, _i, _i, _i, _vp, _i, _vp]),
     "slimk_w4a8_gemm_auto_split_k": (_i, [_i, _i, _i, _i]),

@@ -4,6 +4,8 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include <atomic>
+
 #include <mutex>
 #include <string>
 
@@ -65,8 +67,8 @@ int strips_of(int N) { return (N + w2a8::kStripN - 1) / w2a8::kStripN; }
 // fp32 partial tiles.  Every kernel leaves the counters it used at zero, and because the block does not move
 // with the shape, a workspace zeroed once stays valid for any sequence of problems (a counter block sized by the
 // problem would let a later, larger block overlap an earlier call's partial sums).
-constexpr size_t kCounterBlockBytes = 64 << 10;
-constexpr int kMaxCounters = (int)(kCounterBlockBytes / sizeof(unsigned));
+constexpr size_t kCounterBlockBytes = w2a8::kCounterBlockBytes;
+constexpr int kMaxCounters = w2a8::kMaxSplitCounters;  // (the block's last two slots belong to the row-quantising kernels)
 
 // The skinny kernel takes any number of token rows (16 at a time, the passes side by side as workgroups of their
 // own, each re-reading the weights, all but the first out of L2).  Measured against the tiled kernel on 33..256 rows: it wins while the reduction is short
@@ -125,6 +127,7 @@ int skinny_shared_split(int M, int N, int K, int group_size) {
 // 256 workgroups, because a quarter of the CUs cannot pull full HBM bandwidth - and never beyond:
 // with more workgroups than CUs some CUs carry two (5120 x 13824, 80 strips: 8.2 us at split 3,
 // 11.6 us at split 4).
+int skinny_plain_split(int N, int K, int group_size);
 int auto_split(int M, int N, int K, int group_size, int kernel) {
     if (kernel != SLIMK_KERNEL_SKINNY) {
         // the fast tiled kernel splits K when its tiles would leave CUs idle (groups of up to 256)
@@ -132,6 +135,10 @@ int auto_split(int M, int N, int K, int group_size, int kernel) {
         return w2a8::tiled_fast_auto_split(M, strips_of(N), K / w2a8::kStepK, group_size / w2a8::kStepK);
     }
     if (skinny_shared_applies(M, N, K)) return skinny_shared_split(M, N, K, group_size);
+    return skinny_plain_split(N, K, group_size);
+}
+
+int skinny_plain_split(int N, int K, int group_size) {
     const int strips = strips_of(N);
     const int G = K / group_size;
     const int chunks = (K / 64 + 3) / 4;
@@ -150,6 +157,16 @@ int auto_split(int M, int N, int K, int group_size, int kernel) {
 // up to 16 MiB with at most four token rows is bound by latency: eight waves per strip instead of
 // four shorten each wave's run (measured 5.09 -> 4.72 us at 4096 x 4096, M = 1; larger matrices
 // and more rows lose).
+// slimk_w2a8_gemm_fused: up to four rows of at most 32 KiB of int8 values together are quantised by every workgroup for
+// itself into LDS; more rows (up to 32) or longer ones by the grid's first workgroups into the workspace.
+bool fused_in_workgroup(int M, int K) { return M <= w2a8::kFusedMaxRows && (size_t)M * K <= (size_t)w2a8::kFusedMaxBytes; }
+size_t fused_rows_q_bytes(int K) { return ((size_t)w2a8::kRowsMax * K + 255) / 256 * 256; }
+size_t fused_rows_area_bytes(int K, int G) {  // int8 rows, 32 token scales, group sums [G][32]
+    return fused_rows_q_bytes(K) + 256 + ((size_t)G * w2a8::kRowsMax * 4 + 255) / 256 * 256;
+}
+// polls of the row-quantising kernels' wait before a workgroup quantises the rows itself (a poll is about a microsecond)
+std::atomic<int> g_rows_spin_limit{20000};
+
 int skinny_waves(int M, int N, int K, int split) {
     if (split > 1) return 16;
     const size_t weight_bytes = (size_t)strips_of(N) * 64 * (K / 4);
@@ -466,15 +483,14 @@ int slimk_w2a8_gemm_fused(const void* x, int ldx, int x_dtype,
     if (out_dtype != SLIMK_F16 && out_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "out_dtype=%d", out_dtype);
     if (zp_const < 0 || zp_const > 3) return fail(SLIMK_ERR_BAD_SHAPE, "zp_const=%d must be 0..3", zp_const);
     if (ldx < K || ldo < N) return fail(SLIMK_ERR_BAD_SHAPE, "ldx=%d / ldo=%d too small for K=%d / N=%d", ldx, ldo, K, N);
-    if (M > w2a8::kFusedMaxRows || (size_t)M * K > (size_t)w2a8::kFusedMaxBytes)
-        return fail(SLIMK_ERR_UNSUPPORTED, "gemm_fused handles M <= %d with M * K <= %d (M=%d, K=%d)", w2a8::kFusedMaxRows,
-                    w2a8::kFusedMaxBytes, M, K);
+    if (M > w2a8::kRowsMax) return fail(SLIMK_ERR_UNSUPPORTED, "gemm_fused handles M <= %d (M=%d)", w2a8::kRowsMax, M);
     if (int rc = check_extent(M, N, K, K)) return rc;
     if (!aligned16(x) || ldx % 8 != 0 || !aligned16(w_r) || !aligned16(s_r) || (zp_r && !aligned16(zp_r)) ||
         (reinterpret_cast<uintptr_t>(out) & 1u))
         return fail(SLIMK_ERR_MISALIGNED, "gemm_fused: x, w_r, s_r, zp_r must be 16-byte aligned; ldx %% 8 == 0; out 2-byte aligned");
     const int G = K / group_size;
-    if (split_k <= 0) split_k = auto_split(M, N, K, group_size, SLIMK_KERNEL_SKINNY);
+    const bool in_workgroup = fused_in_workgroup(M, K);
+    if (split_k <= 0) split_k = in_workgroup ? auto_split(M, N, K, group_size, SLIMK_KERNEL_SKINNY) : skinny_plain_split(N, K, group_size);
     if (split_k > G) return fail(SLIMK_ERR_BAD_SHAPE, "split_k=%d exceeds the number of groups %d", split_k, G);
     const int gps = groups_per_split(G, group_size, split_k);
     split_k = (G + gps - 1) / gps;
@@ -484,6 +500,28 @@ int slimk_w2a8_gemm_fused(const void* x, int ldx, int x_dtype,
     p.w_r = w_r; p.s_r = s_r; p.zp_r = zp_r; p.out = out; p.ldo = ldo;
     p.M = M; p.N = N; p.K = K; p.G = G; p.steps = K / w2a8::kStepK; p.strips = strips_of(N);
     p.zp_const = zp_const; p.split = split_k; p.groups_per_split = gps;
+    if (!in_workgroup) {
+        // The rows are quantised by the grid's first workgroups into the workspace: counter block, the int8 rows, their
+        // scales and group sums, then the split-K partial tiles.
+        const size_t need = slimk_w2a8_gemm_fused_workspace_bytes(M, N, K, group_size, split_k);
+        if (!workspace) return fail(SLIMK_ERR_WORKSPACE, "gemm_fused with M=%d, K=%d needs a workspace of %zu bytes", M, K, need);
+        if (workspace_bytes < need)
+            return fail(SLIMK_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, need);
+        if (!aligned16(workspace)) return fail(SLIMK_ERR_MISALIGNED, "workspace must be 16-byte aligned");
+        const int counters = p.strips * ((M + 15) / 16);
+        if (split_k > 1 && counters > kMaxCounters)
+            return fail(SLIMK_ERR_UNSUPPORTED, "split_k over %d output tiles (at most %d arrival counters)", counters, kMaxCounters);
+        char* base = reinterpret_cast<char*>(workspace);
+        char* rows = base + kCounterBlockBytes;
+        p.ws_counter = reinterpret_cast<unsigned*>(base);
+        p.q = reinterpret_cast<const int8_t*>(rows); p.ldq = K;
+        p.s_a = reinterpret_cast<const float*>(rows + fused_rows_q_bytes(K));
+        p.rowsum = reinterpret_cast<const int32_t*>(rows + fused_rows_q_bytes(K) + 256); p.ldr = w2a8::kRowsMax;
+        p.ws_partial = reinterpret_cast<float*>(rows + fused_rows_area_bytes(K, G));
+        return hip_result(w2a8::launch_skinny_rows(p, group_size / w2a8::kStepK, skinny_waves(M, N, K, split_k), zp_r != nullptr,
+                                                   out_dtype == SLIMK_BF16, g_rows_spin_limit.load(), (hipStream_t)stream),
+                          "row-quantising skinny gemm");
+    }
     if (split_k > 1) {
         const size_t need = slimk_w2a8_gemm_workspace_bytes(M, N, K, group_size, SLIMK_KERNEL_SKINNY, split_k);
         if (!workspace) return fail(SLIMK_ERR_WORKSPACE, "split_k=%d needs a workspace of %zu bytes", split_k, need);
@@ -498,6 +536,23 @@ int slimk_w2a8_gemm_fused(const void* x, int ldx, int x_dtype,
     return hip_result(w2a8::launch_skinny_fused(p, group_size / w2a8::kStepK, skinny_waves(M, N, K, split_k), zp_r != nullptr,
                                                 out_dtype == SLIMK_BF16, (hipStream_t)stream),
                       "fused skinny gemm");
+}
+
+size_t slimk_w2a8_gemm_fused_workspace_bytes(int M, int N, int K, int group_size, int split_k) {
+    if (M <= 0 || M > w2a8::kRowsMax || N <= 0 || !shape_ok(K, group_size)) return 0;
+    if (fused_in_workgroup(M, K)) return slimk_w2a8_gemm_workspace_bytes(M, N, K, group_size, SLIMK_KERNEL_SKINNY, split_k);
+    const int G = K / group_size;
+    if (split_k <= 0) split_k = skinny_plain_split(N, K, group_size);
+    const int gps = groups_per_split(G, group_size, split_k);
+    split_k = (G + gps - 1) / gps;
+    size_t bytes = kCounterBlockBytes + fused_rows_area_bytes(K, G);
+    if (split_k > 1) bytes += (size_t)split_k * strips_of(N) * ((M + 15) / 16) * 16 * w2a8::kStripN * sizeof(float);
+    return bytes;
+}
+
+int slimk_w2a8_set_fused_spin_limit(int polls) {
+    if (polls < 0) polls = 0;
+    return g_rows_spin_limit.exchange(polls);
 }
 
 }  // extern "C"

@@ -163,12 +163,14 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
 // between the absmax pass and the quantising pass, all of its loads in flight together.  With many rows the
 // two-pass kernel moves every row twice (the second time from L2) in phases that the workgroups of a round
 // go through together; this one moves it once.  Same arithmetic per element: bit-identical results.
-template <bool BF16, int KEEP>
-__global__ __launch_bounds__(256) void act_quant_keep_kernel(const uint16_t* __restrict__ x, int ldx, int K,
+// THREADS: 256 in general (many rows: several workgroups per CU); 1024 for a few long rows, where one row per
+// workgroup leaves most of the chip idle and a row's time is what a thread's chain of loads, divisions and stores takes.
+template <bool BF16, int KEEP, int THREADS = 256>
+__global__ __launch_bounds__(THREADS) void act_quant_keep_kernel(const uint16_t* __restrict__ x, int ldx, int K,
                                                              int group_size, int8_t* __restrict__ q, int ldq,
                                                              float* __restrict__ s_a,
                                                              int32_t* __restrict__ rowsum, int ldr, int copies) {
-    __shared__ float red[4];
+    __shared__ float red[THREADS / 64];
     const int m = blockIdx.x;
     const int tid = threadIdx.x;
     const uint16_t* xr = x + (size_t)m * ldx;
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(256) void act_quant_keep_kernel(const uint16_t* __r
     uint4 raw[KEEP];
 #pragma unroll
     for (int it = 0; it < KEEP; ++it) {
-        const int v = it * 256 + tid;
+        const int v = it * THREADS + tid;
         raw[it] = v < nvec ? *reinterpret_cast<const uint4*>(xr + (size_t)v * 8) : make_uint4(0, 0, 0, 0);
     }
     float amax = 0.0f;
@@ -191,7 +193,9 @@ __global__ __launch_bounds__(256) void act_quant_keep_kernel(const uint16_t* __r
     for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
     if ((tid & 63) == 0) red[tid >> 6] = amax;
     __syncthreads();
-    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    amax = red[0];
+#pragma unroll
+    for (int w = 1; w < THREADS / 64; ++w) amax = fmaxf(amax, red[w]);
     const float s = fmaxf(amax, 1e-9f) / 127.0f;
     if (tid == 0) s_a[m] = s;
 
@@ -199,7 +203,7 @@ __global__ __launch_bounds__(256) void act_quant_keep_kernel(const uint16_t* __r
     int8_t* qr = q + (size_t)m * ldq;
 #pragma unroll
     for (int it = 0; it < KEEP; ++it) {
-        const int v = it * 256 + tid;
+        const int v = it * THREADS + tid;
         int sum = 0;
         if (v < nvec) {
             float f[8];
@@ -223,10 +227,22 @@ __global__ __launch_bounds__(256) void act_quant_keep_kernel(const uint16_t* __r
     }
 }
 
+constexpr int kFewRows = 64;  // up to this many rows a long row gets 1024 threads
+
 template <bool BF16>
 static void launch_act_quant_keep(const void* x, int ldx, int M, int K, int group_size, int8_t* q, int ldq, float* s_a,
                                   int32_t* rowsum, int ldr, int copies, hipStream_t stream) {
     const dim3 grid((unsigned)M), block(256);
+    if (M <= kFewRows && K > 4096) {  // a few long rows: 1024 threads a row
+        const dim3 wide(1024);
+        if (K <= 8192)
+            act_quant_keep_kernel<BF16, 1, 1024><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+        else if (K <= 16384)
+            act_quant_keep_kernel<BF16, 2, 1024><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+        else
+            act_quant_keep_kernel<BF16, 4, 1024><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+        return;
+    }
     if (K <= 4096)
         act_quant_keep_kernel<BF16, 2><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
     else if (K <= 8192)
@@ -237,7 +253,7 @@ static void launch_act_quant_keep(const void* x, int ldx, int M, int K, int grou
 
 hipError_t launch_act_quant(const void* x, int ldx, bool x_bf16, int M, int K, int group_size,
                             int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, int copies, hipStream_t stream) {
-    if (K <= 16384) {
+    if (K <= 16384 || (M <= kFewRows && K <= 32768)) {
         if (x_bf16) launch_act_quant_keep<true>(x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies, stream);
         else launch_act_quant_keep<false>(x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies, stream);
         return hipGetLastError();

@@ -61,6 +61,133 @@ struct SkinnySmem {
     typename std::conditional<FUSED, FusedRows, NoFusedRows>::type fused;
 };
 
+// ---------------------------------------------------------------------------------------------
+// Activation rows quantised inside the GEMM launch by the grid's own first workgroups (skinny_rows_kernel: 5..32 token
+// rows, or fewer rows too long for the in-workgroup form above).  Workgroup i < M of the grid (in dispatch order)
+// quantises row i (and i + the grid's size, ..., should the grid be smaller than M) of the fp16 / bf16 activations p.x into the caller's workspace, where p.q / p.s_a / p.rowsum point
+// -- the numbers of act_quant_kernel: per-token scale absmax / 127, IEEE binary32 division, round-half-even, clip to
+// +-127, the per-group sums of q -- and then raises the first of two counters at the end of the workspace's counter
+// block; every workgroup, the quantising ones included, goes on to its GEMM share, starts its weight stream and only
+// then waits for the counter to reach M.  The second counter counts the workgroups that are past the wait; the last
+// of them puts both back to zero, so the workspace is ready for the next call when the kernel ends.
+template <int THREADS>
+__device__ __forceinline__ void rows_quantise_row(const GemmParams& p, const int m, float* scratch) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint16_t* xr = p.x + (size_t)m * p.ldx;
+    const int nvec = p.K / 8;
+    const bool bf16 = p.x_bf16 != 0;
+    auto load8 = [&](const uint16_t* src, float (&f)[8]) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(src);
+        const uint32_t wds[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (bf16) {
+                f[2 * i] = __uint_as_float(wds[i] << 16);
+                f[2 * i + 1] = __uint_as_float(wds[i] & 0xffff0000u);
+            } else {
+                f[2 * i] = half_bits_to_float((uint16_t)(wds[i] & 0xffffu));
+                f[2 * i + 1] = half_bits_to_float((uint16_t)(wds[i] >> 16));
+            }
+        }
+    };
+    float amax = 0.0f;
+    for (int v = tid; v < nvec; v += THREADS) {
+        float f[8];
+        load8(xr + (size_t)v * 8, f);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(f[i]));
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    if (lane == 0) scratch[wave] = amax;
+    __syncthreads();
+    float a = scratch[0];
+#pragma unroll
+    for (int w = 1; w < THREADS / 64; ++w) a = fmaxf(a, scratch[w]);
+    __syncthreads();  // scratch is free again
+    const float s = fmaxf(a, 1e-9f) / 127.0f;
+    if (tid == 0) const_cast<float*>(p.s_a)[m] = s;
+    int8_t* qr = const_cast<int8_t*>(p.q) + (size_t)m * p.ldq;
+    int32_t* rs = const_cast<int32_t*>(p.rowsum);
+    const int tpg = p.K / p.G / 8;  // threads per scale group (8 elements each): 8, 16 or 32, whole groups per wave
+    for (int v0 = 0; v0 < nvec; v0 += THREADS) {  // (every thread makes every trip: the shuffles need whole waves)
+        const int v = v0 + tid;
+        int sum = 0;
+        if (v < nvec) {
+            float f[8];
+            load8(xr + (size_t)v * 8, f);  // second read of the row: from the cache
+            uint32_t lo = 0, hi = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float r = rintf(f[i] / s);
+                r = fminf(fmaxf(r, -127.0f), 127.0f);
+                const int qi = (int)r;
+                sum += qi;
+                if (i < 4) lo |= (uint32_t)(qi & 0xff) << (8 * i);
+                else hi |= (uint32_t)(qi & 0xff) << (8 * (i - 4));
+            }
+            *reinterpret_cast<uint2*>(qr + (size_t)v * 8) = make_uint2(lo, hi);
+        }
+        for (int off = 1; off < tpg; off <<= 1) sum += __shfl_xor(sum, off, 64);
+        if (v < nvec && v % tpg == 0) rs[(size_t)(v / tpg) * p.ldr + m] = sum;
+    }
+}
+
+template <int THREADS>
+__device__ __forceinline__ void rows_quantise_and_signal(const GemmParams& p, float* scratch) {
+    const int wg = (int)(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z));  // dispatch order
+    if (wg >= p.M) return;  // (the same for the whole workgroup)
+    const int total = (int)(gridDim.x * gridDim.y * gridDim.z);
+    unsigned done = 0;
+    for (int m = wg; m < p.M; m += total, ++done) rows_quantise_row<THREADS>(p, m, scratch);  // (a grid smaller than M: several rows)
+    // Every thread's stores have reached this XCD's L2 (s_waitcnt), then ONE thread writes that L2 back to where the
+    // other XCDs see it and raises the counter: the write-back is an operation on the whole L2 and serialises there,
+    // one per workgroup is what is needed and a fence in every wave is 4..16 times that.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        __hip_atomic_fetch_add(p.ws_counter + kRowFlagSlot, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// The bounded wait for the rows.  flag: one int of LDS.  A workgroup whose polls run out quantises every row itself:
+// the same bytes to the same places as the workgroups it gave up on, so whoever reads them reads the same thing.
+template <int THREADS>
+__device__ __forceinline__ void rows_wait(const GemmParams& p, float* scratch, int* flag, const int spin_limit) {
+    unsigned* const flags = p.ws_counter + kRowFlagSlot;
+    if (threadIdx.x == 0) {
+        int ok = 0;
+        for (int i = 0; i < spin_limit; ++i) {
+            if (__hip_atomic_load(flags, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (unsigned)p.M) {
+                ok = 1;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(2);
+        }
+        *flag = ok;
+        // one invalidate per workgroup (this CU's L1 and the XCD's L2 drop what they hold of memory other XCDs write),
+        // before the barrier that lets the other waves read the rows: an invalidate in every wave serialises on the L2
+        if (ok) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    }
+    __syncthreads();
+    if (*flag == 0) {
+        for (int m = 0; m < p.M; ++m) rows_quantise_row<THREADS>(p, m, scratch);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "agent");
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const unsigned total = gridDim.x * gridDim.y * gridDim.z;
+        const unsigned prev = __hip_atomic_fetch_add(flags + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (prev == total - 1) {  // every workgroup is past its wait: ready for the next call
+            __hip_atomic_store(flags, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(flags + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
 // One wave's share of one strip and one block of 16 token rows (a problem with 17..32 rows is
 // run as two row blocks by two sets of waves: the second read of the weights comes from L2, and
 // the small register footprint of a single block is what lets four waves share a SIMD).
@@ -85,10 +212,12 @@ struct SkinnySmem {
 // product over the groups (16 tokens x 16 channels x up to 4 groups of a chunk) and goes through
 // one v_mfma_f32_16x16x4_f32 per chunk and sub-block, accumulating straight into the fp32 running
 // sums (same D layout as the int8 MFMA).
-template <int J, int GS, int NWK, int NWP, bool ASYM, bool DUMP, bool NT, bool WIDE, bool FUSED, typename OutT>
+template <int J, int GS, int NWK, int NWP, bool ASYM, bool DUMP, bool NT, bool WIDE, bool FUSED, typename OutT, bool ROWS = false>
 __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip, const int split, const int mblk,
-                                            const int kwave, const int pwave, SkinnySmem<NWP, WIDE, FUSED>& sm) {
+                                            const int kwave, const int pwave, SkinnySmem<NWP, WIDE, FUSED>& sm,
+                                            const int spin_limit = 0) {
     static_assert(!FUSED || (!WIDE && !DUMP && NWK == NWP), "fused activation quantisation: the plain production body");
+    static_assert(!ROWS || (!FUSED && !DUMP && NWK == NWP), "rows quantised by the grid's first workgroups: a production body");
     constexpr int MB = 1;
     static_assert(NWK == 1 || NWK == NWP, "K is split over one wave or over the whole workgroup");
     constexpr int kThreads = NWP * 64;
@@ -115,17 +244,18 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
 
     // token scales for the epilogue, fetched first
     float sa[NWK == 1 ? MB * J : kOutPerThread];
-    if (FUSED) {
-        // set once the rows are quantised
-    } else if (NWK == 1) {  // this wave stores D fragments itself: rows mb*16 + quad*4 + j
+    auto load_sa = [&]() {
+        if (NWK == 1) {  // this wave stores D fragments itself: rows mb*16 + quad*4 + j
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
+            for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-            for (int j = 0; j < J; ++j) sa[mb * J + j] = sap[min(mb * 16 + quad * 4 + j, M - 1)];
-    } else {  // element e = tid + kThreads*i of the reduced tile -> row e >> 6
+                for (int j = 0; j < J; ++j) sa[mb * J + j] = sap[min(mb * 16 + quad * 4 + j, M - 1)];
+        } else {  // element e = tid + kThreads*i of the reduced tile -> row e >> 6
 #pragma unroll
-        for (int i = 0; i < kOutPerThread; ++i) sa[i] = sap[min((tid + kThreads * i) >> 6, M - 1)];
-    }
+            for (int i = 0; i < kOutPerThread; ++i) sa[i] = sap[min((tid + kThreads * i) >> 6, M - 1)];
+        }
+    };
+    if (!FUSED && !ROWS) load_sa();  // (FUSED, ROWS: once the rows are quantised)
 
     // Step range of this workgroup (groups_per_split is a multiple of a chunk's groups), then of this
     // wave, in whole chunks of kDepth steps; only a range's last chunk can be ragged.
@@ -177,7 +307,7 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
         }
         if (FUSED) {
             if (rowsum_part) m_rs[0] = (lane & 3) == 0 ? fused_rowsum(gq) : v4i{0, 0, 0, 0};  // rows 0..3 only
-        } else {
+        } else if (rowsum_part) {
             const int32_t* rp = rsp + (size_t)gq * p.ldr;
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
@@ -200,13 +330,16 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     // ---- weight / activation register ring
     v4u wring[kDepth];
     v4u aring[kDepth][MB];
-    auto issue = [&](int slot, int step) {  // step is wave-uniform
-        wring[slot] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane, step * wstride + wbase, NT ? kStreamOnce : 0);
+    auto issue_a = [&](int slot, int step) {
         if (!WIDE && !FUSED) {
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
                 aring[slot][mb] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, aoff[mb], step * kStepK, 0);
         }
+    };
+    auto issue = [&](int slot, int step, bool with_a = true) {  // step is wave-uniform
+        wring[slot] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane, step * wstride + wbase, NT ? kStreamOnce : 0);
+        if (with_a) issue_a(slot, step);
     };
     // WIDE: fragment (pair q, row half h) of a chunk: lane l reads row 8h + l/8, 16-byte piece l%8 of the
     // 128 bytes the pair's two steps cover, and parks it at step 2q + piece/4, lane (piece%4)*16 + row.
@@ -244,12 +377,27 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     if (s0 < s1) {
         // Same issue order as inside the loop (metadata first, then the ring), fenced, so that the
         // wait counts the compiler derives for the loop head hold on the entry path as well.
-        fetch_meta(stepof(0) / GS, true, !FUSED);
+        fetch_meta(stepof(0) / GS, true, !FUSED && !ROWS);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < kDepth; ++i) issue(i, stepof(i));
-        if (WIDE) fetch_wide(0);
+        for (int i = 0; i < kDepth; ++i) issue(i, stepof(i), !ROWS);
+        if (WIDE && !ROWS) fetch_wide(0);
         __builtin_amdgcn_sched_barrier(0);
+    }
+
+    if constexpr (ROWS) {
+        // ---- the token rows are being quantised by the first p.M workgroups of this grid (rows_quantise_and_signal,
+        // called by the kernel before this body): with the first weights on their way, wait until all rows are in
+        // memory, then fetch what depends on them.  The wait is bounded: a workgroup that does not see the rows arrive
+        // within spin_limit polls quantises them itself (same arithmetic, same bytes to the same places), so every wave
+        // reaches the end of the kernel whatever happens to the others.
+        rows_wait<kThreads>(p, &sm.red[0][0][0], &sm.last, spin_limit);
+        load_sa();
+        if (s0 < s1) {
+#pragma unroll
+            for (int i = 0; i < kDepth; ++i) issue_a(i, stepof(i));
+            if (WIDE) fetch_wide(0);
+        }
     }
 
     if constexpr (FUSED) {
@@ -378,7 +526,7 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     }
 
     if (s0 < s1) {
-        if (FUSED) fetch_meta(stepof(0) / GS, false, true);  // the row sums of the first chunk, now that they exist
+        if (FUSED || ROWS) fetch_meta(stepof(0) / GS, false, true);  // the row sums of the first chunk, now that they exist
 
         v4i acc[MB][4];
         v4h sc;          // the group's four sub-block scales, kept in fp16: the drain's fma reads them as such
@@ -585,6 +733,16 @@ __global__ __launch_bounds__(NW * 64) void skinny_fused_kernel(const GemmParams 
     __shared__ __attribute__((aligned(16))) SkinnySmem<NW, false, true> sm;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     skinny_body<J, GS, NW, NW, ASYM, false, true, false, true, OutT>(p, blockIdx.x, blockIdx.y, 0, wave, wave, sm);
+}
+
+// The same with the token rows quantised by the grid's first workgroups (see rows_quantise_row): fp16 / bf16 rows in.
+template <int GS, int NW, bool ASYM, bool NT, bool WIDE, typename OutT>
+__global__ __launch_bounds__(NW * 64) void skinny_rows_kernel(const GemmParams p, const int spin_limit) {
+    __shared__ __attribute__((aligned(16))) SkinnySmem<NW, WIDE> sm;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    rows_quantise_and_signal<NW * 64>(p, &sm.red[0][0][0]);
+    skinny_body<4, GS, NW, NW, ASYM, false, NT, WIDE, false, OutT, true>(p, blockIdx.x, blockIdx.y, blockIdx.z, wave, wave, sm,
+                                                                          spin_limit);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -62,6 +62,14 @@ struct GemmParams {
     int groups_per_split;   // ceil(G / split)
 };
 
+// A split-K workspace starts with a block of arrival counters of fixed size (64 KiB), whatever the problem; the
+// kernels that quantise the token rows themselves keep their two counters (rows ready, workgroups past the wait) in
+// its last two slots.
+constexpr int kCounterBlockBytes = 64 << 10;
+constexpr int kRowFlagSlot = kCounterBlockBytes / 4 - 2;
+constexpr int kMaxSplitCounters = kRowFlagSlot;  // arrival counters a split-K launch may use
+constexpr int kRowsMax = 32;                     // token rows of a launch that quantises them itself
+
 // Problem table of a grouped skinny launch; passed by value in the kernel arguments (< 4 KiB).
 constexpr int kGroupedWavesPerWg = 8;  // wavefronts per workgroup of the grouped skinny kernel
 constexpr int kFusedMaxRows = 4;       // fused activation quantisation: at most this many token rows ...

@@ -35,6 +35,9 @@ hipError_t launch_skinny(const GemmParams& p, int gs, int waves, bool asym, bool
 // the same kernel with the activation quantisation inside: p.x / p.ldx / p.x_bf16 instead of p.q, p.s_a, p.rowsum;
 // at most kFusedMaxRows token rows with rows x K <= kFusedMaxBytes
 hipError_t launch_skinny_fused(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, hipStream_t stream);
+// The same for up to 32 rows, quantised by the grid's first workgroups into the workspace (p.q / p.s_a / p.rowsum point
+// there, p.ws_counter at the workspace's counter block); spin_limit bounds the wait for the rows.
+hipError_t launch_skinny_rows(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, int spin_limit, hipStream_t stream);
 
 // one problem of 17..32 token rows through the shared-activation workgroups (kSharedParts k-parts x
 // 8 / kSharedParts strips per workgroup, p.split K splits across workgroups)

@@ -219,19 +219,22 @@ def w2a8_gemm(qa: QuantizedActivation, w: W2A8Weight, out_dtype=torch.float16, *
     return (out, acc) if acc is not None else out
 
 
-FUSED_MAX_ROWS, FUSED_MAX_BYTES = 4, 32768
+FUSED_MAX_ROWS = 32
+FUSED_IN_WORKGROUP_ROWS, FUSED_IN_WORKGROUP_BYTES = 4, 32768
 
 
 def fused_applies(M: int, K: int) -> bool:
-    """Whether w2a8_linear_fused takes this shape (at most four token rows, M * K <= 32768)."""
-    return 1 <= M <= FUSED_MAX_ROWS and M * K <= FUSED_MAX_BYTES
+    """Whether w2a8_linear_fused takes this shape: up to 32 token rows (up to four rows of at most 32 KiB of int8
+    values together are quantised by every workgroup for itself, more or longer rows by the grid's first workgroups
+    into the workspace)."""
+    return 1 <= M <= FUSED_MAX_ROWS
 
 
 def w2a8_linear_fused(x: torch.Tensor, w: W2A8Weight, out_dtype=torch.float16, *, split_k: int = 0,
                       out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[M, N] for at most four token rows x [M, K] fp16 / bf16 in ONE launch: the activation
+    """out[M, N] for up to 32 token rows x [M, K] fp16 / bf16 in ONE launch: the activation
     quantisation runs inside the GEMM kernel.  Bit-identical with
-    ``w2a8_gemm(quantize_act_int8(x), w, kernel="skinny", split_k=...)``."""
+    ``w2a8_gemm(quantize_act_int8(x), w, kernel="skinny", split_k=...)`` on the one-strip-per-workgroup kernel."""
     L = _lib.lib()
     _require_cuda(x, "x")
     if x.dim() != 2 or x.dtype not in _DT:
@@ -242,7 +245,7 @@ def w2a8_linear_fused(x: torch.Tensor, w: W2A8Weight, out_dtype=torch.float16, *
     if K != w.K:
         raise ValueError(f"activation K={K} does not match weight K={w.K}")
     if not fused_applies(M, K):
-        raise ValueError(f"w2a8_linear_fused handles M <= {FUSED_MAX_ROWS} with M * K <= {FUSED_MAX_BYTES} (M={M}, K={K})")
+        raise ValueError(f"w2a8_linear_fused handles 1 <= M <= {FUSED_MAX_ROWS} (M={M})")
     if x.stride(1) != 1 or x.stride(0) % 8 != 0 or x.stride(0) < K or x.data_ptr() % 16 != 0:
         x = x.contiguous()
         if x.data_ptr() % 16 != 0:      # contiguous already, but not at a 16-byte boundary
@@ -251,7 +254,7 @@ def w2a8_linear_fused(x: torch.Tensor, w: W2A8Weight, out_dtype=torch.float16, *
     if out is None:
         out = torch.empty((M, w.N), dtype=out_dtype, device=dev)
     with torch.cuda.device(dev):
-        ws_bytes = L.slimk_w2a8_gemm_workspace_bytes(M, w.N, K, w.group_size, _lib.KERNEL_SKINNY, split_k)
+        ws_bytes = L.slimk_w2a8_gemm_fused_workspace_bytes(M, w.N, K, w.group_size, split_k)
         ws = _workspace(w, ws_bytes)
         _lib.check(L.slimk_w2a8_gemm_fused(
             x.data_ptr(), x.stride(0), _DT[x.dtype], w.w_r.data_ptr(), w.s_r.data_ptr(),

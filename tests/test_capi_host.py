@@ -178,8 +178,18 @@ def test_repack_and_act_quant_validation(L):
     # (x, ldx, dtype, w_r, s_r, zp_r, zp_const, M, N, K, group, out, ldo, out_dtype, ws, ws_bytes, split, stream)
     gf = L.slimk_w2a8_gemm_fused
     assert gf(None, 4096, 0, FAKE, FAKE, None, 2, 1, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 0, None) == 1
-    assert gf(FAKE, 4096, 0, FAKE, FAKE, None, 2, 5, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 0, None) == 7   # more than four rows
-    assert gf(FAKE, 16384, 0, FAKE, FAKE, None, 2, 4, 4096, 16384, 128, FAKE, 4096, 0, None, 0, 0, None) == 7  # rows x K > 32768
+    # more than four rows, or rows x K > 32768: the rows go through the workspace, which must be there and big enough
+    assert gf(FAKE, 4096, 0, FAKE, FAKE, None, 2, 5, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 0, None) == 5
+    assert gf(FAKE, 16384, 0, FAKE, FAKE, None, 2, 4, 4096, 16384, 128, FAKE, 4096, 0, FAKE, 65536, 0, None) == 5
+    assert gf(FAKE, 4096, 0, FAKE, FAKE, None, 2, 33, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 0, None) == 7  # more than 32 rows
+    fw = L.slimk_w2a8_gemm_fused_workspace_bytes   # (M, N, K, group, split)
+    assert fw(1, 4096, 4096, 128, 0) == 0 and fw(4, 4096, 4096, 128, 1) == 0       # in-workgroup form, K unsplit
+    assert fw(1, 4096, 14336, 128, 0) == L.slimk_w2a8_gemm_workspace_bytes(1, 4096, 14336, 128, 1, 0)
+    assert fw(5, 4096, 4096, 128, 1) == 65536 + 32 * 4096 + 256 + 32 * 32 * 4       # counters, int8 rows, scales, group sums
+    assert fw(32, 4096, 4096, 128, 2) == fw(5, 4096, 4096, 128, 1) + 2 * 64 * 2 * 16 * 64 * 4
+    assert fw(33, 4096, 4096, 128, 0) == 0 and fw(5, 4096, 4000, 128, 0) == 0
+    old = L.slimk_w2a8_set_fused_spin_limit(7)
+    assert L.slimk_w2a8_set_fused_spin_limit(old) == 7 and old > 0
     assert gf(FAKE, 4000, 0, FAKE, FAKE, None, 2, 1, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 0, None) == 2   # ldx < K
     assert gf(FAKE, 4100, 0, FAKE, FAKE, None, 2, 1, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 0, None) == 3   # ldx % 8
     assert gf(FAKE, 4096, 2, FAKE, FAKE, None, 2, 1, 4096, 4096, 128, FAKE, 4096, 0, None, 0, 0, None) == 4

@@ -87,7 +87,11 @@ def test_weight_quantisation_on_gpu_bit_exact(gpu_ops, oracle, N, K, g, mode, bf
                                                  # many rows, long rows, odd row counts
                                                  (64, 4096, 128, False, True), (77, 8192, 64, True, False),
                                                  (130, 14336, 128, False, True), (67, 192, 64, False, False),
-                                                 (65, 6144, 256, True, False), (66, 16448, 64, False, False)])
+                                                 (65, 6144, 256, True, False), (66, 16448, 64, False, False),
+                                                 # a few long rows: 1024 threads a row (one, two or four vectors each)
+                                                 (16, 14336, 128, False, True), (64, 8192, 128, True, False),
+                                                 (3, 28672, 64, False, False), (32, 32768, 256, False, False),
+                                                 (7, 33280, 64, False, False)])
 def test_act_quant_bit_exact(gpu_ops, oracle, M, K, g, bf16, outliers):
     _say("act_quant", M, K, g, bf16)
     case = pu.small_case(M, 64, K, g, "sym", seed=M * 7 + K, outliers=outliers)
@@ -480,9 +484,18 @@ def test_grouped_kernel_shape_classes(gpu_ops, oracle, g, mode, shapes):
     (4, 1024, 8192, 64, "ref", "bfloat16", "float16", 1),
     (4, 64, 2368, 64, "sym", "float16", "float16", 0),         # 37 steps: a ragged last chunk
     (1, 5120, 28672, 64, "sym", "float16", "bfloat16", 0),
+    # more than four rows, or rows too long for LDS: the grid's first workgroups quantise them into the workspace
+    (5, 4096, 4096, 128, "sym", "float16", "float16", 0),
+    (4, 256, 14336, 128, "sym", "float16", "float16", 0),      # few rows, but 56 KiB of them; K split across workgroups
+    (16, 1000, 4096, 64, "asym", "bfloat16", "bfloat16", 0),
+    (17, 130, 8192, 128, "ref", "float16", "float16", 1),      # two row blocks, activations fetched two steps wide
+    (32, 4096, 4096, 128, "sym", "float16", "bfloat16", 0),
+    (32, 192, 14336, 128, "asym", "float16", "float16", 0),
+    (24, 64, 512, 256, "asym", "float16", "float16", 0),       # a grid of two workgroups for 24 rows: several rows each
+    (9, 64, 2368, 64, "sym", "bfloat16", "float16", 0),        # 37 steps: a ragged last chunk
 ])
 def test_fused_activation_quantisation_matches_two_launches(gpu_ops, oracle, M, N, K, g, mode, xdt, out, split):
-    """At most four token rows: slimk_w2a8_gemm_fused quantises the rows inside the GEMM kernel.  Same
+    """Up to 32 token rows: slimk_w2a8_gemm_fused quantises the rows inside the GEMM launch.  Same
     bits as act-quant followed by the skinny kernel with the same split, and the oracle's output."""
     _say("fused", M, N, K, g, mode, xdt, out, split)
     case = pu.small_case(M, N, K, g, mode, seed=M + N + K, out_dtype=out)
@@ -510,4 +523,19 @@ def test_fused_activation_quantisation_matches_two_launches(gpu_ops, oracle, M, 
     np.testing.assert_array_equal(pu.out_tensor_bits(lin(xd)), pu.out_tensor_bits(
         gpu_ops.w2a8_gemm(gpu_ops.quantize_act_int8(xd, g), w, odt)))
     with pytest.raises(ValueError):
-        gpu_ops.w2a8_linear_fused(torch.zeros(5, K, dtype=xd.dtype, device="cuda"), w, odt)
+        gpu_ops.w2a8_linear_fused(torch.zeros(33, K, dtype=xd.dtype, device="cuda"), w, odt)
+    if M > 4 or M * K > 32768:
+        # the bounded wait: with no polls at all every workgroup quantises the rows itself; with few, some do
+        from slimkernels_amd import _lib
+        for polls in (0, 3):
+            old = _lib.lib().slimk_w2a8_set_fused_spin_limit(polls)
+            try:
+                again = gpu_ops.w2a8_linear_fused(xd, w, odt, split_k=split)
+                torch.cuda.synchronize()
+            finally:
+                _lib.lib().slimk_w2a8_set_fused_spin_limit(old)
+            np.testing.assert_array_equal(pu.out_tensor_bits(again), pu.out_tensor_bits(fused))
+        # and the workspace is left ready for the next call, of this or another kind
+        np.testing.assert_array_equal(pu.out_tensor_bits(gpu_ops.w2a8_linear_fused(xd, w, odt, split_k=split)), pu.out_tensor_bits(fused))
+        np.testing.assert_array_equal(pu.out_tensor_bits(gpu_ops.w2a8_gemm(gpu_ops.quantize_act_int8(xd, g), w, odt, kernel="skinny", split_k=split)),
+                                      pu.out_tensor_bits(two))

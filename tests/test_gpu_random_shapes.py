@@ -59,7 +59,7 @@ def test_random_single_gemms(gpu_ops, oracle, seed):
         bound = pu.reorder_bound(ref["acc"], scales, ref["s_a"])
         for o in (out, out2):
             pu.assert_out_close(pu.out_tensor_bits(o), ref["out_bits"], bf16, bound, tag)
-        if case.M <= 4 and case.M * case.K <= 32768:
+        if case.M <= 32:
             o3 = gpu_ops.w2a8_linear_fused(xd, w, pu.torch_dtype(case))
             pu.assert_out_close(pu.out_tensor_bits(o3), ref["out_bits"], bf16, bound, tag + " fused")
         checked += 1
