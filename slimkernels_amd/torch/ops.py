@@ -16,6 +16,7 @@ computes on the CPU.
 from __future__ import annotations
 
 import ctypes
+import collections
 import dataclasses
 from typing import Optional
 
@@ -46,11 +47,18 @@ class W2A8Weight:
     N: int
     K: int
     group_size: int
-    workspace: Optional[torch.Tensor] = None  # lazily created split-K workspace (uint8)
+    # lazily created split-K workspaces (uint8), one per stream the weight is used on: calls that share a workspace
+    # must not overlap in time, and work on one stream does not
+    workspaces: dict = dataclasses.field(default_factory=dict)
 
     @property
     def device(self):
         return self.w_r.device
+
+    @property
+    def workspace(self) -> Optional[torch.Tensor]:
+        """The workspace of the current stream (None if no call on it has needed one yet)."""
+        return self.workspaces.get(_stream_ptr(self.device))
 
 
 @dataclasses.dataclass
@@ -177,11 +185,13 @@ def quantize_act_int8(x: torch.Tensor, group_size: int = 128, copies: int = 1) -
 def _workspace(w: W2A8Weight, nbytes: int) -> Optional[torch.Tensor]:
     if nbytes == 0:
         return None
-    if w.workspace is None or w.workspace.numel() < nbytes:
-        w.workspace = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
-        _lib.check(_lib.lib().slimk_w2a8_workspace_init(w.workspace.data_ptr(), w.workspace.numel(),
-                                                       _stream_ptr(w.device)))
-    return w.workspace
+    key = _stream_ptr(w.device)
+    ws = w.workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+        _lib.check(_lib.lib().slimk_w2a8_workspace_init(ws.data_ptr(), ws.numel(), key))
+        w.workspaces[key] = ws
+    return ws
 
 
 def w2a8_gemm(qa: QuantizedActivation, w: W2A8Weight, out_dtype=torch.float16, *, kernel: str = "auto",
@@ -351,16 +361,39 @@ def wint2_gemm(activation: torch.Tensor, weight: torch.Tensor, scale: torch.Tens
     """One-shot form with the argument order of the upstream notebook entry
     wint2_gemm(activation, weight, scale) (triton.ipynb cell 1): ``activation`` [M, K]
     fp16/bf16, ``weight`` the packed matrix transposed, [K/4, N] uint8 (upstream passes
-    ``packed_weight.T``), ``scale`` [G, N] fp16.  Repacks on every call — use
-    repack_w2 + w2a8_gemm or W2A8Linear in a real loop."""
+    ``packed_weight.T``), ``scale`` [G, N] fp16.  The weight is re-laid for the GPU on the first call with
+    a given (weight, scale, zp) and kept for the next ones (a handful of layers; tensors are recognised by
+    identity and version counter, so an in-place change re-lays them; numpy arrays are re-laid every time)."""
     _require_cuda(activation, "activation")
-    packed = weight.t().contiguous()
-    K = packed.shape[1] * 4
+    K = weight.shape[0] * 4
     if group_size is None:
         group_size = K // scale.shape[0]
-    w = repack_w2(packed, scale, zp, group_size, zp_const, device=activation.device)
+    w = _wint2_weight(weight, scale, zp, group_size, zp_const, activation.device)
     qa = quantize_act_int8(activation, group_size)
     return w2a8_gemm(qa, w, out_dtype or activation.dtype)
+
+
+_WINT2_CACHE: "collections.OrderedDict" = collections.OrderedDict()
+_WINT2_CACHE_SIZE = 16
+
+
+def _wint2_weight(weight, scale, zp, group_size, zp_const, device) -> W2A8Weight:
+    """The repacked form of wint2_gemm's weight operands, cached by tensor identity and version."""
+    tensors = [t for t in (weight, scale, zp) if t is not None]
+    if not all(isinstance(t, torch.Tensor) for t in tensors):
+        return repack_w2(np.ascontiguousarray(np.asarray(weight).T) if not isinstance(weight, torch.Tensor) else weight.t().contiguous(),
+                         scale, zp, group_size, zp_const, device=device)
+    key = tuple((id(t), t.data_ptr(), t._version, tuple(t.shape), tuple(t.stride())) for t in tensors) + (
+        zp is None, group_size, zp_const, str(device))
+    hit = _WINT2_CACHE.get(key)
+    if hit is not None:
+        _WINT2_CACHE.move_to_end(key)
+        return hit[0]
+    w = repack_w2(weight.t().contiguous(), scale, zp, group_size, zp_const, device=device)
+    _WINT2_CACHE[key] = (w, tensors)   # the tensors are held so that their ids and addresses stay theirs
+    while len(_WINT2_CACHE) > _WINT2_CACHE_SIZE:
+        _WINT2_CACHE.popitem(last=False)
+    return w
 
 
 class W2A8Linear(torch.nn.Module):

@@ -384,6 +384,54 @@ def test_wint2_gemm_and_linear_entry_points(gpu_ops, oracle):
     np.testing.assert_array_equal(pu.out_tensor_bits(y2.reshape(5, 128)), pu.out_tensor_bits(y))
 
 
+def test_wint2_gemm_keeps_the_repacked_weight_until_it_changes(gpu_ops, oracle):
+    from slimkernels_amd.torch import ops as ops_mod
+    case = pu.small_case(3, 192, 512, 128, "sym", seed=21)
+    packed, scales, zero = pu.quantized_weight(case)
+    x = workloads.make_activation(case)
+    xd = torch.from_numpy(x).cuda()
+    wt, sc = torch.from_numpy(packed).cuda().t(), torch.from_numpy(scales).cuda()
+    ops_mod._WINT2_CACHE.clear()
+    y1 = gpu_ops.wint2_gemm(xd, wt, sc)
+    assert len(ops_mod._WINT2_CACHE) == 1
+    held = next(iter(ops_mod._WINT2_CACHE.values()))[0]
+    y2 = gpu_ops.wint2_gemm(xd, wt, sc)
+    assert len(ops_mod._WINT2_CACHE) == 1 and next(iter(ops_mod._WINT2_CACHE.values()))[0] is held
+    assert torch.equal(y1, y2)
+    ref = oracle.reference_forward(x, packed, scales, zero, 128)
+    pu.assert_out_close(pu.out_tensor_bits(y2), ref["out_bits"], False, pu.reorder_bound(ref["acc"], scales, ref["s_a"]), "wint2 cached")
+    # an in-place change of the packed weight is seen (version counter): re-laid, new result
+    packed2 = packed.copy()
+    packed2[:, :8] ^= 0x55
+    wt.copy_(torch.from_numpy(packed2).cuda().t())
+    y3 = gpu_ops.wint2_gemm(xd, wt, sc)
+    ref3 = oracle.reference_forward(x, packed2, scales, zero, 128)
+    pu.assert_out_close(pu.out_tensor_bits(y3), ref3["out_bits"], False, pu.reorder_bound(ref3["acc"], scales, ref3["s_a"]), "wint2 changed")
+    assert not torch.equal(y3, y1)
+    for _ in range(40):   # the cache stays small
+        gpu_ops.wint2_gemm(xd, wt.clone(), sc)
+    assert len(ops_mod._WINT2_CACHE) <= ops_mod._WINT2_CACHE_SIZE
+
+
+def test_split_k_workspaces_are_per_stream(gpu_ops, oracle):
+    """A weight used on two streams gets a workspace for each (calls that share one must not overlap in time)."""
+    case = pu.small_case(16, 128, 14336, 128, "sym", seed=4)
+    packed, scales, zero = pu.quantized_weight(case)
+    x = workloads.make_activation(case)
+    w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, x)
+    qa = gpu_ops.quantize_act_int8(xd, 128)
+    y0 = gpu_ops.w2a8_gemm(qa, w, kernel="skinny", split_k=4)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        y1 = gpu_ops.w2a8_gemm(qa, w, kernel="skinny", split_k=4)
+    side.synchronize()
+    assert len(w.workspaces) == 2
+    a, b = w.workspaces.values()
+    assert a.data_ptr() != b.data_ptr()
+    assert torch.equal(y0, y1)
+
+
 def test_grouped_launch_matches_single_launches(gpu_ops, oracle):
     """One grouped launch over problems of different M, N, K against the oracle, and against the same
     problems launched one by one (another kernel body with another fp32 summation order: the two may
