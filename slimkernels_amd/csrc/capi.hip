@@ -49,7 +49,7 @@ int check_kg(int K, int group_size) {
 
 // The kernels address weights and activations through 32-bit buffer offsets.
 int check_extent(int M, int N, int K, int ldq) {
-    const size_t wbytes = (size_t)((N + w2a8::kStripN - 1) / w2a8::kStripN) * (size_t)(K / w2a8::kStepK) * (w2a8::kUnitDwords * 4);
+    const size_t wbytes = w2a8::weight_bytes((N + w2a8::kStripN - 1) / w2a8::kStripN, K / w2a8::kStepK);
     const size_t qbytes = (size_t)M * (size_t)ldq;
     if (wbytes > 0x7fffffffu || qbytes > 0x7fffffffu)
         return fail(SLIMK_ERR_UNSUPPORTED, "repacked weights (%zu bytes) or activations (%zu bytes) exceed 2 GiB", wbytes, qbytes);
@@ -183,7 +183,7 @@ const char* slimk_w2a8_last_error(void) { return g_last_error.c_str(); }
 
 size_t slimk_w2a8_repacked_weight_bytes(int N, int K) {
     if (N <= 0 || K <= 0 || K % 64 != 0) return 0;
-    return (size_t)strips_of(N) * (K / 64) * w2a8::kUnitDwords * 4;
+    return w2a8::weight_bytes(strips_of(N), K / 64);
 }
 
 size_t slimk_w2a8_repacked_scale_bytes(int N, int K, int group_size) {

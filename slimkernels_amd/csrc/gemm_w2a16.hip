@@ -57,8 +57,8 @@ __global__ __launch_bounds__(kWaves * 64) void w2a16_kernel(const W2A16Params p)
     const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(p.x), 0, (int)min((size_t)p.M * p.ldx * 2, (size_t)0x7fffffff), 0x00020000);
     const uint32_t x_lane = ((uint32_t)(m0 + col) * (uint32_t)p.ldx + quad * 16) * 2;   // bytes
-    const uint32_t* w_lane = p.w_r + ((size_t)strip * 64 + lane) * 4;
-    const size_t w_step = (size_t)p.strips * kUnitDwords;                               // dwords between steps
+    const uint32_t* w_lane = p.w_r + ((size_t)strip * kRunSteps * 64 + lane) * 4;       // the strip's first run of four steps
+    const size_t w_run = (size_t)p.strips * kRunSteps * kUnitDwords;                    // dwords between runs
     const uint16_t* s_lane = p.s_r + ((size_t)strip * 16 + col) * 4;
     const uint8_t* z_lane = ZP ? p.zp_r + ((size_t)strip * 16 + col) * 4 : nullptr;
     const size_t sz_group = (size_t)p.strips * 64;                                      // elements between groups
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kWaves * 64) void w2a16_kernel(const W2A16Params p)
         WChunk ch;
         const int st = step0 + c * kChunkSteps;
 #pragma unroll
-        for (int s = 0; s < kChunkSteps; ++s) ch.w[s] = *reinterpret_cast<const v4i*>(w_lane + (size_t)(st + s) * w_step);
+        for (int s = 0; s < kChunkSteps; ++s) ch.w[s] = *reinterpret_cast<const v4i*>(w_lane + (size_t)((st + s) / kRunSteps) * w_run + (size_t)((st + s) % kRunSteps) * kUnitDwords);
         return ch;
     };
     auto load_a = [&](int c) {

@@ -8,15 +8,20 @@ namespace w2a8 {
 // interchange layout (matrix_packer.py:33-34: byte j of row n holds k = 4j..4j+3,
 // k = 4j in bits 7:6).  See w2a8_common.h for the target layout.
 __global__ __launch_bounds__(256) void repack_codes_kernel(const uint8_t* __restrict__ w_packed, int ldw,
-                                                           int N, int strips, size_t total_dwords,
+                                                           int N, int strips, int steps, size_t total_dwords,
                                                            uint32_t* __restrict__ w_r) {
     size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total_dwords) return;
     const int i = (int)(idx & 3);
     const int lane = (int)((idx >> 2) & 63);
-    const size_t unit = idx >> 8;
-    const int strip = (int)(unit % (size_t)strips);
-    const int step = (int)(unit / (size_t)strips);
+    const size_t unit = idx >> 8;                       // units in memory order: run, strip, step of the run
+    const size_t rs = unit / kRunSteps;
+    const int strip = (int)(rs % (size_t)strips);
+    const int step = (int)(rs / (size_t)strips) * kRunSteps + (int)(unit % kRunSteps);
+    if (step >= steps) {                                // padding of the last run
+        w_r[idx] = 0u;
+        return;
+    }
     const int col = lane & 15, quad = lane >> 4;
     const int src_byte = step * 16 + quad * 4 + i;  // (step*64 + quad*16 + 4*i) / 4
     uint32_t out = 0;
@@ -57,9 +62,9 @@ hipError_t launch_repack(const uint8_t* w_packed, int ldw, const uint16_t* scale
     const int steps = K / kStepK;
     const int strips = (N + kStripN - 1) / kStripN;
     const int G = K / group_size;
-    const size_t total = (size_t)strips * steps * kUnitDwords;
+    const size_t total = weight_bytes(strips, steps) / 4;
     repack_codes_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream>>>(
-        w_packed, ldw, N, strips, total, w_r);
+        w_packed, ldw, N, strips, steps, total, w_r);
     const size_t stotal = (size_t)strips * G * 64;
     repack_scales_kernel<<<dim3((unsigned)((stotal + 255) / 256)), dim3(256), 0, stream>>>(
         scales, zp, N, strips, stotal, s_r, zp ? zp_r : nullptr);

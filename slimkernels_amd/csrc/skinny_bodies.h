@@ -2,8 +2,8 @@
 //
 // skinny_kernel: one GEMM per launch.  Grid (strips, split, 16-row token blocks).  A workgroup of
 // NW (4, 8 or 16) wavefronts owns one 64-channel strip and a contiguous range of scale groups; its
-// waves take contiguous sub-ranges, so each wave streams a run of 1 KiB weight units (step-major
-// layout) straight from global memory into VGPRs (one buffer_load_dwordx4 per lane and unit:
+// waves take contiguous sub-ranges, so each wave streams a run of 1 KiB weight units (four consecutive
+// steps of a strip are 4 KiB in one piece) straight from global memory into VGPRs (one buffer_load_dwordx4 per lane and unit:
 // nothing in a unit is shared between waves).  A single decode GEMM is a latency problem before
 // it is a bandwidth problem (the whole thing is a few microseconds), so every load is issued as
 // early as possible:
@@ -276,11 +276,11 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
     // before each use waits for exactly that load (a token row >= M only ever feeds output rows >= M,
     // which are not stored; a clamped step or group is never used).
     const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint32_t*>(p.w_r), 0, (int)((size_t)p.strips * p.steps * (kUnitDwords * 4)), 0x00020000);
+        const_cast<uint32_t*>(p.w_r), 0, (int)weight_bytes(p.strips, p.steps), 0x00020000);
     const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<int8_t*>(qp), 0, (int)((size_t)(M - 1) * p.ldq + p.K), 0x00020000);
-    const uint32_t wstride = (uint32_t)p.strips * (kUnitDwords * 4);  // bytes between consecutive steps of a strip
-    const uint32_t wbase = (uint32_t)strip * (kUnitDwords * 4);
+    const uint32_t wstride = (uint32_t)p.strips * (kRunSteps * kUnitBytes);  // bytes between consecutive runs of a strip
+    const uint32_t wbase = (uint32_t)strip * (kRunSteps * kUnitBytes);
     const uint32_t wlane = lane * 16;
     uint32_t aoff[MB];
 #pragma unroll
@@ -338,7 +338,8 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
         }
     };
     auto issue = [&](int slot, int step, bool with_a = true) {  // step is wave-uniform
-        wring[slot] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane, step * wstride + wbase, NT ? kStreamOnce : 0);
+        wring[slot] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane, (step / kRunSteps) * wstride + (step % kRunSteps) * kUnitBytes + wbase,
+                                                            NT ? kStreamOnce : 0);
         if (with_a) issue_a(slot, step);
     };
     // WIDE: fragment (pair q, row half h) of a chunk: lane l reads row 8h + l/8, 16-byte piece l%8 of the
@@ -841,11 +842,11 @@ __device__ __forceinline__ void shared_body(const GemmParams& p, const int unit,
     auto stepof = [&](int it) { return s0 + max(min(it, len - 1), 0); };
 
     const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint32_t*>(p.w_r), 0, (int)((size_t)p.strips * p.steps * (kUnitDwords * 4)), 0x00020000);
+        const_cast<uint32_t*>(p.w_r), 0, (int)weight_bytes(p.strips, p.steps), 0x00020000);
     const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<int8_t*>(qp), 0, (int)((size_t)(M - 1) * p.ldq + p.K), 0x00020000);
-    const uint32_t wstride = (uint32_t)p.strips * (kUnitDwords * 4);
-    const uint32_t wbase = (uint32_t)strip * (kUnitDwords * 4);
+    const uint32_t wstride = (uint32_t)p.strips * (kRunSteps * kUnitBytes);  // bytes between consecutive runs of a strip
+    const uint32_t wbase = (uint32_t)strip * (kRunSteps * kUnitBytes);
     const uint32_t wlane = lane * 16;
     const uint32_t aoff = (uint32_t)min(col, M - 1) * (uint32_t)p.ldq + quad * 16;
 
@@ -881,7 +882,8 @@ __device__ __forceinline__ void shared_body(const GemmParams& p, const int unit,
     // barrier); otherwise they are fetched once per sharing set and handed round through LDS.
     v4u wring[kDepth];
     auto issue_w = [&](int slot, int step) {
-        wring[slot] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane, step * wstride + wbase, NT ? kStreamOnce : 0);
+        wring[slot] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane, (step / kRunSteps) * wstride + (step % kRunSteps) * kUnitBytes + wbase,
+                                                            NT ? kStreamOnce : 0);
     };
     v4u aring[kDepth];
     auto issue_a = [&](int slot, int step) {

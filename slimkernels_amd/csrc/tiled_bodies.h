@@ -117,7 +117,7 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
     const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<int8_t*>(p.q), 0, (int)min((size_t)p.M * p.ldq, (size_t)0x7fffffff), 0x00020000);
     const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint32_t*>(p.w_r), 0, (int)min((size_t)p.strips * p.steps * (kUnitDwords * 4) * kWPlanes, (size_t)0x7fffffff), 0x00020000);
+        const_cast<uint32_t*>(p.w_r), 0, (int)min(weight_bytes(p.strips, p.steps * kWPlanes), (size_t)0x7fffffff), 0x00020000);
     const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(p.s_r), 0, (int)min((size_t)p.strips * p.G * 128, (size_t)0x7fffffff), 0x00020000);
     uint32_t a_off[kALoads];
@@ -126,8 +126,9 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
         const int blk = wave + 4 * i;  // block = step_in_stage * kMB + token block
         a_off[i] = (uint32_t)(m_tile + (blk % kMB) * 16 + col) * (uint32_t)p.ldq + (blk / kMB) * kStepK + quad * 16;
     }
-    const uint32_t b_step_stride = (uint32_t)p.strips * (kUnitDwords * 4);  // bytes between steps of a strip
-    const uint32_t b_strip_off = (uint32_t)strip * (kUnitDwords * 4);
+    const uint32_t b_run_pitch = (uint32_t)p.strips * (kRunSteps * kUnitBytes);  // bytes between runs of four steps of a strip
+    const uint32_t b_strip_off = (uint32_t)strip * (kRunSteps * kUnitBytes);
+    auto unit_off = [&](int step) { return (uint32_t)(step / kRunSteps) * b_run_pitch + (uint32_t)(step % kRunSteps) * kUnitBytes + b_strip_off; };
     const uint32_t s_lane_off = (uint32_t)(strip * 16 + col) * 8;
     const uint32_t s_group_stride = (uint32_t)p.strips * 128;               // bytes between groups of a strip
     typedef unsigned v2u __attribute__((ext_vector_type(2)));
@@ -146,13 +147,13 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
         for (int s = 0; s < kStageSteps; ++s)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
                 w_rsrc, (__attribute__((address_space(3))) void*)&lds[buf][kStageDwords + (wave * kStageSteps + s) * 256], 16,
-                lane * 16, ((stage0 + stage) * kStageSteps + s) * b_step_stride + b_strip_off, 0, 0);
+                lane * 16, unit_off((stage0 + stage) * kStageSteps + s), 0, 0);
         if constexpr (W4) {
 #pragma unroll
             for (int s = 0; s < kStageSteps; ++s)   // the lo digits of the same steps: p.steps units further on
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(
                     w_rsrc, (__attribute__((address_space(3))) void*)&lds[buf][kStageDwords + kWDwords / 2 + (wave * kStageSteps + s) * 256], 16,
-                    lane * 16, ((stage0 + stage) * kStageSteps + s + p.steps) * b_step_stride + b_strip_off, 0, 0);
+                    lane * 16, unit_off((stage0 + stage) * kStageSteps + s + p.steps), 0, 0);
         }
     };
     auto fetch_scales = [&](int stage) {

@@ -8,10 +8,12 @@
 // so that lane l of a wavefront reads its 16 bytes at offset 16*l (one coalesced
 // global_load_dwordx4 / one conflict-free ds_read_b128 per wave and unit).
 //
-//   unit address   = w_r + ((step * strips + strip) * 64 + lane) * 4     [dwords]
-//   (step-major: the units that all strips need at the same moment are contiguous, so the
-//    chip reads one sequential band per step instead of `strips` power-of-two-strided
-//    streams that pile onto a few HBM channels)
+//   unit address   = w_r + ((((step / 4) * strips + strip) * 4 + step % 4) * 64 + lane) * 4     [dwords]
+//   (four consecutive steps of a strip form one run of 4 KiB, the runs of all strips for the same four steps follow
+//    each other: what a wave streams back to back is contiguous, and what all strips need at the same moment is one
+//    sequential band - a whole strip in one piece would be `strips` power-of-two-strided streams that pile onto a few
+//    HBM channels, single 1 KiB units per step measured 3..9 % slower than the 4 KiB runs; a step count that is no
+//    multiple of four is padded with zero units)
 //   lane l         : col = l & 15, quad = l >> 4
 //   dword i, byte b, 2-bit field p of that byte (bits 2p+1:2p) holds the code of
 //       n = strip*64 + p*16 + col          k = step*64 + quad*16 + 4*i + b
@@ -35,6 +37,20 @@ namespace w2a8 {
 constexpr int kStripN = 64;      // output channels per strip
 constexpr int kStepK = 64;       // reduction elements per MFMA step
 constexpr int kUnitDwords = 256; // dwords per (strip, step) unit
+// Order of the units in memory: kRunSteps consecutive steps of a strip lie together (a run of 4 KiB: what one wave
+// streams back to back), the runs of all strips for the same steps follow each other, then the next kRunSteps steps.
+// A step count that is no multiple of kRunSteps is padded with zero units.
+constexpr int kRunSteps = 4;
+constexpr int kUnitBytes = kUnitDwords * 4;
+__host__ __device__ constexpr int weight_runs(int steps) { return (steps + kRunSteps - 1) / kRunSteps; }
+__host__ __device__ constexpr size_t weight_bytes(int strips, int steps) {
+    return (size_t)weight_runs(steps) * (size_t)strips * kRunSteps * kUnitBytes;
+}
+// byte offset of unit (step, strip): a kernel keeps run_pitch = strips * kRunSteps * kUnitBytes and
+// strip_base = strip * kRunSteps * kUnitBytes and adds (step / kRunSteps) * run_pitch + (step % kRunSteps) * kUnitBytes
+__host__ __device__ constexpr uint32_t weight_unit_offset(int step, int strip, int strips) {
+    return (uint32_t)((((step / kRunSteps) * strips + strip) * kRunSteps + step % kRunSteps) * kUnitBytes);
+}
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 

@@ -7,8 +7,10 @@ e.g. when persisting weights.  Nothing here is used by the GEMM.
 
 Layout: the [N, K] code matrix is cut into units of 64 channels (strip) x 64 reduction
 elements (step); unit (step, strip) is 64 lanes x 4 dwords at dword offset
-((step * strips + strip) * 64 + lane) * 4 (step-major, so that what all strips read at
-the same time is one contiguous band).  With col = lane & 15, quad = lane >> 4, the
+((((step // 4) * strips + strip) * 4 + step % 4) * 64 + lane) * 4: four consecutive steps of a
+strip form one run of 4 KiB (what a wave streams back to back), the runs of all strips for the
+same four steps follow each other (what all strips read at the same time is one contiguous band);
+a step count that is no multiple of four is padded with zero units.  With col = lane & 15, quad = lane >> 4, the
 2-bit field p (bits 2p+1:2p) of byte b of dword i holds the code of
 
     n = strip*64 + p*16 + col        k = step*64 + quad*16 + 4*i + b
@@ -20,10 +22,16 @@ import numpy as np
 
 STRIP_N = 64
 STEP_K = 64
+RUN_STEPS = 4
+
+
+def unit(w_r: np.ndarray, step: int, strip: int) -> np.ndarray:
+    """The [64 lanes, 4 dwords] unit (step, strip) of a repacked array [runs, strips, 4, 64, 4]."""
+    return w_r[step // RUN_STEPS, strip, step % RUN_STEPS]
 
 
 def repack_codes(packed: np.ndarray) -> np.ndarray:
-    """uint8 [N, K/4] interchange bytes -> uint32 [steps, strips, 64, 4] streaming layout."""
+    """uint8 [N, K/4] interchange bytes -> uint32 [runs, strips, 4, 64, 4] streaming layout (run = four steps)."""
     packed = np.asarray(packed, np.uint8)
     N, K = packed.shape[0], packed.shape[1] * 4
     if K % STEP_K:
@@ -41,13 +49,18 @@ def repack_codes(packed: np.ndarray) -> np.ndarray:
         for b in range(4):
             # c[:, p, :, :, :, :, b] has axes strip, col, step, quad, i
             out |= c[:, p, :, :, :, :, b].transpose(0, 2, 3, 1, 4) << np.uint32(8 * b + 2 * p)
-    return np.ascontiguousarray(out.reshape(strips, steps, 64, 4).transpose(1, 0, 2, 3))
+    runs = -(-steps // RUN_STEPS)
+    padded = np.zeros((strips, runs * RUN_STEPS, 64, 4), np.uint32)
+    padded[:, :steps] = out.reshape(strips, steps, 64, 4)
+    return np.ascontiguousarray(padded.reshape(strips, runs, RUN_STEPS, 64, 4).transpose(1, 0, 2, 3, 4))
 
 
 def unrepack_codes(w_r: np.ndarray, N: int, K: int) -> np.ndarray:
     """Inverse of :func:`repack_codes`: streaming layout -> uint8 [N, K/4] interchange bytes."""
     strips, steps = -(-N // STRIP_N), K // STEP_K
-    w = np.asarray(w_r, np.uint32).reshape(steps, strips, 4, 16, 4).transpose(1, 0, 2, 3, 4)  # strip, step, quad, col, i
+    runs = -(-steps // RUN_STEPS)
+    w = np.asarray(w_r, np.uint32).reshape(runs, strips, RUN_STEPS, 64, 4).transpose(1, 0, 2, 3, 4)
+    w = w.reshape(strips, runs * RUN_STEPS, 4, 16, 4)[:, :steps]                                # strip, step, quad, col, i
     codes = np.zeros((strips, 4, 16, steps, 4, 4, 4), np.uint8)       # strip, p, col, step, quad, i, b
     for p in range(4):
         for b in range(4):

@@ -51,7 +51,7 @@ def wave_strip_groups(q, rowsum, w_r, s_r, zp_r, zp_const, strip, groups, gs, M)
                 acc[l, p] = -zpe[l, p] * rs
         for s in range(gs):
             step = g * gs + s
-            w = w_r[step, strip]                          # uint32 [64, 4]
+            w = w_r[step // 4, strip, step % 4]           # uint32 [64, 4]: runs of four steps per strip
             a = np.zeros((64, 16), np.int8)
             for l in range(64):
                 m = col[l]

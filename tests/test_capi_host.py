@@ -39,7 +39,8 @@ def test_version_arch_and_sizes(L):
     assert L.slimk_w2a8_version() == 100
     assert L.slimk_w2a8_arch() == b"gfx950"
     assert L.slimk_w2a8_repacked_weight_bytes(4096, 4096) == 4096 * 4096 // 4
-    assert L.slimk_w2a8_repacked_weight_bytes(100, 128) == 2 * 2 * 1024     # two strips (N padded to 128) x two steps
+    assert L.slimk_w2a8_repacked_weight_bytes(100, 128) == 2 * 4 * 1024     # two strips (N padded to 128) x one run of four steps (two of them padding)
+    assert L.slimk_w2a8_repacked_weight_bytes(64, 576) == 12 * 1024         # nine steps: three runs
     assert L.slimk_w2a8_repacked_scale_bytes(4096, 4096, 128) == 2 * 4096 * 32
     assert L.slimk_w2a8_repacked_zp_bytes(4096, 4096, 128) == 4096 * 32
     assert L.slimk_w2a8_repacked_weight_bytes(4096, 100) == 0               # K % 64

@@ -18,7 +18,8 @@ def _say(*a):
 
 # ------------------------------------------------------------------ repack
 @pytest.mark.parametrize("N,K,g,with_zp", [(64, 64, 64, False), (100, 256, 128, True), (4096, 4096, 128, False),
-                                           (1000, 512, 256, True), (16, 128, 64, True)])
+                                           (1000, 512, 256, True), (16, 128, 64, True), (130, 576, 64, True),
+                                           (77, 1408, 128, False)])
 def test_repack_matches_layout_definition(gpu_ops, N, K, g, with_zp):
     _say("repack", N, K, g, with_zp)
     rng = np.random.default_rng(N + K)
@@ -27,7 +28,7 @@ def test_repack_matches_layout_definition(gpu_ops, N, K, g, with_zp):
     zp = rng.integers(0, 4, (K // g, N), dtype=np.uint8) if with_zp else None
     w = gpu_ops.repack_w2(packed, scales, zp, g)
     strips, steps = -(-N // 64), K // 64
-    got = w.w_r.cpu().numpy().view(np.uint32).reshape(steps, strips, 64, 4)
+    got = w.w_r.cpu().numpy().view(np.uint32).reshape(-(-steps // 4), strips, 4, 64, 4)
     np.testing.assert_array_equal(got, layout.repack_codes(packed))
     np.testing.assert_array_equal(layout.unrepack_codes(got, N, K), packed)
     np.testing.assert_array_equal(w.s_r.cpu().numpy().reshape(K // g, strips, 16, 4), layout.repack_group_values(scales))

@@ -6,12 +6,13 @@ from slimkernels_amd import layout
 from kernel_model import wave_strip_groups
 
 
-@pytest.mark.parametrize("N,K", [(64, 64), (100, 128), (16, 256), (130, 192), (1, 64)])
+@pytest.mark.parametrize("N,K", [(64, 64), (100, 128), (16, 256), (130, 192), (1, 64), (70, 576), (200, 1024)])
 def test_repack_roundtrip(N, K):
     rng = np.random.default_rng(N * 1000 + K)
     packed = rng.integers(0, 256, (N, K // 4), dtype=np.uint8)
     w_r = layout.repack_codes(packed)
-    assert w_r.shape == (K // 64, -(-N // 64), 64, 4)
+    assert w_r.shape == (-(-(K // 64) // 4), -(-N // 64), 4, 64, 4)
+    assert not w_r.reshape(w_r.shape[0], w_r.shape[1], 4, 256)[-1, :, (K // 64 - 1) % 4 + 1:].any()   # padding units are zero
     np.testing.assert_array_equal(layout.unrepack_codes(w_r, N, K), packed)
 
 
@@ -27,7 +28,7 @@ def test_repack_field_definition():
         n, k = int(rng.integers(N)), int(rng.integers(K))
         strip, p, col = n // 64, (n % 64) // 16, n % 16
         step, quad, i, b = k // 64, (k % 64) // 16, (k % 16) // 4, k % 4
-        f = (int(w_r[step, strip, quad * 16 + col, i]) >> (8 * b + 2 * p)) & 3
+        f = (int(layout.unit(w_r, step, strip)[quad * 16 + col, i]) >> (8 * b + 2 * p)) & 3
         assert (f ^ 2 if p == 3 else f) == codes[n, k]
 
 
