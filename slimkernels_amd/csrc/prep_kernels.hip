@@ -168,8 +168,19 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
 // between the absmax pass and the quantising pass, all of its loads in flight together.  With many rows the
 // two-pass kernel moves every row twice (the second time from L2) in phases that the workgroups of a round
 // go through together; this one moves it once.  Same arithmetic per element: bit-identical results.
-// THREADS: 256 in general (many rows: several workgroups per CU); 1024 for a few long rows, where one row per
-// workgroup leaves most of the chip idle and a row's time is what a thread's chain of loads, divisions and stores takes.
+// THREADS: 256 in general (many rows: several workgroups per CU); 512 or 1024 for a few rows, where one row per
+// workgroup leaves most of the chip idle and a row's time is what its one CU needs for the arithmetic: there the
+// IEEE divisions (a dozen instructions each) are most of it, and rne_quotient() below avoids nearly all of them.
+// rintf(x / s) for |x / s| <= 127, with 1 / s at hand.  t = x * (1 / s) lies within 1.5 * 2^-23 * 127 = 2.3e-5 of the
+// quotient the IEEE division returns, so the two round to the same integer unless t is that close to a tie; t - rintf(t)
+// is exact, and within 2^-14 of a tie the division decides.  Bit-identical with rintf(x / s) for finite x.
+__device__ __forceinline__ float rne_quotient(float x, float s, float inv_s) {
+    const float t = x * inv_s;
+    const float r = rintf(t);
+    if (fabsf(fabsf(t - r) - 0.5f) < 6.1035156e-5f) return rintf(x / s);
+    return r;
+}
+
 template <bool BF16, int KEEP, int THREADS = 256>
 __global__ __launch_bounds__(THREADS) void act_quant_keep_kernel(const uint16_t* __restrict__ x, int ldx, int K,
                                                              int group_size, int8_t* __restrict__ q, int ldq,
@@ -203,6 +214,8 @@ __global__ __launch_bounds__(THREADS) void act_quant_keep_kernel(const uint16_t*
     for (int w = 1; w < THREADS / 64; ++w) amax = fmaxf(amax, red[w]);
     const float s = fmaxf(amax, 1e-9f) / 127.0f;
     if (tid == 0) s_a[m] = s;
+    constexpr bool kFewRowsForm = THREADS > 256;
+    const float inv_s = 1.0f / s;
 
     const int tpg = group_size / 8;  // threads per scale group: 8, 16 or 32
     int8_t* qr = q + (size_t)m * ldq;
@@ -216,7 +229,7 @@ __global__ __launch_bounds__(THREADS) void act_quant_keep_kernel(const uint16_t*
             uint32_t lo = 0, hi = 0;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                float r = rintf(f[i] / s);
+                float r = kFewRowsForm ? rne_quotient(f[i], s, inv_s) : rintf(f[i] / s);
                 r = fminf(fmaxf(r, -127.0f), 127.0f);
                 const int qi = (int)r;
                 sum += qi;
@@ -238,6 +251,10 @@ template <bool BF16>
 static void launch_act_quant_keep(const void* x, int ldx, int M, int K, int group_size, int8_t* q, int ldq, float* s_a,
                                   int32_t* rowsum, int ldr, int copies, hipStream_t stream) {
     const dim3 grid((unsigned)M), block(256);
+    if (M <= kFewRows && K > 2048 && K <= 4096) {  // a few rows: 512 threads a row, one vector each
+        act_quant_keep_kernel<BF16, 1, 512><<<grid, dim3(512), 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+        return;
+    }
     if (M <= kFewRows && K > 4096) {  // a few long rows: 1024 threads a row
         const dim3 wide(1024);
         if (K <= 8192)

@@ -122,6 +122,35 @@ def test_act_quant_bit_exact(gpu_ops, oracle, M, K, g, bf16, outliers):
     np.testing.assert_array_equal(qa.rowsum.cpu().numpy()[:, :M], rs)
 
 
+@pytest.mark.parametrize("M,K", [(8, 4096), (16, 8192), (3, 28672), (80, 4096)])
+def test_act_quant_values_next_to_rounding_ties(gpu_ops, oracle, M, K):
+    """Rows of values chosen next to the ties of q = rne(x / s): for a random absmax A (s = A / 127) the fp16 numbers
+    nearest to (k + 1/2) * s and their neighbours.  The kernels for a few rows round x * (1 / s) and fall back on the
+    division near a tie; those for many rows divide: all must give the oracle's bits."""
+    _say("act_quant near ties", M, K)
+    rng = np.random.default_rng(M * 31 + K)
+    x = np.zeros((M, K), np.float16)
+    for m in range(M):
+        A = np.float16(rng.uniform(0.01, 300.0))
+        s = np.float32(max(np.float32(A), np.float32(1e-9))) / np.float32(127.0)
+        k = rng.integers(-127, 127, K).astype(np.float32) + 0.5
+        base = (k * s).astype(np.float16)
+        step = rng.integers(-2, 3, K)          # up to two fp16 neighbours either side
+        moved = base.copy()
+        for d in (1, 2):
+            moved = np.where(step >= d, np.nextafter(moved, np.float16(np.inf)), moved)
+            moved = np.where(step <= -d, np.nextafter(moved, np.float16(-np.inf)), moved)
+        moved = np.clip(moved.astype(np.float32), -np.float32(A), np.float32(A)).astype(np.float16)
+        moved[rng.integers(K)] = A              # the row's absmax is exactly A
+        x[m] = moved
+    q, s_a, rs = oracle.c_act_quant(x, 128)
+    qa = gpu_ops.quantize_act_int8(torch.from_numpy(x).cuda(), 128)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(qa.s_a.cpu().numpy(), s_a)
+    np.testing.assert_array_equal(qa.q.cpu().numpy(), q)
+    np.testing.assert_array_equal(qa.rowsum.cpu().numpy()[:, :M], rs)
+
+
 # ------------------------------------------------------------------ GEMM on small and ragged shapes
 def _run_case(gpu_ops, oracle, case, kernel, split_k=0, dump="groups", exact_out=False, same_bits=True, strict=False):
     """One GEMM twice: with the int32 dump (the verification instantiation of the kernel body the call
