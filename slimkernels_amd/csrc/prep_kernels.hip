@@ -170,17 +170,7 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
 // go through together; this one moves it once.  Same arithmetic per element: bit-identical results.
 // THREADS: 256 in general (many rows: several workgroups per CU); 512 or 1024 for a few rows, where one row per
 // workgroup leaves most of the chip idle and a row's time is what its one CU needs for the arithmetic: there the
-// IEEE divisions (a dozen instructions each) are most of it, and rne_quotient() below avoids nearly all of them.
-// rintf(x / s) for |x / s| <= 127, with 1 / s at hand.  t = x * (1 / s) lies within 1.5 * 2^-23 * 127 = 2.3e-5 of the
-// quotient the IEEE division returns, so the two round to the same integer unless t is that close to a tie; t - rintf(t)
-// is exact, and within 2^-14 of a tie the division decides.  Bit-identical with rintf(x / s) for finite x.
-__device__ __forceinline__ float rne_quotient(float x, float s, float inv_s) {
-    const float t = x * inv_s;
-    const float r = rintf(t);
-    if (fabsf(fabsf(t - r) - 0.5f) < 6.1035156e-5f) return rintf(x / s);
-    return r;
-}
-
+// IEEE divisions (a dozen instructions each) are most of it, and rne_quotient() avoids nearly all of them (w2a8_common.h).
 template <bool BF16, int KEEP, int THREADS = 256>
 __global__ __launch_bounds__(THREADS) void act_quant_keep_kernel(const uint16_t* __restrict__ x, int ldx, int K,
                                                              int group_size, int8_t* __restrict__ q, int ldq,

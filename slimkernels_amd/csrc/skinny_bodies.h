@@ -106,6 +106,7 @@ __device__ __forceinline__ void rows_quantise_row(const GemmParams& p, const int
     for (int w = 1; w < THREADS / 64; ++w) a = fmaxf(a, scratch[w]);
     __syncthreads();  // scratch is free again
     const float s = fmaxf(a, 1e-9f) / 127.0f;
+    const float inv_s = 1.0f / s;
     if (tid == 0) const_cast<float*>(p.s_a)[m] = s;
     int8_t* qr = const_cast<int8_t*>(p.q) + (size_t)m * p.ldq;
     int32_t* rs = const_cast<int32_t*>(p.rowsum);
@@ -119,7 +120,7 @@ __device__ __forceinline__ void rows_quantise_row(const GemmParams& p, const int
             uint32_t lo = 0, hi = 0;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                float r = rintf(f[i] / s);
+                float r = rne_quotient(f[i], s, inv_s);  // = rintf(f[i] / s), bit for bit
                 r = fminf(fmaxf(r, -127.0f), 127.0f);
                 const int qi = (int)r;
                 sum += qi;
@@ -429,9 +430,10 @@ __device__ __forceinline__ void skinny_body(const GemmParams& p, const int strip
         auto quantise8 = [&](const float (&f)[8], float s, uint32_t& lo, uint32_t& hi) -> int {
             int sum = 0;
             lo = 0; hi = 0;
+            const float inv_s = 1.0f / s;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                float r = rintf(f[i] / s);
+                float r = rne_quotient(f[i], s, inv_s);  // = rintf(f[i] / s), bit for bit
                 r = fminf(fmaxf(r, -127.0f), 127.0f);
                 const int qi = (int)r;
                 sum += qi;

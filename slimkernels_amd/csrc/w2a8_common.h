@@ -106,6 +106,16 @@ __device__ __forceinline__ v4i mfma_i8_16x16x64(v4i a, v4i b, v4i c) {
     return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
 }
 
+// rintf(x / s) for |x / s| <= 127, with 1 / s at hand.  t = x * (1 / s) lies within 1.5 * 2^-23 * 127 = 2.3e-5 of the
+// quotient the IEEE division returns, so the two round to the same integer unless t is that close to a tie; t - rintf(t)
+// is exact, and within 2^-14 of a tie the division decides.  Bit-identical with rintf(x / s) for finite x.
+__device__ __forceinline__ float rne_quotient(float x, float s, float inv_s) {
+    const float t = x * inv_s;
+    const float r = rintf(t);
+    if (fabsf(fabsf(t - r) - 0.5f) < 6.1035156e-5f) return rintf(x / s);
+    return r;
+}
+
 __device__ __forceinline__ float half_bits_to_float(uint16_t h) {
     return (float)__builtin_bit_cast(_Float16, h);
 }
