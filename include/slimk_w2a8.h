@@ -25,9 +25,11 @@
  *    the host before anything is launched, so a bad call never reaches the GPU.
  *    slimk_w2a8_last_error() returns a thread-local description of the most
  *    recent failure on the calling thread.  Nothing throws or aborts.
- *  - Re-entrant: no mutable global state; concurrent calls from several host
- *    threads on different streams are fine as long as they do not share a
- *    split-K workspace.
+ *  - Re-entrant: concurrent calls from several host threads on different streams
+ *    are fine as long as they do not share a split-K workspace.  The only state
+ *    the library keeps is the device array behind slimk_w2a8_gemm_static (one per
+ *    GPU, shared by the calls of that entry point) and the poll limit set by the
+ *    test hook slimk_w2a8_set_fused_spin_limit.
  *
  * Shape limits: K % 64 == 0, group_size in {64, 128, 256}, K % group_size == 0.
  * M, N >= 1 are otherwise arbitrary (ragged tiles are handled inside).
