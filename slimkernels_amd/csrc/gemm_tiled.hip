@@ -39,24 +39,38 @@ int tiled_fast_max_split(int M, int strips, int steps, int gs) {
     return gs == 4 ? steps / 4 : (steps + fast::kStageSteps - 1) / fast::kStageSteps;
 }
 
-// With at most half as many 64-row tiles as CUs, K is split over several workgroups per tile so that
-// about two workgroups per CU exist.  Measured: a workgroup alone on a CU spends about 0.7 us per
-// 128-element stage and two on a CU about 1.25 us for both; a split costs the reducing workgroup
-// about a microsecond plus 0.8 us per partial tile it reads.  Hence up to eight splits, each at
-// least eight stages (K >= 1024 per split) long; with more tiles than that a split gains nothing
-// unless the reduction is long.
+// K splits of the 64-row tiles.  A split is judged by three factors, fitted to measurements of 1, 2, 3, 4, 6 and 8
+// splits on thirty shapes (64..512 token rows on the Llama-8B and 70B-class linears, groups of 64 and 128; the rule
+// picks within 1 % of the best measured split on average, 9 % at worst, where the rule it replaces lost up to 32 %):
+//  * how evenly its workgroups fill the CUs: with n = ceil(workgroups / 256) on the fullest CU, workgroups / (256 n);
+//  * how well a CU runs with n workgroups on it: one alone reaches about 0.7 of what three reach together, two 0.9
+//    (nothing hides a lone workgroup's latencies);
+//  * what a workgroup spends outside its stages (prologue, epilogue, publishing or adding up partial tiles): about
+//    ten stages' worth, so a split of `per` stages is per / (per + 10) efficient.
+// 128-row tiles (a chip-filling problem) are not split: measured slower.
 int tiled_fast_auto_split(int M, int strips, int steps, int gs) {
     int bm, tiles;
     tiled_fast_tiles(M, strips, gs, &bm, &tiles);
+    if (bm != 64) return 1;
     const int stages = (steps + fast::kStageSteps - 1) / fast::kStageSteps;
-    // one workgroup per CU on most CUs and a long reduction: two halves (measured at 128 x 28672 x 8192,
-    // 224 tiles of 64 stages: 67.5 -> 61.2 us; at 32 stages per tile the halves are slower: 28.1 -> 31.6 us)
-    if (tiles > 128) return tiles <= 256 && stages >= 64 ? 2 : 1;
-    int split = 512 / tiles;
-    if (split > 8) split = 8;
-    if (split > stages / 8) split = stages / 8;
-    if (split < 1) split = 1;
-    return tiled_fast_effective_split(steps, gs, split, nullptr);
+    static const int kCandidates[] = {1, 2, 3, 4, 6, 8};
+    int best_split = 1;
+    double best_score = -1.0;
+    for (int split : kCandidates) {
+        int per = (stages + split - 1) / split;               // stages per split
+        if (gs == 4) per = (per + 1) / 2 * 2;                 // whole groups of 256: pairs of stages
+        if (split > 1 && per < 4) break;
+        const long long wgs = (long long)tiles * ((stages + per - 1) / per);
+        const long long n = (wgs + 255) / 256;
+        const double fill = (double)wgs / (256.0 * (double)n);
+        const double together = n == 1 ? 0.7 : (n == 2 ? 0.9 : 1.0);
+        const double score = fill * together * (double)per / ((double)per + 10.0);
+        if (score > best_score * 1.0001) {
+            best_score = score;
+            best_split = split;
+        }
+    }
+    return tiled_fast_effective_split(steps, gs, best_split, nullptr);
 }
 
 // What a requested split comes to: whole stages per split (an even number of them with a group of 256), the last
