@@ -47,18 +47,26 @@ int tiled_fast_max_split(int M, int strips, int steps, int gs) {
 //    (nothing hides a lone workgroup's latencies);
 //  * what a workgroup spends outside its stages (prologue, epilogue, publishing or adding up partial tiles): about
 //    ten stages' worth, so a split of `per` stages is per / (per + 10) efficient.
-// 128-row tiles (a chip-filling problem) are not split: measured slower.
+// 128-row tiles (a chip-filling problem) are not split, nor are more than 400 64-row tiles: measured slower (the
+// partial tiles of a thousand workgroups are 130 MB of traffic: 2048 x 4096 x 14336 in two halves 151 against 134 us).
+// Groups of 256 (two workgroups per CU, not three) keep the rule by tile count they were measured with.
 int tiled_fast_auto_split(int M, int strips, int steps, int gs) {
     int bm, tiles;
     tiled_fast_tiles(M, strips, gs, &bm, &tiles);
-    if (bm != 64) return 1;
+    if (bm != 64 || tiles > 400) return 1;
     const int stages = (steps + fast::kStageSteps - 1) / fast::kStageSteps;
+    if (gs == 4) {
+        if (tiles > 128) return tiled_fast_effective_split(steps, gs, tiles <= 256 && stages >= 64 ? 2 : 1, nullptr);
+        int split = 512 / tiles;
+        if (split > 8) split = 8;
+        if (split > stages / 8) split = stages / 8;
+        return tiled_fast_effective_split(steps, gs, split < 1 ? 1 : split, nullptr);
+    }
     static const int kCandidates[] = {1, 2, 3, 4, 6, 8};
     int best_split = 1;
     double best_score = -1.0;
     for (int split : kCandidates) {
-        int per = (stages + split - 1) / split;               // stages per split
-        if (gs == 4) per = (per + 1) / 2 * 2;                 // whole groups of 256: pairs of stages
+        const int per = (stages + split - 1) / split;         // stages per split
         if (split > 1 && per < 4) break;
         const long long wgs = (long long)tiles * ((stages + per - 1) / per);
         const long long n = (wgs + 255) / 256;
