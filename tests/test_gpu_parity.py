@@ -122,11 +122,12 @@ def test_act_quant_bit_exact(gpu_ops, oracle, M, K, g, bf16, outliers):
     np.testing.assert_array_equal(qa.rowsum.cpu().numpy()[:, :M], rs)
 
 
-@pytest.mark.parametrize("M,K", [(8, 4096), (16, 8192), (3, 28672), (80, 4096)])
+@pytest.mark.parametrize("M,K", [(8, 4096), (16, 8192), (3, 28672), (80, 4096), (70, 20480), (130, 14336)])
 def test_act_quant_values_next_to_rounding_ties(gpu_ops, oracle, M, K):
     """Rows of values chosen next to the ties of q = rne(x / s): for a random absmax A (s = A / 127) the fp16 numbers
-    nearest to (k + 1/2) * s and their neighbours.  The kernels for a few rows round x * (1 / s) and fall back on the
-    division near a tie; those for many rows divide: all must give the oracle's bits."""
+    nearest to (k + 1/2) * s and their neighbours.  The kernels round x * (1 / s) and fall back on the IEEE division
+    near a tie (the forms for a few rows, for many rows, and the two-pass form for very long rows): all must give the
+    oracle's bits."""
     _say("act_quant near ties", M, K)
     rng = np.random.default_rng(M * 31 + K)
     x = np.zeros((M, K), np.float16)
