@@ -39,12 +39,12 @@ COLD_FOOTPRINT = 640 << 20    # bytes of distinct weight copies between two uses
 
 # HBM bytes per launch of the dominant kernel from two rocprofv3 --pmc runs of
 # `python3 bench.py --skip-detail` (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same
-# counter reads for this file's 256 MiB calibration read (read_probe_kernel: 131080 -> x2.0) and
-# calibration fill (fill_zero_kernel: 262144 -> x1.0):  (115983 * 2.0 + 2898 * 1.0) KiB.
+# counter reads for this file's 256 MiB calibration read (read_probe_kernel: 131077 -> x2.0) and
+# calibration fill (fill_zero_kernel: 262144 -> x1.0):  (115915 * 2.0 + 2898 * 1.0) KiB.
 # Counters cannot be read from inside a run: the figure is the one of the committed profile summary named in
 # TRAFFIC_SOURCE, taken on the same kernel code (the summary gives the command).
 CLOCK_WARMUP_MS = 150   # untimed run of the measured work before every timed region (see timed_run, time_graph)
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = int((115983 * 2.0 + 2898 * 1.0) * 1024)
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = int((115915 * 2.0 + 2898 * 1.0) * 1024)
 TRAFFIC_SOURCE = "profiles/skinny_grouped_kernel__c2_decode_sweep.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by the in-run 256 MiB read / fill calibration)"
 
 
