@@ -341,6 +341,32 @@ def test_w4a8_one_pass_kernel(gpu_ops, oracle, M, N, K, g, out, mode):
         assert torch.equal(y2.view(torch.int16), y.view(torch.int16))
 
 
+@pytest.mark.gpu
+def test_w4_routes_share_one_workspace(gpu_ops, oracle):
+    """The two-plane road (few rows: split-K skinny kernel over 2K) and the one-pass road (tiled kernel, K split over
+    workgroups) of one weight object use the same workspace, in turn and with changing token counts: every result is
+    the one a fresh weight object gives."""
+    from slimkernels_amd.torch import w4 as tw4
+    N, K, g = 256, 7168, 128
+    w, _ = _w4_case(8, N, K, g, "sym", seed=77)
+    packed4, scales, zp = w4.prepare_w4(w, g, "sym")
+    shared = tw4.repack_w4(packed4, scales, zp, g)
+    rng = np.random.default_rng(5)
+    for M in (20, 64, 8, 200, 20, 40, 64):
+        print("W4 workspace reuse M", M, flush=True)
+        x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float16)).cuda()
+        qa = gpu_ops.quantize_act_int8(x, g)
+        fresh = tw4.repack_w4(packed4, scales, zp, g)
+        if tw4.one_pass_applies(M, shared):
+            got, want = tw4.w4a8_gemm_one_pass(qa, shared), tw4.w4a8_gemm_one_pass(qa, fresh)
+        else:
+            got, want = tw4.w4a8_gemm(qa, shared), tw4.w4a8_gemm(qa, fresh)
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"M={M}"
+    ws = shared.planes.workspace
+    assert ws is not None and int(ws[:65536].view(torch.int32).abs().max()) == 0   # the counter block is back at zero
+
+
 def test_one_pass_is_for_more_than_32_rows():
     from slimkernels_amd.torch import w4 as tw4
     big = dict(N=14336, K=4096, group_size=128)
