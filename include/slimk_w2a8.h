@@ -104,7 +104,7 @@ size_t slimk_w2a8_repacked_zp_bytes(int N, int K, int group_size);
  * and the workspace bytes a given split needs (0 when split_k <= 1).  Both kernels can split K:
  * the skinny one when few strips leave CUs idle (and for 17..32 token rows on matrices of 24 MiB
  * or more, where workgroups of four strips share the activations), the tiled one when its 64-row tiles
- * alone would leave CUs idle or unevenly loaded (up to eight splits of at least four 128-element stages each).
+ * alone would leave CUs idle or unevenly loaded (up to eight splits of at least 1024 elements of K each).
  * Split results are deterministic (partials are added in split order)
  * but their fp32 summation order differs from the unsplit one.
  * No upstream counterpart: upstream has no split-K launcher (the idea appears only in
