@@ -4,8 +4,8 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include <algorithm>
 #include <atomic>
-
 #include <mutex>
 #include <string>
 
@@ -138,25 +138,24 @@ int auto_split(int M, int N, int K, int group_size, int kernel) {
     return skinny_plain_split(N, K, group_size);
 }
 
+// K splits of the one-strip skinny kernel, from a sweep of waves x splits on eleven shapes at 1, 4 and 16 token rows:
+// a split costs its workgroups a round trip through the workspace (about 0.8 us), so it pays only for long reductions
+// (128 steps and more); never more workgroups than CUs, and every wave of a part keeps a chunk of four steps.
 int skinny_plain_split(int N, int K, int group_size) {
     const int strips = strips_of(N);
     const int G = K / group_size;
-    const int chunks = (K / 64 + 3) / 4;
-    const size_t weight_bytes = (size_t)strips * 64 * (K / 4);
+    const int steps = K / 64;
     int split = 1;
-    if (strips <= 128 && weight_bytes > (size_t)6 << 20) split = 256 / strips;  // never more workgroups than CUs
-    const int max_split = chunks / 4 > 0 ? chunks / 4 : 1;
-    if (split > max_split) split = max_split;
+    if (strips <= 128 && steps >= 128) split = std::min(256 / strips, steps / 32);
     if (split > 32) split = 32;
     const int gps = groups_per_split(G, group_size, split);
     return (G + gps - 1) / gps;
 }
 
-// Wavefronts per workgroup of the skinny kernel (the in-workgroup split of K): split runs are the
-// long-K ones, more waves per workgroup keep more loads in flight per CU.  An unsplit matrix of
-// up to 16 MiB with at most four token rows is bound by latency: eight waves per strip instead of
-// four shorten each wave's run (measured 5.09 -> 4.72 us at 4096 x 4096, M = 1; larger matrices
-// and more rows lose).
+// Wavefronts per workgroup of the skinny kernel (the in-workgroup split of K).  Split runs: eight (sixteen measured
+// 3..9 % slower on every split shape of the sweep).  An unsplit matrix of up to 16 MiB with at most four token rows is
+// bound by latency: eight waves per strip instead of four shorten each wave's run (measured 5.09 -> 4.72 us at
+// 4096 x 4096, M = 1; larger matrices and more rows lose).
 // slimk_w2a8_gemm_fused: up to four rows of at most 32 KiB of int8 values together are quantised by every workgroup for
 // itself into LDS; more rows (up to 32) or longer ones by the grid's first workgroups into the workspace.
 bool fused_in_workgroup(int M, int K) { return M <= w2a8::kFusedMaxRows && (size_t)M * K <= (size_t)w2a8::kFusedMaxBytes; }
@@ -168,7 +167,7 @@ size_t fused_rows_area_bytes(int K, int G) {  // int8 rows, 32 token scales, gro
 std::atomic<int> g_rows_spin_limit{20000};
 
 int skinny_waves(int M, int N, int K, int split) {
-    if (split > 1) return 16;
+    if (split > 1) return 8;
     const size_t weight_bytes = (size_t)strips_of(N) * 64 * (K / 4);
     return M <= 4 && weight_bytes <= ((size_t)16 << 20) && K >= 2048 ? 8 : 4;
 }
