@@ -74,8 +74,8 @@ enum slimk_dtype { SLIMK_F16 = 0, SLIMK_BF16 = 1 };
 
 /* which GEMM kernel slimk_w2a8_gemm runs */
 enum slimk_kernel {
-    SLIMK_KERNEL_AUTO = 0,   /* skinny for M <= 32 and for 33..256 rows on short reductions (K <= 4096) over small and
-                                medium matrices (passes over the weights under 100 MiB in all), tiled otherwise */
+    SLIMK_KERNEL_AUTO = 0,   /* skinny for M <= 32; for 33..256 rows whichever of the two skinny forms and the tiled
+                                kernel is predicted the fastest (slimk_w2a8_gemm_auto_route tells which); tiled beyond */
     SLIMK_KERNEL_SKINNY = 1, /* weight-streaming split-K kernel, M <= 256 (16 rows per pass over the weights) */
     SLIMK_KERNEL_TILED = 2   /* LDS-pipelined MFMA tile kernel, any M */
 };
@@ -111,6 +111,13 @@ size_t slimk_w2a8_repacked_zp_bytes(int N, int K, int group_size);
  * slimkernels/triton/gemm_splitk.ipynb cell 0). */
 int slimk_w2a8_gemm_auto_split_k(int M, int N, int K, int group_size, int kernel);
 size_t slimk_w2a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int kernel, int split_k);
+
+/* Which kernel form SLIMK_KERNEL_AUTO takes for this problem: 1 = skinny, one 64-channel strip per workgroup;
+ * 2 = tiled; 3 = skinny, workgroups of four strips that share the activations (17..32 token rows on matrices of
+ * 24 MiB or more, and the problems of 33..256 rows for which it is predicted the fastest of the three).
+ * 0 for a shape the library does not take.  A query for tests and tuning; no upstream counterpart (upstream's
+ * launcher has one kernel with one fixed tiling, slimkernels/cute/gemm/wgmma_sm90_W2A8.cu:448-450). */
+int slimk_w2a8_gemm_auto_route(int M, int N, int K, int group_size);
 
 /* ---- device work ------------------------------------------------------------------------ */
 

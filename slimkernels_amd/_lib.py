@@ -27,6 +27,7 @@ SIGNATURES = {
     "slimk_w2a8_repacked_zp_bytes": (_sz, [_i, _i, _i]),
     "slimk_w2a8_gemm_auto_split_k": (_i, [_i, _i, _i, _i, _i]),
     "slimk_w2a8_gemm_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
+    "slimk_w2a8_gemm_auto_route": (_i, [_i, _i, _i, _i]),
     "slimk_w2a8_workspace_init": (_i, [_vp, _sz, _vp]),
     "slimk_w2a8_repack": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "slimk_w2a8_quantize_weight": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp]),

@@ -70,22 +70,7 @@ int strips_of(int N) { return (N + w2a8::kStripN - 1) / w2a8::kStripN; }
 constexpr size_t kCounterBlockBytes = w2a8::kCounterBlockBytes;
 constexpr int kMaxCounters = w2a8::kMaxSplitCounters;  // (the block's last two slots belong to the row-quantising kernels)
 
-// The skinny kernel takes any number of token rows (16 at a time, the passes side by side as workgroups of their
-// own, each re-reading the weights, all but the first out of L2).  Measured against the tiled kernel on 33..256 rows: it wins while the reduction is short
-// (K <= 4096: the tiled kernel's few stages do not amortise its start-up) and the passes over the weights stay under
-// about 100 MiB in all (14336 x 4096: up to 96 rows, 11008 x 4096: up to 160, 4096 x 4096: 15.1 -> 6.3 us at 33 rows, 15.9 -> 9.6 us at 128;
-// two row blocks per wave, which halve the passes, lose at the small sizes and gain under 10 % at the large ones).
 constexpr int kSkinnyMaxRows = 256;
-bool skinny_wins_mid(int M, int N, int K) {
-    if (M <= 32 || M > kSkinnyMaxRows || K > 4096) return false;
-    const size_t weight_bytes = (size_t)strips_of(N) * 64 * (K / 4);
-    return (size_t)((M + 15) / 16) * weight_bytes <= ((size_t)100 << 20);
-}
-
-int resolve_kernel(int M, int N, int K, int kernel) {
-    if (kernel == SLIMK_KERNEL_AUTO) return M <= 32 || skinny_wins_mid(M, N, K) ? SLIMK_KERNEL_SKINNY : SLIMK_KERNEL_TILED;
-    return kernel;
-}
 
 // The skinny kernel partitions K in chunks of four 64-element steps; a split owns whole chunks.
 int chunk_groups(int group_size) { return group_size >= 256 ? 1 : 256 / group_size; }
@@ -98,16 +83,11 @@ int groups_per_split(int G, int group_size, int split) {
     return (gps + cg - 1) / cg * cg;
 }
 
-// One problem with 17..32 token rows on a matrix big enough to be bound by bandwidth goes through
-// the shared-activation workgroups (eight waves = two k-parts x four strips whose waves fetch the
-// activations once): 8..27 % faster there than one strip per workgroup (at 16 rows and below the
-// one-strip kernel is as fast or faster).  K is split across workgroups until about 256 exist, as
-// long as a wave keeps at least six chunks of four steps.
+// The shared-activation workgroups (eight waves = two k-parts x four strips whose waves fetch the activations once)
+// as a launch of one problem: K is split across workgroups until about 256 exist, as long as a wave keeps at least
+// six chunks of four steps.
 constexpr size_t kSharedMinWeightBytes = (size_t)24 << 20;
 constexpr int kSharedParts = w2a8::kSharedParts;
-bool skinny_shared_applies(int M, int N, int K) {
-    return M > 16 && M <= 32 && (size_t)strips_of(N) * 64 * (K / 4) >= kSharedMinWeightBytes;
-}
 int skinny_shared_split(int M, int N, int K, int group_size) {
     const int per_unit = w2a8::kGroupedWavesPerWg / kSharedParts;
     const int units = (strips_of(N) + per_unit - 1) / per_unit * ((M + 15) / 16);
@@ -118,24 +98,6 @@ int skinny_shared_split(int M, int N, int K, int group_size) {
     const int G = K / group_size;
     const int gps = groups_per_split(G, group_size, split);
     return (G + gps - 1) / gps;
-}
-
-// Split-K heuristic of the skinny kernel (measured on MI355X, cold weights).  One workgroup per
-// 64-channel strip covers at least half the CUs when there are more than 128 strips, and a matrix of a few
-// MiB is latency-bound whatever is done, so both run unsplit: the cross-workgroup reduction
-// costs about 3 us.  Only a large matrix with few strips (small N, long K) is split, up to about
-// 256 workgroups, because a quarter of the CUs cannot pull full HBM bandwidth - and never beyond:
-// with more workgroups than CUs some CUs carry two (5120 x 13824, 80 strips: 8.2 us at split 3,
-// 11.6 us at split 4).
-int skinny_plain_split(int N, int K, int group_size);
-int auto_split(int M, int N, int K, int group_size, int kernel) {
-    if (kernel != SLIMK_KERNEL_SKINNY) {
-        // the fast tiled kernel splits K when its tiles would leave CUs idle (groups of up to 256)
-        if (group_size > 256) return 1;
-        return w2a8::tiled_fast_auto_split(M, strips_of(N), K / w2a8::kStepK, group_size / w2a8::kStepK);
-    }
-    if (skinny_shared_applies(M, N, K)) return skinny_shared_split(M, N, K, group_size);
-    return skinny_plain_split(N, K, group_size);
 }
 
 // K splits of the one-strip skinny kernel, from a sweep of waves x splits on eleven shapes at 1, 4 and 16 token rows:
@@ -150,6 +112,85 @@ int skinny_plain_split(int N, int K, int group_size) {
     if (split > 32) split = 32;
     const int gps = groups_per_split(G, group_size, split);
     return (G + gps - 1) / gps;
+}
+
+// 33..256 token rows: three kernels can take the problem.
+//   plain  - the one-strip skinny kernel, 16 rows at a time, the passes side by side as workgroups of their own (each
+//            re-reading weights and activations, all but the first out of L2): the fastest while the workgroups are
+//            few (4096 x 4096: 5.6 us at 33 rows, tiled 17.3).
+//   shared - the shared-activation workgroups (four strips x two k-parts fetch a row block's activations once): a
+//            quarter of the plain kernel's workgroups at a higher cost each (11008 x 4096 at 80 rows: 13.5 us, plain
+//            16.0, tiled 20.8; 4096 x 11008 at 33..80 rows: 15.1..15.4 us, tiled 20.1..25.7, plain 15.6..21.4).
+//   tiled  - 64 x 256 tiles through LDS: the cheapest per row once the rows fill its tiles and the reduction is long
+//            enough to amortise its start-up.
+// The choice is the smallest of three predicted times.  Each prediction is a start-up cost, a cost of splitting K
+// across workgroups, and rounds of 256 workgroups (one per CU) times a cost per round that grows with the steps a
+// workgroup (plain, tiled) or a wave (shared) runs through; plain and shared also pay for the weights' first trip
+// from HBM.  The coefficients are a least-squares fit (on the logarithm of predicted / measured) to timings of all
+// three kernels on 23 matrices (1024..28672 channels, K = 3072..28672) at 33, 48, 64, 80, 96, 128, 160 and 256 rows,
+// weights streamed from HBM: picking by the prediction costs 1.1 % over the best kernel of each case on average
+// (worst case 33 %; the rule by size it replaces: 4.2 % on the same cases and up to 85 %).
+// Reductions of up to 2048 elements keep the rule they were measured with (plain while its passes over the weights
+// stay under 100 MiB).
+enum MidRoute { kMidPlain, kMidShared, kMidTiled };
+MidRoute mid_route(int M, int N, int K, int group_size) {
+    if (M > kSkinnyMaxRows) return kMidTiled;
+    const int strips = strips_of(N), steps = K / w2a8::kStepK, blocks = (M + 15) / 16;
+    const size_t weight_bytes = (size_t)strips * 64 * (K / 4);
+    if (K <= 2048) return (size_t)blocks * weight_bytes <= ((size_t)100 << 20) ? kMidPlain : kMidTiled;
+    if (K > 4096 && weight_bytes > ((size_t)32 << 20)) return kMidTiled;  // (28672 x 8192: tiled ahead at every row count)
+    const float weight_mib = (float)weight_bytes / 1048576.0f;
+    const auto rounds = [](long long wgs, float smooth) {  // between whole rounds and the plain ratio
+        const float whole = (float)((wgs + 255) / 256), ratio = std::max(1.0f, (float)wgs / 256.0f);
+        return smooth * ratio + (1.0f - smooth) * whole;
+    };
+    const int plain_split = skinny_plain_split(N, K, group_size);
+    const float plain_cost = 1.786f + (plain_split > 1 ? 3.684f : 0.0f) + 0.1085f * weight_mib +
+                             rounds((long long)strips * plain_split * blocks, 0.475f) * (1.050f + 0.0369f * (float)steps / (float)plain_split);
+    const int shared_split = skinny_shared_split(M, N, K, group_size);
+    const int units = (strips + 3) / 4 * blocks;
+    const float shared_cost = 5.066f + (shared_split > 1 ? 2.920f : 0.0f) + 0.1165f * weight_mib +
+                              rounds((long long)units * shared_split, 0.386f) * (-1.437f + 0.2702f * (float)steps / (2.0f * (float)shared_split));
+    float tiled_cost = 1e30f;
+    if (group_size <= 256) {
+        const int gs = group_size / w2a8::kStepK;
+        const int tiled_split = w2a8::tiled_fast_auto_split(M, strips, steps, gs);
+        const int tiles = (int)w2a8::tiled_fast_workspace_tiles(M, strips, gs);
+        const int stages = (steps + 1) / 2;
+        const int per = (stages + tiled_split - 1) / tiled_split;
+        const int n = (tiles * tiled_split + 255) / 256;  // workgroups per CU: up to three run side by side
+        const float together = n == 1 ? 1.0f : (n == 2 ? 1.424f : (n == 3 ? 1.860f : 0.608f * (float)n));
+        tiled_cost = -10.21f + (tiled_split > 1 ? 6.384f : 0.0f) +
+                     ((float)per + 23.97f) * 0.6773f * together * (group_size == 64 ? 1.184f : 1.0f);
+    }
+    if (plain_cost <= shared_cost && plain_cost <= tiled_cost) return kMidPlain;
+    return shared_cost <= tiled_cost ? kMidShared : kMidTiled;
+}
+
+int resolve_kernel(int M, int N, int K, int group_size, int kernel) {
+    if (kernel == SLIMK_KERNEL_AUTO)
+        return M <= 32 || mid_route(M, N, K, group_size) != kMidTiled ? SLIMK_KERNEL_SKINNY : SLIMK_KERNEL_TILED;
+    return kernel;
+}
+
+// One problem with 17..32 token rows on a matrix big enough to be bound by bandwidth goes through the shared-activation
+// workgroups: 8..27 % faster there than one strip per workgroup (at 16 rows and below the one-strip kernel is as fast
+// or faster); with more rows, where mid_route says so (a request for the skinny kernel where the tiled one is
+// predicted ahead takes the faster of the two skinny forms).
+bool skinny_shared_applies(int M, int N, int K, int group_size) {
+    if (M <= 16 || M > kSkinnyMaxRows) return false;
+    if (M <= 32) return (size_t)strips_of(N) * 64 * (K / 4) >= kSharedMinWeightBytes;
+    return mid_route(M, N, K, group_size) == kMidShared;
+}
+
+int auto_split(int M, int N, int K, int group_size, int kernel) {
+    if (kernel != SLIMK_KERNEL_SKINNY) {
+        // the fast tiled kernel splits K when its tiles would leave CUs idle (groups of up to 256)
+        if (group_size > 256) return 1;
+        return w2a8::tiled_fast_auto_split(M, strips_of(N), K / w2a8::kStepK, group_size / w2a8::kStepK);
+    }
+    if (skinny_shared_applies(M, N, K, group_size)) return skinny_shared_split(M, N, K, group_size);
+    return skinny_plain_split(N, K, group_size);
 }
 
 // Wavefronts per workgroup of the skinny kernel (the in-workgroup split of K).  Split runs: eight (sixteen measured
@@ -197,12 +238,18 @@ size_t slimk_w2a8_repacked_zp_bytes(int N, int K, int group_size) {
 
 int slimk_w2a8_gemm_auto_split_k(int M, int N, int K, int group_size, int kernel) {
     if (M <= 0 || N <= 0 || !shape_ok(K, group_size)) return 0;
-    return auto_split(M, N, K, group_size, resolve_kernel(M, N, K, kernel));
+    return auto_split(M, N, K, group_size, resolve_kernel(M, N, K, group_size, kernel));
+}
+
+int slimk_w2a8_gemm_auto_route(int M, int N, int K, int group_size) {
+    if (M <= 0 || N <= 0 || !shape_ok(K, group_size)) return 0;
+    if (resolve_kernel(M, N, K, group_size, SLIMK_KERNEL_AUTO) == SLIMK_KERNEL_TILED) return 2;
+    return skinny_shared_applies(M, N, K, group_size) ? 3 : 1;
 }
 
 size_t slimk_w2a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int kernel, int split_k) {
     if (M <= 0 || N <= 0 || !shape_ok(K, group_size)) return 0;
-    const int kern = resolve_kernel(M, N, K, kernel);
+    const int kern = resolve_kernel(M, N, K, group_size, kernel);
     if (split_k <= 0) split_k = auto_split(M, N, K, group_size, kern);
     if (split_k <= 1) return 0;
     const int strips = strips_of(N);
@@ -313,7 +360,7 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
     if (M <= 0 || N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "M=%d, N=%d must be positive", M, N);
     if (int rc = check_kg(K, group_size)) return rc;
     // the row sums fold zero-points; the fast tiled kernel centres its operand bytes on 2 and reads none for that value
-    const bool rowsum_unused = !zp_r && zp_const == 2 && resolve_kernel(M, N, K, kernel) == SLIMK_KERNEL_TILED &&
+    const bool rowsum_unused = !zp_r && zp_const == 2 && resolve_kernel(M, N, K, group_size, kernel) == SLIMK_KERNEL_TILED &&
                                group_size <= 256;
     if (!rowsum && !rowsum_unused)
         return fail(SLIMK_ERR_NULL_POINTER, "gemm: rowsum is NULL (only the tiled kernel with the uniform zero-point 2 and a group size of at most 256 does without)");
@@ -330,7 +377,7 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
         return fail(SLIMK_ERR_MISALIGNED, "gemm: q, rowsum, w_r, s_r, zp_r must be 16-byte aligned; ldq %% 16 == 0; ldr %% 4 == 0");
     if ((reinterpret_cast<uintptr_t>(out) & 1u) != 0) return fail(SLIMK_ERR_MISALIGNED, "gemm: out must be 2-byte aligned");
 
-    const int kern = resolve_kernel(M, N, K, kernel);
+    const int kern = resolve_kernel(M, N, K, group_size, kernel);
     if (kern == SLIMK_KERNEL_SKINNY && M > kSkinnyMaxRows)
         return fail(SLIMK_ERR_UNSUPPORTED, "the skinny kernel handles M <= %d (M=%d)", kSkinnyMaxRows, M);
     const int G = K / group_size;
@@ -396,7 +443,7 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
     const bool out_bf16 = out_dtype == SLIMK_BF16;
     // a call with a dump runs the verification instantiation of the kernel the same call without one would run
     const bool dump = p.acc_dump != nullptr;
-    if (kern == SLIMK_KERNEL_SKINNY && skinny_shared_applies(M, N, K))
+    if (kern == SLIMK_KERNEL_SKINNY && skinny_shared_applies(M, N, K, group_size))
         return hip_result(dump ? w2a8::launch_skinny_shared_verify(p, gs, asym, out_bf16, st)
                                : w2a8::launch_skinny_shared(p, gs, asym, out_bf16, st), "shared skinny gemm");
     if (kern == SLIMK_KERNEL_SKINNY)

@@ -68,6 +68,21 @@ def test_split_heuristic_and_workspace(L):
     assert L.slimk_w2a8_gemm_auto_split_k(0, 4096, 4096, 128, 0) == 0
 
 
+def test_auto_route(L):
+    """Which kernel form AUTO takes: 1 one-strip skinny, 2 tiled, 3 shared-activation skinny."""
+    route = L.slimk_w2a8_gemm_auto_route
+    assert route(1, 4096, 4096, 128) == 1 and route(16, 28672, 8192, 64) == 1
+    assert route(20, 4096, 4096, 128) == 1          # 17..32 rows: shared only on matrices of 24 MiB or more
+    assert route(20, 8192, 14336, 128) == 3
+    assert route(33, 4096, 4096, 128) == 1          # few workgroups: the one-strip kernel
+    assert route(77, 11008, 4096, 128) == 3         # five row blocks on 172 strips: the shared-activation workgroups
+    assert route(64, 4096, 14336, 128) == 3         # long reduction, few 256-channel tiles
+    assert route(128, 28672, 8192, 64) == 2
+    assert route(257, 4096, 4096, 128) == 2 and route(2048, 4096, 4096, 128) == 2
+    assert route(100, 14336, 2048, 128) in (1, 2)   # reductions of up to 2048 never take the shared form
+    assert route(0, 4096, 4096, 128) == 0 and route(16, 4096, 4000, 128) == 0 and route(16, 4096, 4096, 96) == 0
+
+
 def _gemm(L, **kw):
     a = dict(q=FAKE, ldq=4096, s_a=FAKE, rowsum=FAKE, ldr=16, w_r=FAKE, s_r=FAKE, zp_r=None, zp_const=2,
              M=16, N=4096, K=4096, g=128, out=FAKE, ldo=4096, odt=0, acc=None, dump=0, ws=None, wsb=0,

@@ -250,6 +250,24 @@ def test_skinny_shared_one_problem(gpu_ops, oracle, M, N, K, g, mode, out, split
     _run_case(gpu_ops, oracle, case, "skinny", split_k=split, dump="sum")
 
 
+@pytest.mark.parametrize("M,N,K,g,mode,out,split", [
+    (100, 6200, 2304, 64, "asym", "bfloat16", 0),   # short reduction: seven row blocks, the last ragged, ragged last strip
+    (130, 1000, 12288, 128, "sym", "float16", 0),   # long reduction, few strips: nine row blocks, K split across workgroups
+    (33, 4000, 12288, 256, "ref", "float16", 0),    # the third row block holds one row
+    (50, 4000, 12288, 128, "sym", "float16", 2),    # explicit split
+    (250, 3000, 2304, 128, "asym", "float16", 0),   # sixteen row blocks
+])
+def test_skinny_shared_more_than_32_rows(gpu_ops, oracle, M, N, K, g, mode, out, split):
+    """33..256 token rows where the library sends them through the shared-activation workgroups (one workgroup per
+    four strips and block of 16 rows): int32 sums exact, the output criterion, and the library's own choice of kernel
+    is that form (should the choice move, pick cases that it still sends there)."""
+    from slimkernels_amd import _lib
+    assert _lib.lib().slimk_w2a8_gemm_auto_route(M, N, K, g) == 3
+    case = pu.small_case(M, N, K, g, mode, seed=M + N + K, out_dtype=out)
+    _run_case(gpu_ops, oracle, case, "auto", split_k=split, dump="sum")
+    _run_case(gpu_ops, oracle, case, "skinny", split_k=split)
+
+
 @pytest.mark.parametrize("M,N,K,g,mode,out", SMALL + [
     (77, 200, 512, 128, "asym", "float16"),
     (129, 130, 320, 64, "sym", "float16"),
