@@ -123,16 +123,20 @@ def main():
         if grouped:
             ops.w2a8_gemm_grouped(probs, torch.float16)
 
-    # touch every copy once eagerly: creates and zeroes the split-K workspaces outside any capture
-    for sh in shapes.values():
-        for w in sh.copies:
-            _, qa, out = acts[(sh.N, sh.K, 16)]
-            ops.w2a8_gemm(qa, w, torch.float16, out=out)
+    # Every capture in this file records on one stream of its own, and what is captured runs eagerly on that stream
+    # first: the wrapper keeps a split-K workspace per (weight, stream), so the workspaces exist before the capture
+    # and no allocation or counter fill ends up inside a graph.
+    cap_stream = _capture_stream(torch)
+    with torch.cuda.stream(cap_stream):
+        for c in cases:
+            _, qa, out = acts[(c.N, c.K, c.M)]
+            for w in shapes[name_of[(c.N, c.K)]].copies:
+                ops.w2a8_gemm(qa, w, torch.float16, out=out)
     torch.cuda.synchronize()
 
     def capture(n_steps, warm=False, grouped=True):
         g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
+        with torch.cuda.graph(g, stream=cap_stream):
             for _ in range(n_steps):
                 launch_step(warm, grouped)
         return g
@@ -279,10 +283,23 @@ def _lib_check(rc):
     _lib.check(rc)
 
 
+_CAPTURE_STREAM = []
+
+
+def _capture_stream(torch):
+    if not _CAPTURE_STREAM:
+        _CAPTURE_STREAM.append(torch.cuda.Stream())
+    return _CAPTURE_STREAM[0]
+
+
 def time_graph(torch, fn, launches_in_graph, replays=6):
     """Mean microseconds per launch of `fn` (which enqueues `launches_in_graph` launches)."""
+    s = _capture_stream(torch)
+    with torch.cuda.stream(s):  # eagerly first, on the capturing stream: per-stream workspaces come to exist here
+        fn()
+    torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
+    with torch.cuda.graph(g, stream=s):
         fn()
     g.replay()
     torch.cuda.synchronize()

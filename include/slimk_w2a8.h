@@ -126,7 +126,10 @@ int slimk_w2a8_gemm_auto_route(int M, int N, int K, int group_size);
  * partial tiles.  Every GEMM leaves the counters it used at zero again when it finishes, and the counter block
  * never moves, so one initialisation serves any number of later calls of any shapes and kernels (2-bit, 4-bit
  * one-pass, fused) that use the workspace one at a time; calls that overlap in time (different streams) need
- * a workspace each. */
+ * a workspace each.  Only the counter block has to start at zero (the partial tiles are written before they are
+ * read): passing min(workspace_bytes, SLIMK_W2A8_COUNTER_BLOCK_BYTES) here is enough and spares the fill of a
+ * large workspace. */
+#define SLIMK_W2A8_COUNTER_BLOCK_BYTES (64u << 10)
 int slimk_w2a8_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 
 /* Re-lay the interchange format into the gfx950 streaming layout.

@@ -52,6 +52,7 @@ SIGNATURES = {
     "slimk_w2a8_read_probe": (_i, [_vp, _sz, _vp, _vp]),
 }
 MAX_GROUP = 24
+COUNTER_BLOCK_BYTES = 64 << 10  # SLIMK_W2A8_COUNTER_BLOCK_BYTES
 
 
 class Problem(ctypes.Structure):

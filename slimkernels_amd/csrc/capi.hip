@@ -68,6 +68,7 @@ int strips_of(int N) { return (N + w2a8::kStripN - 1) / w2a8::kStripN; }
 // with the shape, a workspace zeroed once stays valid for any sequence of problems (a counter block sized by the
 // problem would let a later, larger block overlap an earlier call's partial sums).
 constexpr size_t kCounterBlockBytes = w2a8::kCounterBlockBytes;
+static_assert(kCounterBlockBytes == SLIMK_W2A8_COUNTER_BLOCK_BYTES, "the header names the counter block's size");
 constexpr int kMaxCounters = w2a8::kMaxSplitCounters;  // (the block's last two slots belong to the row-quantising kernels)
 
 constexpr int kSkinnyMaxRows = 256;

@@ -189,7 +189,8 @@ def _workspace(w: W2A8Weight, nbytes: int) -> Optional[torch.Tensor]:
     ws = w.workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
-        _lib.check(_lib.lib().slimk_w2a8_workspace_init(ws.data_ptr(), ws.numel(), key))
+        # only the arrival counters at its start have to be zero; the partial tiles are written before they are read
+        _lib.check(_lib.lib().slimk_w2a8_workspace_init(ws.data_ptr(), min(ws.numel(), _lib.COUNTER_BLOCK_BYTES), key))
         w.workspaces[key] = ws
     return ws
 
