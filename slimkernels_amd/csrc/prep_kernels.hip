@@ -106,13 +106,27 @@ __device__ __forceinline__ void load8(const uint16_t* p, float (&v)[8]) {
     }
 }
 
+// Row of a workgroup.  rowsum is [group][row]: a row's sums are 4 bytes each, a cache line of 128 bytes holds those
+// of 32 consecutive rows.  Workgroup ids go round the eight XCDs, each with an L2 of its own, so with row = id the 32
+// writers of a line sit on all eight L2s and the line goes to memory in pieces (a fifth of the kernel's time at
+// 4096 x 14336: 8 of 43.6 us).  With blocks of 32 consecutive rows dealt to the XCDs instead, a line is put together
+// in one L2.  The grid is rounded up to whole sets of 256 rows; ids whose row is past the end do nothing.
+__device__ __forceinline__ int act_quant_row(int id, bool by_xcd) {
+    if (!by_xcd) return id;
+    const int xcd = id & 7, k = id >> 3;
+    return (((k >> 5) << 3) + xcd) * 32 + (k & 31);
+}
+constexpr int kRowsByXcd = 256;  // from this many rows on
+static int act_quant_grid(int M) { return M >= kRowsByXcd ? (M + 255) / 256 * 256 : M; }
+
 template <bool BF16>
-__global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restrict__ x, int ldx, int K,
+__global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restrict__ x, int ldx, int M, int K,
                                                         int group_size, int8_t* __restrict__ q, int ldq,
                                                         float* __restrict__ s_a,
                                                         int32_t* __restrict__ rowsum, int ldr, int copies) {
     __shared__ float red[4];
-    const int m = blockIdx.x;
+    const int m = act_quant_row(blockIdx.x, M >= kRowsByXcd);
+    if (m >= M) return;  // (uniform: the grid is rounded up to whole sets of rows)
     const int tid = threadIdx.x;
     const uint16_t* xr = x + (size_t)m * ldx;
     const int nvec = K / 8;
@@ -174,12 +188,13 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
 // divisions (a dozen instructions each) were most of that arithmetic: rne_quotient() (w2a8_common.h) avoids nearly
 // all of them (32 rows x 28672: 8.2 -> 7.2 us; 4096 x 4096: 17.6 -> 15.2 us).
 template <bool BF16, int KEEP, int THREADS = 256>
-__global__ __launch_bounds__(THREADS) void act_quant_keep_kernel(const uint16_t* __restrict__ x, int ldx, int K,
+__global__ __launch_bounds__(THREADS) void act_quant_keep_kernel(const uint16_t* __restrict__ x, int ldx, int M, int K,
                                                              int group_size, int8_t* __restrict__ q, int ldq,
                                                              float* __restrict__ s_a,
                                                              int32_t* __restrict__ rowsum, int ldr, int copies) {
     __shared__ float red[THREADS / 64];
-    const int m = blockIdx.x;
+    const int m = act_quant_row(blockIdx.x, M >= kRowsByXcd);
+    if (m >= M) return;  // (uniform: the grid is rounded up to whole sets of rows)
     const int tid = threadIdx.x;
     const uint16_t* xr = x + (size_t)m * ldx;
     const int nvec = K / 8;
@@ -241,27 +256,27 @@ constexpr int kFewRows = 64;  // up to this many rows a long row gets 1024 threa
 template <bool BF16>
 static void launch_act_quant_keep(const void* x, int ldx, int M, int K, int group_size, int8_t* q, int ldq, float* s_a,
                                   int32_t* rowsum, int ldr, int copies, hipStream_t stream) {
-    const dim3 grid((unsigned)M), block(256);
+    const dim3 grid((unsigned)act_quant_grid(M)), block(256);
     if (M <= kFewRows && K > 2048 && K <= 4096) {  // a few rows: 512 threads a row, one vector each
-        act_quant_keep_kernel<BF16, 1, 512><<<grid, dim3(512), 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+        act_quant_keep_kernel<BF16, 1, 512><<<grid, dim3(512), 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
         return;
     }
     if (M <= kFewRows && K > 4096) {  // a few long rows: 1024 threads a row
         const dim3 wide(1024);
         if (K <= 8192)
-            act_quant_keep_kernel<BF16, 1, 1024><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+            act_quant_keep_kernel<BF16, 1, 1024><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
         else if (K <= 16384)
-            act_quant_keep_kernel<BF16, 2, 1024><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+            act_quant_keep_kernel<BF16, 2, 1024><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
         else
-            act_quant_keep_kernel<BF16, 4, 1024><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+            act_quant_keep_kernel<BF16, 4, 1024><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
         return;
     }
     if (K <= 4096)
-        act_quant_keep_kernel<BF16, 2><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+        act_quant_keep_kernel<BF16, 2><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
     else if (K <= 8192)
-        act_quant_keep_kernel<BF16, 4><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+        act_quant_keep_kernel<BF16, 4><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
     else
-        act_quant_keep_kernel<BF16, 8><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+        act_quant_keep_kernel<BF16, 8><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
 }
 
 hipError_t launch_act_quant(const void* x, int ldx, bool x_bf16, int M, int K, int group_size,
@@ -272,10 +287,10 @@ hipError_t launch_act_quant(const void* x, int ldx, bool x_bf16, int M, int K, i
         return hipGetLastError();
     }
     if (x_bf16)
-        act_quant_kernel<true><<<dim3(M), dim3(256), 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q,
+        act_quant_kernel<true><<<dim3(act_quant_grid(M)), dim3(256), 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q,
                                                                  ldq, s_a, rowsum, ldr, copies);
     else
-        act_quant_kernel<false><<<dim3(M), dim3(256), 0, stream>>>((const uint16_t*)x, ldx, K, group_size, q,
+        act_quant_kernel<false><<<dim3(act_quant_grid(M)), dim3(256), 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q,
                                                                   ldq, s_a, rowsum, ldr, copies);
     return hipGetLastError();
 }
