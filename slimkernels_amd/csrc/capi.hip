@@ -195,9 +195,10 @@ int auto_split(int M, int N, int K, int group_size, int kernel) {
 }
 
 // Wavefronts per workgroup of the skinny kernel (the in-workgroup split of K).  Split runs: eight (sixteen measured
-// 3..9 % slower on every split shape of the sweep).  An unsplit matrix of up to 16 MiB with at most four token rows is
-// bound by latency: eight waves per strip instead of four shorten each wave's run (measured 5.09 -> 4.72 us at
-// 4096 x 4096, M = 1; larger matrices and more rows lose).
+// 3..9 % slower on every split shape of the sweep).  Unsplit with at most four token rows and at most one workgroup
+// per CU (256 strips): eight waves per strip instead of four shorten each wave's run and put more loads in flight on
+// a CU (4096 x 4096, M = 1: 5.09 -> 4.72 us; 11008 x 8192: 8.3 -> 7.2 us; 12288 x 12288: 11.5 -> 9.8 us); with
+// more strips than CUs (28672 x 8192: 12.9 -> 14.4 us) and with more rows they lose.
 // slimk_w2a8_gemm_fused: up to four rows of at most 32 KiB of int8 values together are quantised by every workgroup for
 // itself into LDS; more rows (up to 32) or longer ones by the grid's first workgroups into the workspace.
 bool fused_in_workgroup(int M, int K) { return M <= w2a8::kFusedMaxRows && (size_t)M * K <= (size_t)w2a8::kFusedMaxBytes; }
@@ -210,8 +211,7 @@ std::atomic<int> g_rows_spin_limit{20000};
 
 int skinny_waves(int M, int N, int K, int split) {
     if (split > 1) return 8;
-    const size_t weight_bytes = (size_t)strips_of(N) * 64 * (K / 4);
-    return M <= 4 && weight_bytes <= ((size_t)16 << 20) && K >= 2048 ? 8 : 4;
+    return M <= 4 && strips_of(N) <= 256 && K >= 2048 ? 8 : 4;
 }
 
 }  // namespace

@@ -17,7 +17,7 @@ void rows_out(const GemmParams& p, bool out_bf16, int spin_limit, hipStream_t st
 // cache policy and activation fetch as launch_rows picks them for already quantised rows
 template <int GS, int NW, bool ASYM>
 void rows_shape(const GemmParams& p, bool out_bf16, int spin_limit, hipStream_t stream) {
-    const bool wide = p.M >= kWideRows && p.K >= kWideK;
+    const bool wide = p.M >= kWideRows && p.K >= kWideK && p.strips * max(p.split, 1) * NW * ((p.M + 15) / 16) >= kWideWaves;
     const bool once = p.M <= 16;  // one row block: every weight byte is used once
     if (once && !wide) rows_out<GS, NW, ASYM, true, false>(p, out_bf16, spin_limit, stream);
     else if (once) rows_out<GS, NW, ASYM, true, true>(p, out_bf16, spin_limit, stream);

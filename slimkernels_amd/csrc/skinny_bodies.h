@@ -1228,13 +1228,15 @@ static void launch_zm(const GemmParams& p, bool asym, bool out_bf16, hipStream_t
 }
 
 // Two-steps-wide activation fetch pays from 16 token rows on when the reduction is long (measured:
-// 5..15 % faster at K >= 8192, M = 16..32; the LDS turn costs a short problem more than the saved
-// cache-line slots bring).
-constexpr int kWideRows = 16, kWideK = 8192;
+// 4..15 % faster at K >= 8192, M = 16..32; the LDS turn costs a short problem more than the saved
+// cache-line slots bring) and the launch puts enough waves on a CU to hide that turn: with four waves or fewer per
+// CU (224 or 256 strips, unsplit, four waves each) it is 17..19 % slower (14336 x 8192 at 16 rows: 12.4 against
+// 10.1 us; 16384 x 16384: 21.9 against 18.1 us), with seven or more 4..5 % faster.
+constexpr int kWideRows = 16, kWideK = 8192, kWideWaves = 1536;
 
 template <int GS, int NW, bool DUMP>
 static void launch_rows(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
-    const bool wide = p.M >= kWideRows && p.K >= kWideK;
+    const bool wide = p.M >= kWideRows && p.K >= kWideK && p.strips * max(p.split, 1) * NW * ((p.M + 15) / 16) >= kWideWaves;
     if (p.M == 1) launch_zm<1, GS, NW, DUMP, true, false>(p, asym, out_bf16, stream);
     else if (p.M <= 16 && !wide) launch_zm<4, GS, NW, DUMP, true, false>(p, asym, out_bf16, stream);
     else if (p.M <= 16) launch_zm<4, GS, NW, DUMP, true, true>(p, asym, out_bf16, stream);
