@@ -95,6 +95,9 @@ int skinny_shared_split(int M, int N, int K, int group_size) {
     const int chunks = (K / 64 + 3) / 4;
     int split = (256 + units / 2) / units;
     if (split > chunks / (kSharedParts * 6)) split = chunks / (kSharedParts * 6);
+    // never a few workgroups more than CUs: they would run as a second round (12288 x 12288 at 17..32 rows, 96 units:
+    // 22.6 us at three splits, 20.1 us at two)
+    while (split > 1 && units * split > 256) --split;
     if (split < 1) split = 1;
     const int G = K / group_size;
     const int gps = groups_per_split(G, group_size, split);
