@@ -113,8 +113,9 @@ int slimk_w2a8_gemm_auto_split_k(int M, int N, int K, int group_size, int kernel
 size_t slimk_w2a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int kernel, int split_k);
 
 /* Which kernel form SLIMK_KERNEL_AUTO takes for this problem: 1 = skinny, one 64-channel strip per workgroup;
- * 2 = tiled; 3 = skinny, workgroups of four strips that share the activations (17..32 token rows on matrices of
- * 24 MiB or more, and the problems of 33..256 rows for which it is predicted the fastest of the three).
+ * 2 = tiled; 3 = skinny, workgroups of several strips that share the activations (12..16 token rows on 384 strips
+ * and more, 17..32 rows on matrices of 24 MiB or more, and the problems of 33..256 rows for which it is predicted
+ * the fastest of the three).
  * 0 for a shape the library does not take.  A query for tests and tuning; no upstream counterpart (upstream's
  * launcher has one kernel with one fixed tiling, slimkernels/cute/gemm/wgmma_sm90_W2A8.cu:448-450). */
 int slimk_w2a8_gemm_auto_route(int M, int N, int K, int group_size);

@@ -89,12 +89,20 @@ int groups_per_split(int G, int group_size, int split) {
 // six chunks of four steps.
 constexpr size_t kSharedMinWeightBytes = (size_t)24 << 20;
 constexpr int kSharedParts = w2a8::kSharedParts;
+// 12..16 rows on 384 strips and more take the form with four k-parts x two strips: one strip per workgroup leaves
+// 448 four-wave workgroups on 256 CUs, a quarter of the CUs with half the load, and every strip fetches the
+// activations for itself (28672 x 8192 at 14 / 16 rows: 18.9 / 18.8 -> 17.3 / 17.4 us, 28672 x 4096: 10.7 / 11.1 ->
+// 10.0 us, 32768 x 8192 at 12 rows: 18.2 -> 16.5 us; at 10 rows and below, and on 256 strips and fewer, the one-strip
+// kernel is ahead or level).
+constexpr int kWideSharedStrips = 384, kWideSharedRows = 12;
+int skinny_shared_parts(int M, int N) { return M <= 16 && strips_of(N) >= kWideSharedStrips ? 2 * kSharedParts : kSharedParts; }
 int skinny_shared_split(int M, int N, int K, int group_size) {
-    const int per_unit = w2a8::kGroupedWavesPerWg / kSharedParts;
+    const int parts = skinny_shared_parts(M, N);
+    const int per_unit = w2a8::kGroupedWavesPerWg / parts;
     const int units = (strips_of(N) + per_unit - 1) / per_unit * ((M + 15) / 16);
     const int chunks = (K / 64 + 3) / 4;
     int split = (256 + units / 2) / units;
-    if (split > chunks / (kSharedParts * 6)) split = chunks / (kSharedParts * 6);
+    if (split > chunks / (parts * 6)) split = chunks / (parts * 6);
     // never a few workgroups more than CUs: they would run as a second round (12288 x 12288 at 17..32 rows, 96 units:
     // 22.6 us at three splits, 20.1 us at two)
     while (split > 1 && units * split > 256) --split;
@@ -182,6 +190,7 @@ int resolve_kernel(int M, int N, int K, int group_size, int kernel) {
 // or faster); with more rows, where mid_route says so (a request for the skinny kernel where the tiled one is
 // predicted ahead takes the faster of the two skinny forms).
 bool skinny_shared_applies(int M, int N, int K, int group_size) {
+    if (M >= kWideSharedRows && M <= 16) return strips_of(N) >= kWideSharedStrips;
     if (M <= 16 || M > kSkinnyMaxRows) return false;
     if (M <= 32) return (size_t)strips_of(N) * 64 * (K / 4) >= kSharedMinWeightBytes;
     return mid_route(M, N, K, group_size) == kMidShared;
@@ -448,8 +457,8 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
     // a call with a dump runs the verification instantiation of the kernel the same call without one would run
     const bool dump = p.acc_dump != nullptr;
     if (kern == SLIMK_KERNEL_SKINNY && skinny_shared_applies(M, N, K, group_size))
-        return hip_result(dump ? w2a8::launch_skinny_shared_verify(p, gs, asym, out_bf16, st)
-                               : w2a8::launch_skinny_shared(p, gs, asym, out_bf16, st), "shared skinny gemm");
+        return hip_result(dump ? w2a8::launch_skinny_shared_verify(p, gs, skinny_shared_parts(M, N), asym, out_bf16, st)
+                               : w2a8::launch_skinny_shared(p, gs, skinny_shared_parts(M, N), asym, out_bf16, st), "shared skinny gemm");
     if (kern == SLIMK_KERNEL_SKINNY)
         return hip_result(dump ? w2a8::launch_skinny_verify(p, gs, skinny_waves(M, N, K, split_k), asym, out_bf16, st)
                                : w2a8::launch_skinny(p, gs, skinny_waves(M, N, K, split_k), asym, out_bf16, st), "skinny gemm");

@@ -40,8 +40,8 @@ hipError_t launch_skinny(const GemmParams& p, int gs, int waves, bool asym, bool
     return launch_skinny_impl<false>(p, gs, waves, asym, out_bf16, stream);
 }
 
-hipError_t launch_skinny_shared(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream) {
-    return launch_skinny_shared_impl<false>(p, gs, asym, out_bf16, stream);
+hipError_t launch_skinny_shared(const GemmParams& p, int gs, int kparts, bool asym, bool out_bf16, hipStream_t stream) {
+    return launch_skinny_shared_impl<false>(p, gs, kparts, asym, out_bf16, stream);
 }
 
 hipError_t launch_skinny_grouped(const GroupedParams& gp, int gs, bool asym, bool out_bf16, hipStream_t stream) {

@@ -16,8 +16,8 @@ hipError_t launch_skinny_verify(const GemmParams& p, int gs, int waves, bool asy
     return launch_skinny_verify_gs4(p, waves, asym, out_bf16, stream);
 }
 
-hipError_t launch_skinny_shared_verify(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream) {
-    return launch_skinny_shared_impl<true>(p, gs, asym, out_bf16, stream);
+hipError_t launch_skinny_shared_verify(const GemmParams& p, int gs, int kparts, bool asym, bool out_bf16, hipStream_t stream) {
+    return launch_skinny_shared_impl<true>(p, gs, kparts, asym, out_bf16, stream);
 }
 
 hipError_t launch_skinny_grouped_verify(const GroupedParams& gp, int gs, bool asym, bool out_bf16, hipStream_t stream) {

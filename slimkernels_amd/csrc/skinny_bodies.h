@@ -1174,8 +1174,9 @@ __global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_grouped_kernel(c
 
 // One problem through the shared-activation body: grid.x = sets of strips (in whole sets of eight per
 // row block, as in the grouped kernel), grid.y = K splits.  For 17..32 token rows on matrices big
-// enough to be bound by bandwidth (measured 8..27 % faster than one strip per workgroup there; at
-// 16 rows and below the one-strip kernel is as fast or faster).
+// enough to be bound by bandwidth (measured 8..27 % faster than one strip per workgroup there), for the problems of
+// 33..256 rows the host predicts it fastest for, and with four k-parts x two strips for 12..16 rows on very wide
+// matrices (more strips than the CUs take as one-strip workgroups at a time).
 template <int GS, int NK, bool ASYM, typename OutT, bool DUMP = false>
 __global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_shared_kernel(const GemmParams p) {
     __shared__ __attribute__((aligned(16))) GroupedSmem sm;
@@ -1185,7 +1186,12 @@ __global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_shared_kernel(co
     const int mblk = (local >> 3) % mblocks;
     const int unit = (local / (8 * mblocks)) * 8 + (local & 7);
     if (unit * (kGroupedWaves / NK) >= p.strips) return;  // padding workgroup (uniform)
-    // two row blocks (the host sends 17..32 token rows here): the second read of the weights comes from L2
+    if (mblocks == 1) {  // one row block: every weight byte is used once (loads marked stream-once)
+        if (p.split > 1) shared_body<4, GS, NK, true, ASYM, true, true, OutT, DUMP>(p, unit, mblk, wave, sm, blockIdx.y);
+        else shared_body<4, GS, NK, true, ASYM, true, false, OutT, DUMP>(p, unit, mblk, wave, sm);
+        return;
+    }
+    // several row blocks: all but the first read of the weights come from L2
     if (p.split > 1) shared_body<4, GS, NK, true, ASYM, false, true, OutT, DUMP>(p, unit, mblk, wave, sm, blockIdx.y);
     else shared_body<4, GS, NK, true, ASYM, false, false, OutT, DUMP>(p, unit, mblk, wave, sm);
 }
@@ -1204,11 +1210,18 @@ static void launch_shared_nk(const GemmParams& p, bool asym, bool out_bf16, hipS
     }
 }
 
+// kparts: k-parts per workgroup, kSharedParts (four strips share an activation stream) or twice that (two strips)
 template <bool DUMP>
-static hipError_t launch_skinny_shared_impl(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream) {
-    if (gs == 1) launch_shared_nk<1, kSharedParts, DUMP>(p, asym, out_bf16, stream);
-    else if (gs == 2) launch_shared_nk<2, kSharedParts, DUMP>(p, asym, out_bf16, stream);
-    else launch_shared_nk<4, kSharedParts, DUMP>(p, asym, out_bf16, stream);
+static hipError_t launch_skinny_shared_impl(const GemmParams& p, int gs, int kparts, bool asym, bool out_bf16, hipStream_t stream) {
+    if (kparts == kSharedParts) {
+        if (gs == 1) launch_shared_nk<1, kSharedParts, DUMP>(p, asym, out_bf16, stream);
+        else if (gs == 2) launch_shared_nk<2, kSharedParts, DUMP>(p, asym, out_bf16, stream);
+        else launch_shared_nk<4, kSharedParts, DUMP>(p, asym, out_bf16, stream);
+    } else {
+        if (gs == 1) launch_shared_nk<1, 2 * kSharedParts, DUMP>(p, asym, out_bf16, stream);
+        else if (gs == 2) launch_shared_nk<2, 2 * kSharedParts, DUMP>(p, asym, out_bf16, stream);
+        else launch_shared_nk<4, 2 * kSharedParts, DUMP>(p, asym, out_bf16, stream);
+    }
     return hipGetLastError();
 }
 

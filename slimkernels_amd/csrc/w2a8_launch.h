@@ -39,9 +39,9 @@ hipError_t launch_skinny_fused(const GemmParams& p, int gs, int waves, bool asym
 // there, p.ws_counter at the workspace's counter block); spin_limit bounds the wait for the rows.
 hipError_t launch_skinny_rows(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, int spin_limit, hipStream_t stream);
 
-// one problem of 17..32 token rows through the shared-activation workgroups (kSharedParts k-parts x
-// 8 / kSharedParts strips per workgroup, p.split K splits across workgroups)
-hipError_t launch_skinny_shared(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
+// one problem through the shared-activation workgroups (kparts k-parts x 8 / kparts strips per workgroup, kparts =
+// kSharedParts or twice that; p.split K splits across workgroups)
+hipError_t launch_skinny_shared(const GemmParams& p, int gs, int kparts, bool asym, bool out_bf16, hipStream_t stream);
 
 // asym: every problem carries per-group zero-points (zp_r); otherwise each uses its uniform zp_const
 hipError_t launch_skinny_grouped(const GroupedParams& gp, int gs, bool asym, bool out_bf16, hipStream_t stream);
@@ -49,7 +49,7 @@ hipError_t launch_skinny_grouped(const GroupedParams& gp, int gs, bool asym, boo
 // Verification instantiations of the three launches above (gemm_skinny_verify.hip): the same bodies with the int32
 // dump switched on (p.acc_dump / p.dump_mode, per problem in a grouped launch), same instantiation choices.
 hipError_t launch_skinny_verify(const GemmParams& p, int gs, int waves, bool asym, bool out_bf16, hipStream_t stream);
-hipError_t launch_skinny_shared_verify(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
+hipError_t launch_skinny_shared_verify(const GemmParams& p, int gs, int kparts, bool asym, bool out_bf16, hipStream_t stream);
 hipError_t launch_skinny_grouped_verify(const GroupedParams& gp, int gs, bool asym, bool out_bf16, hipStream_t stream);
 
 // 4-bit weights as two planes (w_r over 2 * p.steps steps, s_r over 2 * p.G groups), uniform zero-point 8, one pass

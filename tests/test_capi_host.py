@@ -71,7 +71,8 @@ def test_split_heuristic_and_workspace(L):
 def test_auto_route(L):
     """Which kernel form AUTO takes: 1 one-strip skinny, 2 tiled, 3 shared-activation skinny."""
     route = L.slimk_w2a8_gemm_auto_route
-    assert route(1, 4096, 4096, 128) == 1 and route(16, 28672, 8192, 64) == 1
+    assert route(1, 4096, 4096, 128) == 1 and route(11, 28672, 8192, 64) == 1 and route(16, 14336, 8192, 64) == 1
+    assert route(12, 28672, 8192, 64) == 3 and route(16, 28672, 8192, 64) == 3   # 12..16 rows on 384 strips and more
     assert route(20, 4096, 4096, 128) == 1          # 17..32 rows: shared only on matrices of 24 MiB or more
     assert route(20, 8192, 14336, 128) == 3
     assert route(33, 4096, 4096, 128) == 1          # few workgroups: the one-strip kernel

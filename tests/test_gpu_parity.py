@@ -251,6 +251,21 @@ def test_skinny_shared_one_problem(gpu_ops, oracle, M, N, K, g, mode, out, split
 
 
 @pytest.mark.parametrize("M,N,K,g,mode,out,split", [
+    (14, 24640, 512, 64, "asym", "bfloat16", 0),    # two chunks for four k-parts: two of them idle
+    (16, 24577, 2048, 128, "sym", "float16", 0),    # ragged last strip, odd number of two-strip units
+    (12, 25000, 1280, 256, "ref", "float16", 2),    # explicit split, groups of 256
+])
+def test_skinny_shared_12_to_16_rows_on_wide_matrices(gpu_ops, oracle, M, N, K, g, mode, out, split):
+    """12..16 token rows on 384 strips and more run through shared-activation workgroups of four k-parts x two
+    strips: int32 group sums exact, the output criterion, verification and production bits equal."""
+    from slimkernels_amd import _lib
+    assert _lib.lib().slimk_w2a8_gemm_auto_route(M, N, K, g) == 3
+    case = pu.small_case(M, N, K, g, mode, seed=M + N + K, out_dtype=out)
+    _run_case(gpu_ops, oracle, case, "auto", split_k=split, dump="groups")
+    _run_case(gpu_ops, oracle, case, "skinny", split_k=split)
+
+
+@pytest.mark.parametrize("M,N,K,g,mode,out,split", [
     (100, 6200, 2304, 64, "asym", "bfloat16", 0),   # short reduction: seven row blocks, the last ragged, ragged last strip
     (130, 1000, 12288, 128, "sym", "float16", 0),   # long reduction, few strips: nine row blocks, K split across workgroups
     (33, 4000, 12288, 256, "ref", "float16", 0),    # the third row block holds one row
