@@ -396,15 +396,32 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
         const uint32_t ws_lane = (uint32_t)wave * (kMB * 16 * 64 * 4) + lane * 16;   // this wave's fragments, this lane's 16 bytes
         const uint32_t ws_tile = (uint32_t)tile * kTileBytes;
         const uint32_t ws_split_pitch = (uint32_t)total * kTileBytes;
+        // Nothing but the stores between the first of them and the wait for all of them: a 16-byte-per-lane buffer
+        // store with a scalar offset reads its data registers some time after it issues (longer when the memory
+        // pipeline is backed up, as it is for the workgroups of a launch that start last), and the compiler knows of
+        // no hazard there, so a vector instruction scheduled behind a store may reuse the store's first data register -
+        // here it did, for the address of the next stores, and the partial sums of four lanes in sixteen went to
+        // memory as that address (130 x 4096 x 1024 in eight splits, bf16 out: 48..150 outputs short of one split's
+        // share on every run).  So the addresses are made before the first store, and fences keep everything else
+        // out of the run of stores.
+        uint32_t ws_off[kMB];
+#pragma unroll
+        for (int mb = 0; mb < kMB; ++mb) {
+            ws_off[mb] = ws_lane + mb * 4096;
+            asm volatile("" : "+v"(ws_off[mb]));
+        }
+        const uint32_t ws_base = blockIdx.y * ws_split_pitch + ws_tile;
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
             for (int pp = 0; pp < 4; ++pp) {
                 const v4f v = {t[mb][pp][0], t[mb][pp][1], t[mb][pp][2], t[mb][pp][3]};
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_t, v), ws_rsrc, ws_lane + (mb * 4 + pp) * 1024,
-                                                       blockIdx.y * ws_split_pitch + ws_tile, kCoherent);
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_t, v), ws_rsrc, ws_off[mb] + pp * 1024, ws_base, kCoherent);
             }
+        __builtin_amdgcn_sched_barrier(0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
         if (tid == 0) {
             const unsigned prev = __hip_atomic_fetch_add(p.ws_counter + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

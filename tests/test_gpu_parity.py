@@ -336,7 +336,10 @@ def test_tiled_output_views(gpu_ops, oracle, M, N, K, g, out):
 @pytest.mark.parametrize("M,N,K,g,out,split", [(64, 256, 2048, 128, "float16", 2), (77, 300, 4096, 64, "bfloat16", 4),
                                                  (130, 64, 3072, 128, "float16", 3), (40, 512, 8192, 128, "float16", 8),
                                                  (64, 256, 4096, 256, "float16", 3), (77, 300, 4160, 64, "bfloat16", 4),
-                                                 (50, 128, 2816, 256, "bfloat16", 11)])
+                                                 (50, 128, 2816, 256, "bfloat16", 11),
+                                                 # more workgroups than run at once, one stage each: the last ones to start
+                                                 # find the memory pipeline backed up when they store their partial sums
+                                                 (130, 4096, 1024, 64, "bfloat16", 8), (130, 4096, 2048, 128, "float16", 8)])
 def test_tiled_split_k(gpu_ops, oracle, M, N, K, g, out, split):
     """Split-K of the fast tiled kernel: the output criterion, and run-to-run identical bits."""
     case = pu.small_case(M, N, K, g, "sym", seed=M + K, out_dtype=out)
