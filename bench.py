@@ -240,6 +240,7 @@ def main():
             traceback.print_exc(file=sys.stderr)
             detail["detail_error"] = repr(e)
         result["roofline"]["also"] = also_rows(detail, step_bytes, len(cases))
+        result["roofline"].update(flat_fractions(detail))
         result["cpu_baseline"] = cpu_baseline(np, workloads, shapes)
     else:
         result["cpu_baseline"] = None
@@ -276,6 +277,31 @@ def also_rows(detail, step_bytes, n_gemms):
                      "kernel": "w2a8::skinny_grouped_kernel", "avg_us": r["us"], "achieved": r["GBps"], "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": r["frac_hbm"]})
     return rows
+
+
+def flat_fractions(detail):
+    """The same figures as `also`, as scalar keys of the `roofline` object itself (a reader that keeps only an object's
+    scalars still gets both halves of the metric): `mfma_frac_*` against the int8 MFMA peak, `hbm_frac_*` against HBM,
+    named <config>_m<rows>_<N>x<K>; single launches unless the name says grouped."""
+    flat = {}
+    for r in detail.get("prefill", []):
+        flat[f"mfma_frac_c3_m{r['M']}_{r['shape']}"] = r["frac_int8_mfma"]
+        flat[f"act_quant_us_c3_m{r['M']}_{r['shape']}"] = r["act_quant_us"]
+    for r in detail.get("other_configs", []):
+        key = f"{r['config']}_m{r['M']}_{r['shape']}"
+        if r["M"] >= 2048:
+            flat[f"mfma_frac_{key}"] = r["frac_int8_mfma"]
+        elif r["M"] <= 16:
+            flat[f"hbm_frac_{key}"] = r["frac_hbm"]
+        else:  # near the ridge: both
+            flat[f"hbm_frac_{key}"] = r["frac_hbm"]
+            flat[f"mfma_frac_{key}"] = r["frac_int8_mfma"]
+        flat[f"us_{key}"] = r["us"]
+    if "single_launch" in detail:
+        flat["hbm_frac_c2_single_launch"] = detail["single_launch"]["frac_hbm"]
+    if "decode_sweep_m_le_16" in detail:
+        flat["hbm_frac_c2_grouped_m_le_16"] = detail["decode_sweep_m_le_16"]["frac_hbm"]
+    return flat
 
 
 def _lib_check(rc):
@@ -420,7 +446,20 @@ def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, d
     # in rotation, over twice the 256 MiB last-level cache; one graph replay = ten launches), larger M warm.
     def random_weight(N, K, g, asym):
         strips = -(-N // 64)
-        w_r = torch.randint(-2**31, 2**31 - 1, (strips * (K // 64) * 256,), dtype=torch.int32, device=dev)
+        # the streaming layout pads the step count to whole runs of four: size the buffer as the library does and
+        # leave the padding units zero
+        dwords = L.slimk_w2a8_repacked_weight_bytes(N, K) // 4
+        used = strips * (K // 64) * 256
+        w_r = torch.zeros(dwords, dtype=torch.int32, device=dev)
+        if used == dwords:
+            w_r.copy_(torch.randint(-2**31, 2**31 - 1, (dwords,), dtype=torch.int32, device=dev))
+        else:  # runs of four steps per strip: [run][strip][4 steps][256 dwords]; the last run's surplus steps stay zero
+            steps = K // 64
+            view = w_r.view(-1, strips, 4, 256)
+            full = steps // 4
+            view[:full].copy_(torch.randint(-2**31, 2**31 - 1, (full, strips, 4, 256), dtype=torch.int32, device=dev))
+            if steps % 4:
+                view[full, :, :steps % 4].copy_(torch.randint(-2**31, 2**31 - 1, (strips, steps % 4, 256), dtype=torch.int32, device=dev))
         s_r = (torch.rand(strips * (K // g) * 64, device=dev) * 0.02 + 0.005).half()
         zp_r = torch.randint(0, 4, (strips * (K // g) * 64,), dtype=torch.uint8, device=dev) if asym else None
         return ops.W2A8Weight(w_r, s_r, zp_r, 0 if asym else 2, N, K, g)

@@ -186,7 +186,10 @@ int slimk_w2a8_quantize_weight4(const void* w, int ldw, int w_dtype, int N, int 
  *   q [M][ldq] int8     = clip(rne(x / s_a[m]), -127, 127)
  *   s_a [M]    float32  = max(absmax_k |x[m,k]|, 1e-9) / 127
  *   rowsum [G][ldr] int32 = sum of q over each group (needed by the GEMM to fold
- *                           zero-points); ldr >= M, ldr % 4 == 0
+ *                           zero-points); ldr >= M, ldr % 4 == 0.  NULL: the sums are not formed (a quarter
+ *                           faster on prefill-sized inputs); slimk_w2a8_gemm takes such an activation where it
+ *                           reads no row sums: the tiled kernel with zp_r NULL and zp_const 2
+ *                           (slimk_w2a8_gemm_auto_route(M, N, K, group_size) == 2 says when AUTO goes there)
  * ldx, ldq in elements; x, q, rowsum 16-byte aligned; ldx % 8 == 0, ldq % 16 == 0. */
 int slimk_w2a8_act_quant(const void* x, int ldx, int x_dtype, int M, int K, int group_size,
                          int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, void* stream);
@@ -242,8 +245,10 @@ int slimk_w2a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
  *  - Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (different streams,
  *    concurrent graph launches) race on it; calls ordered on one stream, of any shapes, are fine (each leaves
  *    the counters at zero, the partial sums need no clearing).
- *  - The first call on each GPU looks the array's address up and clears its counter block with a small kernel on
- *    `stream`; make that call outside graph capture. */
+ *  - Arguments are validated first, as in slimk_w2a8_gemm: a rejected call touches neither the array nor the GPU.
+ *    The first call on each GPU that splits K looks the array's address up and clears its counter block with a
+ *    small kernel on `stream`; make that call outside stream capture (inside one it is refused with
+ *    SLIMK_ERR_UNSUPPORTED rather than recorded into the caller's graph). */
 #define SLIMK_W2A8_STATIC_WORKSPACE_BYTES ((16u << 20) + (64u << 10))
 size_t slimk_w2a8_static_workspace_bytes(void);
 int slimk_w2a8_gemm_static(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,

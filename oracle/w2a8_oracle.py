@@ -353,11 +353,12 @@ def w2a16_reference_forward(x_half: np.ndarray, codes_nk: np.ndarray, scale_half
 # --------------------------------------------------------------------------- whole-path helper
 
 def reference_forward(x_half: np.ndarray, packed: np.ndarray, scale_half: np.ndarray, zp: np.ndarray,
-                      group_size: int, out_bf16: bool = False, want_acc: bool = True):
-    """act-quant -> int32 per-group accumulate -> epilogue, all on the CPU.
+                      group_size: int, out_bf16: bool = False, want_acc: bool = True, x_bf16: bool = False):
+    """act-quant -> int32 per-group accumulate -> epilogue, all on the CPU.  With x_bf16 the activations are
+    uint16 bf16 bit patterns instead of a float16 array.
 
     Returns dict(q, s_a, rowsum, acc (or None), out_bits, out_f32 (or None))."""
-    q, s_a, rs = c_act_quant(x_half, group_size)
+    q, s_a, rs = c_act_quant(x_half, group_size, is_bf16=x_bf16)
     if want_acc:
         acc = c_gemm_acc(q, packed, zp, group_size)
         out_bits, out_f32 = c_epilogue(acc, scale_half, s_a, out_bf16)

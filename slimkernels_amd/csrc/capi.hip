@@ -187,8 +187,8 @@ int resolve_kernel(int M, int N, int K, int group_size, int kernel) {
 
 // One problem with 17..32 token rows on a matrix big enough to be bound by bandwidth goes through the shared-activation
 // workgroups: 8..27 % faster there than one strip per workgroup (at 16 rows and below the one-strip kernel is as fast
-// or faster); with more rows, where mid_route says so (a request for the skinny kernel where the tiled one is
-// predicted ahead takes the faster of the two skinny forms).
+// or faster); with more rows, where mid_route says so (an explicit request for the skinny kernel on a shape
+// that mid_route gives to the tiled one runs one strip per workgroup, whichever skinny form would be the faster there).
 bool skinny_shared_applies(int M, int N, int K, int group_size) {
     if (M >= kWideSharedRows && M <= 16) return strips_of(N) >= kWideSharedStrips;
     if (M <= 16 || M > kSkinnyMaxRows) return false;
@@ -360,8 +360,12 @@ int slimk_w2a8_act_quant(const void* x, int ldx, int x_dtype, int M, int K, int 
 
 namespace {
 
-// fit_split: a split factor chosen here (split_k <= 0) is lowered until its workspace fits workspace_bytes
-// (the library-owned workspace of slimk_w2a8_gemm_static has a fixed size); a caller's explicit split never is.
+int static_workspace(void** ptr, hipStream_t stream);
+
+// fit_split: the call is slimk_w2a8_gemm_static's: `workspace` is NULL and workspace_bytes the size of the library-owned
+// array; a split factor chosen here (split_k <= 0) is lowered until its workspace fits that size (a caller's explicit
+// split never is), and the array itself is looked up only once every argument has passed validation and the launch
+// turns out to split K.
 int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum, int ldr,
               const uint32_t* w_r, const uint16_t* s_r, const uint8_t* zp_r, int zp_const,
               int M, int N, int K, int group_size,
@@ -435,6 +439,12 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
 
     if (split_k > 1) {
         const size_t need = slimk_w2a8_gemm_workspace_bytes(M, N, K, group_size, kern, split_k);
+        if (fit_split && workspace_bytes < need)
+            return fail(SLIMK_ERR_WORKSPACE, "gemm_static: split_k=%d needs %zu bytes of workspace, the library-owned one holds %zu "
+                        "(pass a smaller split_k, 0 to let the library choose one that fits, or use slimk_w2a8_gemm)",
+                        split_k, need, workspace_bytes);
+        if (fit_split)
+            if (int rc = static_workspace(&workspace, (hipStream_t)stream)) return rc;
         if (!workspace) return fail(SLIMK_ERR_WORKSPACE, "split_k=%d needs a workspace of %zu bytes", split_k, need);
         if (workspace_bytes < need)
             return fail(SLIMK_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, need);
@@ -478,12 +488,18 @@ void* g_scratch_ptr[kMaxDevices];   // per device: where that device's copy of `
 
 // The current device's copy of the array; on the first call on a device its counter block is cleared on `stream`
 // (the array starts as zeros and every GEMM leaves its counters at zero, so this only guards the very first use).
+// That first use must not fall inside a stream capture: the clear would be recorded into the caller's graph.
 int static_workspace(void** ptr, hipStream_t stream) {
     int dev = -1;
     if (hipError_t e = hipGetDevice(&dev)) return hip_result(e, "hipGetDevice");
     if (dev < 0 || dev >= kMaxDevices) return fail(SLIMK_ERR_UNSUPPORTED, "device ordinal %d (at most %d devices)", dev, kMaxDevices);
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     if (!g_scratch_ptr[dev]) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipError_t e = hipStreamIsCapturing(stream, &cap)) return hip_result(e, "hipStreamIsCapturing");
+        if (cap != hipStreamCaptureStatusNone)
+            return fail(SLIMK_ERR_UNSUPPORTED, "gemm_static: the first split-K call on a device sets the library-owned workspace up "
+                        "and must be made outside stream capture");
         void* p = nullptr;
         if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) return hip_result(e, "hipGetSymbolAddress(scratch)");
         if (!p || !aligned16(p)) return fail(SLIMK_ERR_HIP, "hipGetSymbolAddress(scratch) returned %p", p);
@@ -516,18 +532,10 @@ int slimk_w2a8_gemm_static(const int8_t* q, int ldq, const float* s_a, const int
                            int M, int N, int K, int group_size,
                            void* out, int ldo, int out_dtype,
                            int kernel, int split_k, void* stream) {
-    // an explicit split beyond the fixed workspace is an error here, before anything touches the GPU
-    if (split_k > 1 && M > 0 && N > 0 && shape_ok(K, group_size) && kernel >= SLIMK_KERNEL_AUTO && kernel <= SLIMK_KERNEL_TILED) {
-        const size_t need = slimk_w2a8_gemm_workspace_bytes(M, N, K, group_size, kernel, split_k);
-        if (need > kStaticWorkspaceBytes)
-            return fail(SLIMK_ERR_WORKSPACE, "gemm_static: split_k=%d needs %zu bytes of workspace, the library-owned one holds %zu "
-                        "(pass a smaller split_k, 0 to let the library choose one that fits, or use slimk_w2a8_gemm)",
-                        split_k, need, kStaticWorkspaceBytes);
-    }
-    void* ws = nullptr;
-    if (int rc = static_workspace(&ws, (hipStream_t)stream)) return rc;
+    // every argument is validated before anything touches the GPU; the library-owned array is looked up (and, on a
+    // device's first split-K call, its counters cleared) only when the launch splits K
     return gemm_impl(q, ldq, s_a, rowsum, ldr, w_r, s_r, zp_r, zp_const, M, N, K, group_size, out, ldo, out_dtype,
-                     nullptr, SLIMK_DUMP_NONE, ws, kStaticWorkspaceBytes, kernel, split_k, stream, true);
+                     nullptr, SLIMK_DUMP_NONE, nullptr, kStaticWorkspaceBytes, kernel, split_k, stream, true);
 }
 
 int slimk_w2a8_gemm_fused(const void* x, int ldx, int x_dtype,

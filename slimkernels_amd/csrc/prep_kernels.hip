@@ -187,7 +187,10 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
 // workgroup leaves most of the chip idle and a row's time is what its one CU needs for the arithmetic.  The IEEE
 // divisions (a dozen instructions each) were most of that arithmetic: rne_quotient() (w2a8_common.h) avoids nearly
 // all of them (32 rows x 28672: 8.2 -> 7.2 us; 4096 x 4096: 17.6 -> 15.2 us).
-template <bool BF16, int KEEP, int THREADS = 256>
+// SUMS false: no per-group sums of q (rowsum is not touched): what a caller asks for whose GEMM folds no zero-point
+// through them (the tiled kernel with the symmetric levels): the sums' adds, shuffles and scattered 4-byte stores are
+// a sixth of the kernel's time at 4096 x 14336.
+template <bool BF16, int KEEP, int THREADS = 256, bool SUMS = true>
 __global__ __launch_bounds__(THREADS) void act_quant_keep_kernel(const uint16_t* __restrict__ x, int ldx, int M, int K,
                                                              int group_size, int8_t* __restrict__ q, int ldq,
                                                              float* __restrict__ s_a,
@@ -238,52 +241,59 @@ __global__ __launch_bounds__(THREADS) void act_quant_keep_kernel(const uint16_t*
                 float r = rne_quotient(f[i], s, inv_s);  // = rintf(f[i] / s), bit for bit
                 r = fminf(fmaxf(r, -127.0f), 127.0f);
                 const int qi = (int)r;
-                sum += qi;
+                if (SUMS) sum += qi;
                 if (i < 4) lo |= (uint32_t)(qi & 0xff) << (8 * i);
                 else hi |= (uint32_t)(qi & 0xff) << (8 * (i - 4));
             }
             for (int cp = 0; cp < copies; ++cp)   // copies > 1: the row laid down again K further on
                 *reinterpret_cast<uint2*>(qr + (size_t)cp * K + (size_t)v * 8) = make_uint2(lo, hi);
         }
-        for (int off = 1; off < tpg; off <<= 1) sum += __shfl_xor(sum, off, 64);
-        if (rowsum && v < nvec && (v % tpg) == 0)
-            for (int cp = 0; cp < copies; ++cp) rowsum[((size_t)cp * (nvec / tpg) + v / tpg) * ldr + m] = sum;
+        if constexpr (SUMS) {
+            for (int off = 1; off < tpg; off <<= 1) sum += __shfl_xor(sum, off, 64);
+            if (v < nvec && (v % tpg) == 0)
+                for (int cp = 0; cp < copies; ++cp) rowsum[((size_t)cp * (nvec / tpg) + v / tpg) * ldr + m] = sum;
+        }
     }
 }
 
 constexpr int kFewRows = 64;  // up to this many rows a long row gets 1024 threads
 
-template <bool BF16>
+template <bool BF16, bool SUMS>
 static void launch_act_quant_keep(const void* x, int ldx, int M, int K, int group_size, int8_t* q, int ldq, float* s_a,
                                   int32_t* rowsum, int ldr, int copies, hipStream_t stream) {
     const dim3 grid((unsigned)act_quant_grid(M)), block(256);
     if (M <= kFewRows && K > 2048 && K <= 4096) {  // a few rows: 512 threads a row, one vector each
-        act_quant_keep_kernel<BF16, 1, 512><<<grid, dim3(512), 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+        act_quant_keep_kernel<BF16, 1, 512, SUMS><<<grid, dim3(512), 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
         return;
     }
     if (M <= kFewRows && K > 4096) {  // a few long rows: 1024 threads a row
         const dim3 wide(1024);
         if (K <= 8192)
-            act_quant_keep_kernel<BF16, 1, 1024><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+            act_quant_keep_kernel<BF16, 1, 1024, SUMS><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
         else if (K <= 16384)
-            act_quant_keep_kernel<BF16, 2, 1024><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+            act_quant_keep_kernel<BF16, 2, 1024, SUMS><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
         else
-            act_quant_keep_kernel<BF16, 4, 1024><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+            act_quant_keep_kernel<BF16, 4, 1024, SUMS><<<grid, wide, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
         return;
     }
     if (K <= 4096)
-        act_quant_keep_kernel<BF16, 2><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+        act_quant_keep_kernel<BF16, 2, 256, SUMS><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
     else if (K <= 8192)
-        act_quant_keep_kernel<BF16, 4><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+        act_quant_keep_kernel<BF16, 4, 256, SUMS><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
     else
-        act_quant_keep_kernel<BF16, 8><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
+        act_quant_keep_kernel<BF16, 8, 256, SUMS><<<grid, block, 0, stream>>>((const uint16_t*)x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies);
 }
 
 hipError_t launch_act_quant(const void* x, int ldx, bool x_bf16, int M, int K, int group_size,
                             int8_t* q, int ldq, float* s_a, int32_t* rowsum, int ldr, int copies, hipStream_t stream) {
     if (K <= 16384 || (M <= kFewRows && K <= 32768)) {
-        if (x_bf16) launch_act_quant_keep<true>(x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies, stream);
-        else launch_act_quant_keep<false>(x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies, stream);
+        if (rowsum) {
+            if (x_bf16) launch_act_quant_keep<true, true>(x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies, stream);
+            else launch_act_quant_keep<false, true>(x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies, stream);
+        } else {
+            if (x_bf16) launch_act_quant_keep<true, false>(x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies, stream);
+            else launch_act_quant_keep<false, false>(x, ldx, M, K, group_size, q, ldq, s_a, rowsum, ldr, copies, stream);
+        }
         return hipGetLastError();
     }
     if (x_bf16)

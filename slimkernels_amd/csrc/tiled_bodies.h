@@ -396,28 +396,30 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
         const uint32_t ws_lane = (uint32_t)wave * (kMB * 16 * 64 * 4) + lane * 16;   // this wave's fragments, this lane's 16 bytes
         const uint32_t ws_tile = (uint32_t)tile * kTileBytes;
         const uint32_t ws_split_pitch = (uint32_t)total * kTileBytes;
-        // Nothing but the stores between the first of them and the wait for all of them: a 16-byte-per-lane buffer
-        // store with a scalar offset reads its data registers some time after it issues (longer when the memory
-        // pipeline is backed up, as it is for the workgroups of a launch that start last), and the compiler knows of
-        // no hazard there, so a vector instruction scheduled behind a store may reuse the store's first data register -
-        // here it did, for the address of the next stores, and the partial sums of four lanes in sixteen went to
-        // memory as that address (130 x 4096 x 1024 in eight splits, bf16 out: 48..150 outputs short of one split's
-        // share on every run).  So the addresses are made before the first store, and fences keep everything else
-        // out of the run of stores.
+        // A 16-byte-per-lane buffer store reads its data registers some time after it issues (longer when the memory
+        // pipeline is backed up, as it is for the workgroups of a launch that start last).  With a register in the
+        // scalar-offset field the compiler knows of no hazard there, and a vector instruction scheduled behind such a
+        // store once reused the store's first data register for the address of the next stores: the partial sums of
+        // four lanes in sixteen went to memory as that address (130 x 4096 x 1024 in eight splits, bf16 out: 48..150
+        // outputs short of one split's share on every run).  Three independent measures against it: the split's and the tile's base go into the per-lane offset, so the scalar offset is the constant
+        // zero, the form whose wait states the compiler inserts itself; every address is made before the first store
+        // and each store is followed by two idle cycles written here (the wait the hardware needs, whatever the
+        // scheduler and the register allocator do); and fences keep everything else out of the run of stores.
+        const uint32_t ws_base = blockIdx.y * ws_split_pitch + ws_tile;
         uint32_t ws_off[kMB];
 #pragma unroll
         for (int mb = 0; mb < kMB; ++mb) {
-            ws_off[mb] = ws_lane + mb * 4096;
+            ws_off[mb] = ws_lane + mb * 4096 + ws_base;
             asm volatile("" : "+v"(ws_off[mb]));
         }
-        const uint32_t ws_base = blockIdx.y * ws_split_pitch + ws_tile;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
             for (int pp = 0; pp < 4; ++pp) {
                 const v4f v = {t[mb][pp][0], t[mb][pp][1], t[mb][pp][2], t[mb][pp][3]};
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_t, v), ws_rsrc, ws_off[mb] + pp * 1024, ws_base, kCoherent);
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_t, v), ws_rsrc, ws_off[mb] + pp * 1024, 0, kCoherent);
+                asm volatile("s_nop 1" ::: "memory");
             }
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

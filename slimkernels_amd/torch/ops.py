@@ -65,7 +65,7 @@ class W2A8Weight:
 class QuantizedActivation:
     q: torch.Tensor        # int8 [M, K]
     s_a: torch.Tensor      # float32 [M]
-    rowsum: torch.Tensor   # int32 [G, ldr]
+    rowsum: Optional[torch.Tensor]   # int32 [G, ldr]; None: quantised without group sums (tiled kernel, symmetric levels)
     group_size: int
 
 
@@ -157,10 +157,12 @@ def load_w2_weight(path, device="cuda", mmap=True) -> W2A8Weight:
                      zp_const=f["zp_const"] if f["zp_const"] is not None else 0, device=device)
 
 
-def quantize_act_int8(x: torch.Tensor, group_size: int = 128, copies: int = 1) -> QuantizedActivation:
+def quantize_act_int8(x: torch.Tensor, group_size: int = 128, copies: int = 1, rowsum: bool = True) -> QuantizedActivation:
     """Per-token symmetric int8 quantisation: x [M, K] fp16/bf16 -> q, s_a, per-group row sums.  With
     ``copies`` > 1 the quantised row and its group sums are laid down that many times (q [M, copies * K],
-    rowsum [copies * G, ...]): the operand of a reduction over copies * K, as the 4-bit weights take it."""
+    rowsum [copies * G, ...]): the operand of a reduction over copies * K, as the 4-bit weights take it.
+    ``rowsum=False`` leaves the group sums out (faster on many rows); only the tiled kernel on weights with the
+    symmetric levels takes such an activation (see ``needs_rowsum``)."""
     L = _lib.lib()
     _require_cuda(x, "x")
     if x.dim() != 2 or x.dtype not in _DT:
@@ -174,12 +176,20 @@ def quantize_act_int8(x: torch.Tensor, group_size: int = 128, copies: int = 1) -
     copies = int(copies)
     q = torch.empty((M, max(copies, 1) * K), dtype=torch.int8, device=x.device)
     s_a = torch.empty((M,), dtype=torch.float32, device=x.device)
-    rowsum = torch.empty((max(copies, 1) * max(K // group_size, 1), ldr), dtype=torch.int32, device=x.device)
+    rs = torch.empty((max(copies, 1) * max(K // group_size, 1), ldr), dtype=torch.int32, device=x.device) if rowsum else None
     with torch.cuda.device(x.device):
         _lib.check(L.slimk_w2a8_act_quant_rep(x.data_ptr(), x.stride(0), _DT[x.dtype], M, K, group_size, copies,
-                                              q.data_ptr(), q.stride(0), s_a.data_ptr(), rowsum.data_ptr(), ldr,
-                                              _stream_ptr(x.device)))
-    return QuantizedActivation(q, s_a, rowsum, group_size)
+                                              q.data_ptr(), q.stride(0), s_a.data_ptr(),
+                                              rs.data_ptr() if rs is not None else None, ldr, _stream_ptr(x.device)))
+    return QuantizedActivation(q, s_a, rs, group_size)
+
+
+def needs_rowsum(M: int, w: "W2A8Weight") -> bool:
+    """Whether ``w2a8_gemm(..., kernel="auto")`` of M token rows on this weight reads the activation's group sums:
+    everything but the tiled kernel on the symmetric levels (uniform zero-point 2) does."""
+    if w.zp_r is not None or w.zp_const != 2 or w.group_size > 256:
+        return True
+    return _lib.lib().slimk_w2a8_gemm_auto_route(M, w.N, w.K, w.group_size) != 2
 
 
 def _workspace(w: W2A8Weight, nbytes: int) -> Optional[torch.Tensor]:
@@ -221,7 +231,9 @@ def w2a8_gemm(qa: QuantizedActivation, w: W2A8Weight, out_dtype=torch.float16, *
         ws_bytes = L.slimk_w2a8_gemm_workspace_bytes(M, w.N, K, w.group_size, kern, split_k)
         ws = _workspace(w, ws_bytes)
         _lib.check(L.slimk_w2a8_gemm(
-            qa.q.data_ptr(), qa.q.stride(0), qa.s_a.data_ptr(), qa.rowsum.data_ptr(), qa.rowsum.stride(0),
+            qa.q.data_ptr(), qa.q.stride(0), qa.s_a.data_ptr(),
+            qa.rowsum.data_ptr() if qa.rowsum is not None else None,
+            qa.rowsum.stride(0) if qa.rowsum is not None else (M + 3) // 4 * 4,
             w.w_r.data_ptr(), w.s_r.data_ptr(), w.zp_r.data_ptr() if w.zp_r is not None else None, w.zp_const,
             M, w.N, K, w.group_size, out.data_ptr(), out.stride(0), _DT[out.dtype],
             acc.data_ptr() if acc is not None else None, mode,
@@ -384,14 +396,21 @@ def _wint2_weight(weight, scale, zp, group_size, zp_const, device) -> W2A8Weight
     if not all(isinstance(t, torch.Tensor) for t in tensors):
         return repack_w2(np.ascontiguousarray(np.asarray(weight).T) if not isinstance(weight, torch.Tensor) else weight.t().contiguous(),
                          scale, zp, group_size, zp_const, device=device)
-    key = tuple((id(t), t.data_ptr(), t._version, tuple(t.shape), tuple(t.stride())) for t in tensors) + (
-        zp is None, group_size, zp_const, str(device))
+    # A tensor is recognised by the memory it views (storage address, offset, shape, strides, dtype) and its version
+    # counter, not by the Python object: `packed.T` makes a new view object on every call.  The version counter cannot
+    # be read on inference-mode tensors: such operands are re-laid every call instead of failing.
+    try:
+        key = tuple((t.untyped_storage().data_ptr(), t.storage_offset(), tuple(t.shape), tuple(t.stride()), t.dtype,
+                     t._version) for t in tensors) + (zp is None, group_size, zp_const, str(device))
+    except RuntimeError:
+        return repack_w2(weight.t().contiguous(), scale, zp, group_size, zp_const, device=device)
     hit = _WINT2_CACHE.get(key)
     if hit is not None:
         _WINT2_CACHE.move_to_end(key)
         return hit[0]
     w = repack_w2(weight.t().contiguous(), scale, zp, group_size, zp_const, device=device)
-    _WINT2_CACHE[key] = (w, tensors)   # the tensors are held so that their ids and addresses stay theirs
+    # the storages are held (not the views) so that their addresses stay theirs while the entry lives
+    _WINT2_CACHE[key] = (w, [t.untyped_storage() for t in tensors])
     while len(_WINT2_CACHE) > _WINT2_CACHE_SIZE:
         _WINT2_CACHE.popitem(last=False)
     return w
@@ -438,7 +457,9 @@ class W2A8Linear(torch.nn.Module):
             # 4096 x 4096; from two rows on the separate act-quant launch is as fast or faster)
             y = w2a8_linear_fused(x2, self.weight, self.out_dtype)
         else:
-            y = w2a8_gemm(quantize_act_int8(x2, self.weight.group_size), self.weight, self.out_dtype)
+            # prefill-sized inputs on symmetric weights go to the tiled kernel, which reads no group sums: leave them out
+            qa = quantize_act_int8(x2, self.weight.group_size, rowsum=needs_rowsum(x2.shape[0], self.weight))
+            y = w2a8_gemm(qa, self.weight, self.out_dtype)
         if self.bias is not None:
             y = y + self.bias
         return y.reshape(*lead, self.out_features)

@@ -28,3 +28,16 @@ def gpu_ops():
         pytest.skip("no GPU visible")
     from slimkernels_amd import torch as ops  # raises if the HIP library is missing
     return ops
+
+
+def pytest_terminal_summary(terminalreporter):
+    """Output-tolerance accounting of the GPU parity tests: how many compared outputs lay beyond rtol 1e-3 / 1 ULP and
+    passed through the re-association bound only (per workload configuration, then in total)."""
+    try:
+        import parity_utils as pu
+    except ImportError:
+        return
+    if pu.VIA_REORDER_TOTAL["elements"]:
+        terminalreporter.write_line("output tolerance accounting (GPU outputs against the oracle):")
+        for line in pu.via_reorder_summary():
+            terminalreporter.write_line("  " + line)

@@ -34,16 +34,27 @@ class OutStats(float):
     size = 0
 
 
-VIA_REORDER_TOTAL = {"elements": 0, "via_reorder": 0}   # running totals over a test session, printed by callers
+# Running totals over a test session: all comparisons, and per workload configuration ("c1" .. "c5"; everything
+# else under "other").  conftest.py prints them in the terminal summary; tests/test_zy_tolerance_accounting.py
+# asserts the configurations' share.
+VIA_REORDER_TOTAL = {"elements": 0, "via_reorder": 0, "worst_x_strict": 0.0}
+VIA_REORDER_BY_CONFIG = {}
+
+# Elements of one comparison that may pass only through the re-association bound: parts per million of its size
+# (and never fewer than two elements: a 16 x 1024 output is 61 ppm an element).  What randomised sweeps of the
+# kernels have shown so far: one or two such elements in a problem of 16 000 .. 676 000 outputs, most problems none.
+MAX_VIA_REORDER_PPM = 100.0
 
 
-def assert_out_close(gpu_bits, ref_bits, bf16, reorder_bound=None, what=""):
+def assert_out_close(gpu_bits, ref_bits, bf16, reorder_bound=None, what="", max_via_reorder_ppm=MAX_VIA_REORDER_PPM,
+                     config=None):
     """The output criterion of the path: every element within 1 ULP of the output type OR within
     rtol 1e-3 of the oracle.  `reorder_bound` (optional, per element) additionally admits the fp32
     rounding noise of summing the per-group terms in another order (split-K, k-parts, the zero-point
     term through fp32 MFMAs), which is what limits elements whose terms cancel to almost zero; pass
-    None where the kernel sums in the oracle's order.  The result carries how many elements needed
-    that third term (`.via_reorder`), and the count is printed."""
+    None where the kernel sums in the oracle's order.  The elements that needed that third term are
+    counted (`.via_reorder` of the result, the session totals above) and their share is asserted:
+    at most `max_via_reorder_ppm` of the comparison's elements (two elements at least)."""
     g, r = bits_to_f32(gpu_bits, bf16), bits_to_f32(ref_bits, bf16)
     assert np.isfinite(g).all(), f"{what}: non-finite GPU output"
     diff = np.abs(g.astype(np.float64) - r.astype(np.float64))
@@ -55,12 +66,33 @@ def assert_out_close(gpu_bits, ref_bits, bf16, reorder_bound=None, what=""):
     stats = OutStats((np.ascontiguousarray(gpu_bits).view(np.uint16) == np.ascontiguousarray(ref_bits).view(np.uint16)).mean())
     stats.via_reorder = int((diff > strict).sum())
     stats.size = int(diff.size)
-    VIA_REORDER_TOTAL["elements"] += stats.size
-    VIA_REORDER_TOTAL["via_reorder"] += stats.via_reorder
+    worst = float((diff / strict).max()) if diff.size else 0.0
+    if config is None:
+        config = what[:2] if what[:2] in ("c1", "c2", "c3", "c4", "c5") and what[2:3] in ("_", " ", "") else "other"
+    for tot in (VIA_REORDER_TOTAL, VIA_REORDER_BY_CONFIG.setdefault(config, {"elements": 0, "via_reorder": 0, "worst_x_strict": 0.0})):
+        tot["elements"] += stats.size
+        tot["via_reorder"] += stats.via_reorder
+        tot["worst_x_strict"] = max(tot["worst_x_strict"], worst if stats.via_reorder else 0.0)
     if stats.via_reorder:
         print(f"{what}: {stats.via_reorder} of {stats.size} outputs beyond rtol 1e-3 / 1 ULP, inside the re-association bound "
-              f"(worst {float((diff / strict).max()):.3g} x the strict tolerance)", flush=True)
+              f"(worst {worst:.3g} x the strict tolerance)", flush=True)
+    allowed = max(2, int(max_via_reorder_ppm * 1e-6 * stats.size))
+    assert stats.via_reorder <= allowed, (f"{what}: {stats.via_reorder} of {stats.size} outputs pass only through the "
+                                          f"re-association bound (at most {allowed} allowed)")
     return stats
+
+
+def via_reorder_summary():
+    """One line per configuration seen so far, then the total."""
+    lines = []
+    for name in sorted(VIA_REORDER_BY_CONFIG):
+        t = VIA_REORDER_BY_CONFIG[name]
+        lines.append(f"{name}: {t['via_reorder']} of {t['elements']} outputs beyond rtol 1e-3 / 1 ULP "
+                     f"(inside the re-association bound; worst {t['worst_x_strict']:.3g} x strict)")
+    t = VIA_REORDER_TOTAL
+    lines.append(f"all comparisons: {t['via_reorder']} of {t['elements']} outputs beyond rtol 1e-3 / 1 ULP "
+                 f"({1e6 * t['via_reorder'] / max(t['elements'], 1):.3g} ppm; worst {t['worst_x_strict']:.3g} x strict)")
+    return lines
 
 
 def reorder_bound(acc: np.ndarray, scale_half: np.ndarray, s_a: np.ndarray) -> np.ndarray:

@@ -46,6 +46,7 @@ def test_replays_repeat_the_eager_calls(gpu_ops):
         fused.append((case, w, xd))
 
     qas = {}
+    static_outs = [torch.empty((p[0].M, p[0].N), dtype=torch.float16, device="cuda") for p in prepared[:1] + prepared[3:4]]
 
     def step():
         """act-quant + GEMM through every form; returns the outputs in a fixed order."""
@@ -62,6 +63,16 @@ def test_replays_repeat_the_eager_calls(gpu_ops):
         outs += gpu_ops.w2a8_gemm_grouped(probs, torch.float16)
         for case, w, xd in fused:
             outs.append(gpu_ops.w2a8_linear_fused(xd, w, torch.float16))
+        # the entry point that allocates nothing (split-K through the library-owned array): its first call on the
+        # device is the eager one below, outside the capture
+        for (case, w, xd, kernel, _), out in zip(prepared[:1] + prepared[3:4], static_outs):
+            qa = qas[case.name]
+            _lib.check(L.slimk_w2a8_gemm_static(
+                qa.q.data_ptr(), qa.q.stride(0), qa.s_a.data_ptr(), qa.rowsum.data_ptr(), qa.rowsum.stride(0),
+                w.w_r.data_ptr(), w.s_r.data_ptr(), None, w.zp_const, case.M, w.N, w.K, w.group_size,
+                out.data_ptr(), out.stride(0), _lib.F16, {"skinny": _lib.KERNEL_SKINNY, "tiled": _lib.KERNEL_TILED}[kernel], 0,
+                torch.cuda.current_stream().cuda_stream))
+            outs.append(out)
         return outs
 
     stream = torch.cuda.Stream()

@@ -432,7 +432,7 @@ def test_workspace_serves_changing_shapes(gpu_ops, oracle):
 
 def test_config_c5_asym_ragged(gpu_ops, oracle):
     a, b = workloads.config_cases("c5")
-    _run_case(gpu_ops, oracle, a, "auto")                  # M = 77 -> tiled, per-group zero-points
+    _run_case(gpu_ops, oracle, a, "auto")                  # M = 77, per-group zero-points: whichever kernel AUTO routes it to
     _run_case(gpu_ops, oracle, b, "auto")                  # M = 1  -> skinny split-K
 
 
@@ -465,6 +465,19 @@ def test_wint2_gemm_keeps_the_repacked_weight_until_it_changes(gpu_ops, oracle):
     y2 = gpu_ops.wint2_gemm(xd, wt, sc)
     assert len(ops_mod._WINT2_CACHE) == 1 and next(iter(ops_mod._WINT2_CACHE.values()))[0] is held
     assert torch.equal(y1, y2)
+    # the documented call form makes a new view object per call: wint2_gemm(x, packed.t(), scale) must hit as well
+    pk = torch.from_numpy(packed).cuda()
+    ops_mod._WINT2_CACHE.clear()
+    ya = gpu_ops.wint2_gemm(xd, pk.t(), sc)
+    held_t = next(iter(ops_mod._WINT2_CACHE.values()))[0]
+    yb = gpu_ops.wint2_gemm(xd, pk.t(), sc)
+    assert len(ops_mod._WINT2_CACHE) == 1 and next(iter(ops_mod._WINT2_CACHE.values()))[0] is held_t
+    assert torch.equal(ya, yb) and torch.equal(ya, y1)
+    # operands made under inference mode have no version counter to read: re-laid every call, same result
+    with torch.inference_mode():
+        pk_i, sc_i = torch.from_numpy(packed).cuda(), torch.from_numpy(scales).cuda()
+        yi = gpu_ops.wint2_gemm(xd, pk_i.t(), sc_i)
+    assert torch.equal(yi, y1)
     ref = oracle.reference_forward(x, packed, scales, zero, 128)
     pu.assert_out_close(pu.out_tensor_bits(y2), ref["out_bits"], False, pu.reorder_bound(ref["acc"], scales, ref["s_a"]), "wint2 cached")
     # an in-place change of the packed weight is seen (version counter): re-laid, new result
@@ -625,10 +638,12 @@ def test_fused_activation_quantisation_matches_two_launches(gpu_ops, oracle, M, 
     two = gpu_ops.w2a8_gemm(gpu_ops.quantize_act_int8(xd, g), w, odt, kernel="skinny", split_k=split)
     torch.cuda.synchronize()
     np.testing.assert_array_equal(pu.out_tensor_bits(fused), pu.out_tensor_bits(two))
-    if xdt == "float16":
-        ref = oracle.reference_forward(x, packed, scales, zero, g, out_bf16=(out == "bfloat16"), want_acc=True)
-        pu.assert_out_close(pu.out_tensor_bits(fused), ref["out_bits"], out == "bfloat16",
-                            pu.reorder_bound(ref["acc"], scales, ref["s_a"]), case.name)
+    # against the oracle as well (bf16 rows go to it as bit patterns)
+    x_or_bits = pu.out_tensor_bits(xd) if xdt == "bfloat16" else x
+    ref = oracle.reference_forward(x_or_bits, packed, scales, zero, g, out_bf16=(out == "bfloat16"), want_acc=True,
+                                   x_bf16=(xdt == "bfloat16"))
+    pu.assert_out_close(pu.out_tensor_bits(fused), ref["out_bits"], out == "bfloat16",
+                        pu.reorder_bound(ref["acc"], scales, ref["s_a"]), case.name)
     # a strided view of a wider buffer, and the layer's forward (which picks the fused path for few rows)
     wide = torch.zeros(M, K + 16, dtype=xd.dtype, device="cuda")
     wide[:, :K] = xd

@@ -96,3 +96,64 @@ def test_random_grouped_launches(gpu_ops, oracle, seed):
         for (_, _, out), (ref, scales), tag in zip(probs, refs, tags):
             pu.assert_out_close(pu.out_tensor_bits(out), ref["out_bits"], odt == "bfloat16",
                                 pu.reorder_bound(ref["acc"], scales, ref["s_a"]), tag)
+
+
+def _blas_reference(oracle, x, packed, scales, zero, g, bf16):
+    """The oracle's forward with the int32 group sums formed by its exact float BLAS product (every partial sum is an
+    integer below 2^24): the same numbers as reference_forward, in a time that allows every row of a chip-filling
+    problem to be checked."""
+    q, s_a, _ = oracle.c_act_quant(x, g)
+    acc = oracle.np_gemm_acc_blas(q, oracle.np_unpack(packed), zero, g, dtype=np.float32)
+    out_bits, _ = oracle.c_epilogue(acc, scales, s_a, bf16)
+    return dict(q=q, s_a=s_a, acc=acc, out_bits=out_bits)
+
+
+@pytest.mark.parametrize("seed", range(2))
+def test_random_split_k_launches_of_more_workgroups_than_run_at_once(gpu_ops, oracle, seed):
+    """Split-K of the tiled kernel (W2 and the one-pass W4 form) on launches of 600 workgroups and more, one or two
+    stages per workgroup: the last workgroups to start publish their partial sums into a memory pipeline that is
+    backed up.  Every output of every row against the oracle (not against the verification instantiation)."""
+    from slimkernels_amd import w4
+    from slimkernels_amd.torch import w4 as tw4
+    rng = random.Random(3000 + seed)
+    for it in range(3):
+        g = rng.choice([64, 128, 256])
+        split = rng.choice([4, 5, 6, 8])
+        per = rng.choice([1, 2]) * (2 if g == 256 else 1)          # stages of 128 elements per split (whole groups of 256)
+        K = 128 * per * split
+        mt = rng.choice([3, 4])                                    # 64-row token tiles
+        M = 64 * mt - rng.choice([0, 1, 30, 62])
+        nt = -(-(600 + rng.randrange(300)) // (mt * split))        # 256-channel tiles: 600..900 workgroups
+        N = 256 * nt - rng.choice([0, 8, 64, 200])
+        mode = rng.choice(["sym", "sym", "asym"])
+        odt = rng.choice(["float16", "bfloat16"])
+        bf16 = odt == "bfloat16"
+        case = pu.small_case(M, N, K, g, mode, seed=rng.randrange(1 << 20), out_dtype=odt)
+        tag = f"M={M} N={N} K={K} g={g} {mode} {odt} tiled split={split} workgroups={mt * nt * split}"
+        print(tag, flush=True)
+        packed, scales, zero = workloads.make_quantized_weight(case)
+        x = workloads.make_activation(case)
+        ref = _blas_reference(oracle, x, packed, scales, zero, g, bf16)
+        w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, x)
+        qa = gpu_ops.quantize_act_int8(xd, g)
+        out = gpu_ops.w2a8_gemm(qa, w, pu.torch_dtype(case), kernel="tiled", split_k=split)
+        out2 = gpu_ops.w2a8_gemm(qa, w, pu.torch_dtype(case), kernel="tiled", split_k=split)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(qa.q.cpu().numpy(), ref["q"])
+        np.testing.assert_array_equal(pu.out_tensor_bits(out), pu.out_tensor_bits(out2))
+        pu.assert_out_close(pu.out_tensor_bits(out), ref["out_bits"], bf16, pu.reorder_bound(ref["acc"], scales, ref["s_a"]), tag)
+        del w, qa, out, out2
+        if g == 256:
+            continue
+        # the same launch shape through the one-pass 4-bit form of the body (uniform zero-point 8)
+        rngw = np.random.default_rng(rng.randrange(1 << 20))
+        w4f = (rngw.standard_normal((N, K), dtype=np.float32) * np.float32(0.02)).astype(np.float16).astype(np.float32)
+        packed4, scales4, zp4 = w4.prepare_w4(w4f, g, "sym")
+        ref4 = oracle.w4_reference_forward(x, w4.unpack_w4(packed4), scales4, zp4, g, out_bf16=bf16)
+        w4d = tw4.repack_w4(packed4, scales4, zp4, g)
+        qa = gpu_ops.quantize_act_int8(xd, g)
+        print(tag.replace("tiled", "W4 one pass"), flush=True)
+        y = tw4.w4a8_gemm_one_pass(qa, w4d, pu.torch_dtype(case), split_k=split)
+        torch.cuda.synchronize()
+        pu.assert_out_close(pu.out_tensor_bits(y), ref4["out_bits"], bf16, pu.reorder_bound(ref4["acc"], scales4, ref4["s_a"]),
+                            tag + " W4 one pass")
