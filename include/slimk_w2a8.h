@@ -77,7 +77,12 @@ enum slimk_kernel {
     SLIMK_KERNEL_AUTO = 0,   /* skinny for M <= 32; for 33..256 rows whichever of the two skinny forms and the tiled
                                 kernel is predicted the fastest (slimk_w2a8_gemm_auto_route tells which); tiled beyond */
     SLIMK_KERNEL_SKINNY = 1, /* weight-streaming split-K kernel, M <= 256 (16 rows per pass over the weights) */
-    SLIMK_KERNEL_TILED = 2   /* LDS-pipelined MFMA tile kernel, any M */
+    SLIMK_KERNEL_TILED = 2,  /* LDS-pipelined MFMA tile kernel, any M */
+    SLIMK_KERNEL_MID = 3     /* workgroups of four 64-channel strips x up to 96 token rows, activations shared through LDS,
+                                weights streamed once straight to registers, K split across workgroups: M <= 128, groups
+                                of up to 256; split workspace sized as for SLIMK_KERNEL_SKINNY.  On request only:
+                                SLIMK_KERNEL_AUTO never takes it (measured behind the other forms on every shape tried:
+                                11008 x 4096 at 64 rows 19.6 us against 13.3, 28672 x 8192 at 128 rows 56.8 against 49.6) */
 };
 
 /* what the optional int32 verification buffer receives */

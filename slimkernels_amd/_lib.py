@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_CSRC, "libslimk_w2a8.so")
 
 OK = 0
 F16, BF16 = 0, 1
-KERNEL_AUTO, KERNEL_SKINNY, KERNEL_TILED = 0, 1, 2
+KERNEL_AUTO, KERNEL_SKINNY, KERNEL_TILED, KERNEL_MID = 0, 1, 2, 3
 DUMP_NONE, DUMP_GROUPS, DUMP_SUM = 0, 1, 2
 QUANT_REF, QUANT_SYM, QUANT_ASYM = 0, 1, 2
 

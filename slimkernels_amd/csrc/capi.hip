@@ -179,6 +179,27 @@ MidRoute mid_route(int M, int N, int K, int group_size) {
     return shared_cost <= tiled_cost ? kMidShared : kMidTiled;
 }
 
+// The kernel for 33..128 rows (a workgroup = four strips x the rows of a row part): K splits across workgroups in
+// rounds of four pieces (a piece = two 64-element steps, one with groups of 64).  The launch aims at about three
+// workgroups for two CUs and keeps two rounds per workgroup (11008 x 4096 at 64 rows: 33.1 / 25.1 / 19.6 / 22.0 us at
+// 1 / 2 / 4 / 8 splits; 28672 x 8192 at 128 rows, groups of 128: 62.1 / 56.8 / 64.3 us at 1 / 2 / 4).
+int mid_groups_per_split(int G, int group_size, int split) {
+    const int gs = group_size / w2a8::kStepK;
+    const int round_groups = std::max(1, w2a8::mid::kPiecesPerRound * w2a8::mid::piece_steps(gs) / gs);  // groups per round
+    const int gps = (G + split - 1) / split;
+    return (gps + round_groups - 1) / round_groups * round_groups;
+}
+int mid_split(int M, int N, int K, int group_size) {
+    const int units = (strips_of(N) + w2a8::mid::kWaves - 1) / w2a8::mid::kWaves * w2a8::mid_row_parts(M);
+    const int G = K / group_size, gs = group_size / w2a8::kStepK;
+    const int pieces = K / w2a8::kStepK / w2a8::mid::piece_steps(gs);
+    int split = std::max(1, (384 + units / 2) / units);
+    split = std::min(split, std::max(1, pieces / (2 * w2a8::mid::kPiecesPerRound)));
+    if (split > 32) split = 32;
+    const int gps = mid_groups_per_split(G, group_size, split);
+    return (G + gps - 1) / gps;
+}
+
 int resolve_kernel(int M, int N, int K, int group_size, int kernel) {
     if (kernel == SLIMK_KERNEL_AUTO)
         return M <= 32 || mid_route(M, N, K, group_size) != kMidTiled ? SLIMK_KERNEL_SKINNY : SLIMK_KERNEL_TILED;
@@ -197,6 +218,7 @@ bool skinny_shared_applies(int M, int N, int K, int group_size) {
 }
 
 int auto_split(int M, int N, int K, int group_size, int kernel) {
+    if (kernel == SLIMK_KERNEL_MID) return mid_split(M, N, K, group_size);
     if (kernel != SLIMK_KERNEL_SKINNY) {
         // the fast tiled kernel splits K when its tiles would leave CUs idle (groups of up to 256)
         if (group_size > 256) return 1;
@@ -266,7 +288,7 @@ size_t slimk_w2a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int 
     if (split_k <= 0) split_k = auto_split(M, N, K, group_size, kern);
     if (split_k <= 1) return 0;
     const int strips = strips_of(N);
-    if (kern != SLIMK_KERNEL_SKINNY) {  // one arrival counter and `split_k` fp32 tiles of 64 x 256 per 64-row tile
+    if (kern == SLIMK_KERNEL_TILED) {  // one arrival counter and `split_k` fp32 tiles of 64 x 256 per 64-row tile
         const size_t tiles = w2a8::tiled_fast_workspace_tiles(M, strips, group_size / w2a8::kStepK);
         return kCounterBlockBytes + (size_t)split_k * tiles * 64 * 256 * sizeof(float);
     }
@@ -377,13 +399,14 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
     if (M <= 0 || N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "M=%d, N=%d must be positive", M, N);
     if (int rc = check_kg(K, group_size)) return rc;
     // the row sums fold zero-points; the fast tiled kernel centres its operand bytes on 2 and reads none for that value
-    const bool rowsum_unused = !zp_r && zp_const == 2 && resolve_kernel(M, N, K, group_size, kernel) == SLIMK_KERNEL_TILED &&
-                               group_size <= 256;
+    const int kern_for_rowsum = resolve_kernel(M, N, K, group_size, kernel);
+    const bool rowsum_unused = !zp_r && zp_const == 2 && group_size <= 256 &&
+                               (kern_for_rowsum == SLIMK_KERNEL_TILED || kern_for_rowsum == SLIMK_KERNEL_MID);
     if (!rowsum && !rowsum_unused)
-        return fail(SLIMK_ERR_NULL_POINTER, "gemm: rowsum is NULL (only the tiled kernel with the uniform zero-point 2 and a group size of at most 256 does without)");
+        return fail(SLIMK_ERR_NULL_POINTER, "gemm: rowsum is NULL (only the tiled kernel and the one for 33..128 rows, with the uniform zero-point 2 and a group size of at most 256, do without)");
     if (!rowsum) ldr = (M + 3) / 4 * 4;
     if (out_dtype != SLIMK_F16 && out_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "out_dtype=%d", out_dtype);
-    if (kernel < SLIMK_KERNEL_AUTO || kernel > SLIMK_KERNEL_TILED) return fail(SLIMK_ERR_BAD_ENUM, "kernel=%d", kernel);
+    if (kernel < SLIMK_KERNEL_AUTO || kernel > SLIMK_KERNEL_MID) return fail(SLIMK_ERR_BAD_ENUM, "kernel=%d", kernel);
     if (dump_mode < SLIMK_DUMP_NONE || dump_mode > SLIMK_DUMP_SUM) return fail(SLIMK_ERR_BAD_ENUM, "dump_mode=%d", dump_mode);
     if (dump_mode != SLIMK_DUMP_NONE && !acc_dump) return fail(SLIMK_ERR_NULL_POINTER, "gemm: dump_mode set but acc_dump is NULL");
     if (ldq < K || ldo < N || ldr < M) return fail(SLIMK_ERR_BAD_SHAPE, "gemm: ldq=%d, ldo=%d or ldr=%d too small", ldq, ldo, ldr);
@@ -397,6 +420,9 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
     const int kern = resolve_kernel(M, N, K, group_size, kernel);
     if (kern == SLIMK_KERNEL_SKINNY && M > kSkinnyMaxRows)
         return fail(SLIMK_ERR_UNSUPPORTED, "the skinny kernel handles M <= %d (M=%d)", kSkinnyMaxRows, M);
+    if (kern == SLIMK_KERNEL_MID && (M > w2a8::kMidMaxRows || group_size > 256))
+        return fail(SLIMK_ERR_UNSUPPORTED, "SLIMK_KERNEL_MID handles M <= %d and groups of up to 256 (M=%d, group_size=%d)",
+                    w2a8::kMidMaxRows, M, group_size);
     const int G = K / group_size;
     const bool split_chosen_here = split_k <= 0;
     if (split_k <= 0) {
@@ -425,8 +451,8 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
             split_k = w2a8::tiled_fast_effective_split(K / w2a8::kStepK, gs_t, split_k, &gps);
         if (split_k <= 1) gps = G;
     } else {
-        gps = groups_per_split(G, group_size, split_k);
-        split_k = (G + gps - 1) / gps;  // effective split: the request is an upper bound (whole chunks per split)
+        gps = kern == SLIMK_KERNEL_MID ? mid_groups_per_split(G, group_size, split_k) : groups_per_split(G, group_size, split_k);
+        split_k = (G + gps - 1) / gps;  // effective split: the request is an upper bound (whole chunks / rounds per split)
     }
 
     w2a8::GemmParams p{};
@@ -445,12 +471,14 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
                         split_k, need, workspace_bytes);
         if (fit_split)
             if (int rc = static_workspace(&workspace, (hipStream_t)stream)) return rc;
+        if (need - kCounterBlockBytes >= 0x7fffffffu)
+            return fail(SLIMK_ERR_UNSUPPORTED, "split_k=%d: %zu bytes of partial sums, 2 GiB or more", split_k, need - kCounterBlockBytes);
         if (!workspace) return fail(SLIMK_ERR_WORKSPACE, "split_k=%d needs a workspace of %zu bytes", split_k, need);
         if (workspace_bytes < need)
             return fail(SLIMK_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, need);
         if (!aligned16(workspace)) return fail(SLIMK_ERR_MISALIGNED, "workspace must be 16-byte aligned");
         p.ws_counter = reinterpret_cast<unsigned*>(workspace);
-        const int counters = kern == SLIMK_KERNEL_SKINNY ? p.strips * ((M + 15) / 16)
+        const int counters = kern != SLIMK_KERNEL_TILED ? p.strips * ((M + 15) / 16)
                                                          : (int)w2a8::tiled_fast_workspace_tiles(M, p.strips, group_size / w2a8::kStepK);
         if (counters > kMaxCounters)
             return fail(SLIMK_ERR_UNSUPPORTED, "split_k over %d output tiles (at most %d arrival counters)", counters, kMaxCounters);
@@ -466,6 +494,8 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
     const bool out_bf16 = out_dtype == SLIMK_BF16;
     // a call with a dump runs the verification instantiation of the kernel the same call without one would run
     const bool dump = p.acc_dump != nullptr;
+    if (kern == SLIMK_KERNEL_MID)
+        return hip_result(dump ? w2a8::launch_mid_verify(p, gs, asym, out_bf16, st) : w2a8::launch_mid(p, gs, asym, out_bf16, st), "mid gemm");
     if (kern == SLIMK_KERNEL_SKINNY && skinny_shared_applies(M, N, K, group_size))
         return hip_result(dump ? w2a8::launch_skinny_shared_verify(p, gs, skinny_shared_parts(M, N), asym, out_bf16, st)
                                : w2a8::launch_skinny_shared(p, gs, skinny_shared_parts(M, N), asym, out_bf16, st), "shared skinny gemm");

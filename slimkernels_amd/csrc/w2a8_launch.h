@@ -52,6 +52,28 @@ hipError_t launch_skinny_verify(const GemmParams& p, int gs, int waves, bool asy
 hipError_t launch_skinny_shared_verify(const GemmParams& p, int gs, int kparts, bool asym, bool out_bf16, hipStream_t stream);
 hipError_t launch_skinny_grouped_verify(const GroupedParams& gp, int gs, bool asym, bool out_bf16, hipStream_t stream);
 
+// 33..128 token rows: one workgroup per set of four strips (a wave each) and row part (up to six blocks of 16 rows;
+// 97..128 rows run as two parts of four blocks), K split over blockIdx.y in whole groups (p.groups_per_split); the
+// split workspace holds one fp32 tile of 16 x 64 per strip, row block and split and one arrival counter per strip and
+// row block, as the one-strip kernel's does.  launch_mid_verify: the instantiations with the int32 dump.
+constexpr int kMidMaxRows = 128;
+namespace mid {
+constexpr int kWaves = 4;           // strips per workgroup
+constexpr int kSlots = 4;           // pieces of activations in LDS
+constexpr int kPiecesPerRound = 4;  // pieces per unrolled round of the main loop (a piece's ring slot is compile-time)
+__host__ __device__ constexpr int piece_steps(int GS) { return GS >= 2 ? 2 : 1; }   // 64-element steps per piece
+__host__ __device__ constexpr int frags_per_wave(int MB, int GS) { return (MB * piece_steps(GS) + kWaves - 1) / kWaves; }
+}  // namespace mid
+// row blocks a launch is instantiated for (3..6) and the row parts it runs as
+inline int mid_row_parts(int M) { return (M + 15) / 16 > 6 ? 2 : 1; }
+inline int mid_row_blocks(int M) {
+    const int mb = (M + 15) / 16;
+    return mb > 6 ? 4 : (mb < 3 ? 3 : mb);
+}
+
+hipError_t launch_mid(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
+hipError_t launch_mid_verify(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);
+
 // 4-bit weights as two planes (w_r over 2 * p.steps steps, s_r over 2 * p.G groups), uniform zero-point 8, one pass
 // over K: p.K / p.steps / p.G describe K, not 2K; gs 1 or 2; p.steps even
 // p.split > 1: K split over blockIdx.y in whole 128-element stages (p.groups_per_split), workspace = one arrival

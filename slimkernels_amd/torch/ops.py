@@ -210,7 +210,7 @@ def w2a8_gemm(qa: QuantizedActivation, w: W2A8Weight, out_dtype=torch.float16, *
     """out[M, N] = dequant( q @ (codes - zp)^T ).  Returns out, or (out, acc) when ``dump`` is
     "groups" (int32 [M, N, G]) or "sum" (int32 [M, N])."""
     L = _lib.lib()
-    kern = {"auto": _lib.KERNEL_AUTO, "skinny": _lib.KERNEL_SKINNY, "tiled": _lib.KERNEL_TILED}[kernel]
+    kern = {"auto": _lib.KERNEL_AUTO, "skinny": _lib.KERNEL_SKINNY, "tiled": _lib.KERNEL_TILED, "mid": _lib.KERNEL_MID}[kernel]
     M, K = qa.q.shape
     if K != w.K or qa.group_size != w.group_size:
         raise ValueError(f"activation K={K}/group {qa.group_size} does not match weight K={w.K}/group {w.group_size}")

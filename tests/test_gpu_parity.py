@@ -283,6 +283,27 @@ def test_skinny_shared_more_than_32_rows(gpu_ops, oracle, M, N, K, g, mode, out,
     _run_case(gpu_ops, oracle, case, "skinny", split_k=split)
 
 
+@pytest.mark.parametrize("M,N,K,g,mode,out,split", [
+    (33, 4000, 4096, 128, "sym", "float16", 0),      # three row blocks, the last with one row
+    (77, 2752, 4096, 128, "asym", "float16", 0),     # five row blocks, per-group zero-points
+    (128, 1000, 8192, 64, "sym", "bfloat16", 0),     # two row parts of four blocks, groups of 64
+    (100, 520, 2560, 256, "ref", "float16", 2),      # row parts of four and three blocks, groups of 256 (two pieces each), one strip in the last set
+    (64, 300, 1024, 64, "asym", "float16", 1),       # four row blocks, ragged last strip
+    (90, 200, 1536, 128, "sym", "bfloat16", 3),      # six row blocks
+    (48, 128, 192, 64, "sym", "float16", 1),         # three pieces: a round with a dead piece
+    (40, 64, 256, 256, "ref", "float16", 1),         # a single group
+    (20, 192, 2048, 128, "asym", "float16", 2),      # fewer rows than the form is meant for
+    (112, 700, 2048, 128, "asym", "bfloat16", 0),    # seven row blocks: row parts of four and three
+    (96, 1100, 3072, 256, "sym", "float16", 4),      # six row blocks, groups of 256, ragged last strip set
+])
+def test_mid_kernel(gpu_ops, oracle, M, N, K, g, mode, out, split):
+    """SLIMK_KERNEL_MID (a workgroup = four strips x up to six blocks of 16 token rows, the activations shared through
+    LDS, K split across workgroups): int32 group sums exact, the output criterion, verification and production bits equal."""
+    case = pu.small_case(M, N, K, g, mode, seed=M + N + K, out_dtype=out)
+    _run_case(gpu_ops, oracle, case, "mid", split_k=split, dump="groups")
+    _run_case(gpu_ops, oracle, case, "mid", split_k=split, dump="sum")
+
+
 @pytest.mark.parametrize("M,N,K,g,mode,out", SMALL + [
     (77, 200, 512, 128, "asym", "float16"),
     (129, 130, 320, 64, "sym", "float16"),
