@@ -435,9 +435,14 @@ def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, d
             ops.w2a8_gemm(qa, w, torch.float16, out=out)
             us = time_graph(torch, lambda: [ops.w2a8_gemm(qa, w, torch.float16, out=out) for _ in range(4)], 4)
             tops = workloads.algorithmic_ops(c) / (us * 1e-6) / 1e12
-            aq_us = time_graph(torch, lambda: [ops.quantize_act_int8(x, 128) for _ in range(4)], 4)
+            # the quantiser as W2A8Linear runs it in front of this GEMM: without the group sums where the kernel the
+            # library picks does not read them (the tiled kernel with the symmetric levels), and with them for comparison
+            sums = ops.needs_rowsum(M, w)
+            aq_us = time_graph(torch, lambda: [ops.quantize_act_int8(x, 128, rowsum=sums) for _ in range(4)], 4)
+            aq_sums_us = time_graph(torch, lambda: [ops.quantize_act_int8(x, 128) for _ in range(4)], 4)
             pre.append({"shape": f"{N}x{K}", "M": M, "us": round(us, 1), "TOPS": round(tops, 1),
-                        "frac_int8_mfma": round(tops / INT8_PEAK_TOPS, 4), "act_quant_us": round(aq_us, 1)})
+                        "frac_int8_mfma": round(tops / INT8_PEAK_TOPS, 4), "act_quant_us": round(aq_us, 1),
+                        "act_quant_group_sums": bool(sums), "act_quant_with_sums_us": round(aq_sums_us, 1)})
     detail["prefill"] = pre
 
     # ---- the other configurations (c4: Llama-70B-class linears, group 64, bf16 out; c5: ragged shapes

@@ -29,6 +29,7 @@ def test_replays_repeat_the_eager_calls(gpu_ops):
         (100, 1000, 12288, 128, "sym", "auto"),      # 33..256 rows
         (64, 4096, 4096, 128, "sym", "tiled"),       # tiled split-K
         (300, 520, 1024, 64, "ref", "tiled"),        # tiled, unsplit, zero-point prologue
+        (80, 2048, 8192, 128, "asym", "mid"),        # the 33..128-row kernel, split-K (counters reset in the kernel)
     ]
     prepared = []
     for i, (M, N, K, g, mode, kernel) in enumerate(singles):
@@ -36,6 +37,7 @@ def test_replays_repeat_the_eager_calls(gpu_ops):
         prepared.append((case, w, xd, kernel, torch.empty((M, N), dtype=torch.float16, device="cuda")))
     assert L.slimk_w2a8_gemm_auto_split_k(16, 1024, 14336, 128, _lib.KERNEL_SKINNY) > 1
     assert L.slimk_w2a8_gemm_auto_split_k(64, 4096, 4096, 128, _lib.KERNEL_TILED) > 1
+    assert L.slimk_w2a8_gemm_auto_split_k(80, 2048, 8192, 128, _lib.KERNEL_MID) > 1
     grouped = []
     for i, (M, N, K) in enumerate([(1, 2048, 4096), (16, 520, 2048), (32, 1024, 8192)]):
         case, w, xd = _prepare(gpu_ops, M, N, K, 128, "sym", 950 + i)

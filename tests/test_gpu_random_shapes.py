@@ -35,8 +35,10 @@ def test_random_single_gemms(gpu_ops, oracle, seed):
     checked = 0
     for _ in range(25):
         case = _random_case(rng, 300)
-        kernel = rng.choice(["auto", "auto", "skinny", "tiled"])
+        kernel = rng.choice(["auto", "auto", "skinny", "tiled", "mid"])
         if kernel == "skinny" and case.M > 32:
+            kernel = "auto"
+        if kernel == "mid" and case.M > 128:
             kernel = "auto"
         split = 0 if rng.random() < 0.5 else rng.randint(1, 8)
         tag = f"M={case.M} N={case.N} K={case.K} g={case.group_size} {case.mode} {case.out_dtype} {kernel} split={split}"
