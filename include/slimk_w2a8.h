@@ -74,15 +74,16 @@ enum slimk_dtype { SLIMK_F16 = 0, SLIMK_BF16 = 1 };
 
 /* which GEMM kernel slimk_w2a8_gemm runs */
 enum slimk_kernel {
-    SLIMK_KERNEL_AUTO = 0,   /* skinny for M <= 32; for 33..256 rows whichever of the two skinny forms and the tiled
-                                kernel is predicted the fastest (slimk_w2a8_gemm_auto_route tells which); tiled beyond */
+    SLIMK_KERNEL_AUTO = 0,   /* skinny for M <= 32; for 33..256 rows whichever of the two skinny forms, the tiled kernel
+                                and SLIMK_KERNEL_MID is predicted the fastest (slimk_w2a8_gemm_auto_route tells which);
+                                tiled beyond */
     SLIMK_KERNEL_SKINNY = 1, /* weight-streaming split-K kernel, M <= 256 (16 rows per pass over the weights) */
     SLIMK_KERNEL_TILED = 2,  /* LDS-pipelined MFMA tile kernel, any M */
     SLIMK_KERNEL_MID = 3     /* workgroups of four 64-channel strips x up to 96 token rows, activations shared through LDS,
                                 weights streamed once straight to registers, K split across workgroups: M <= 128, groups
-                                of up to 256; split workspace sized as for SLIMK_KERNEL_SKINNY.  On request only:
-                                SLIMK_KERNEL_AUTO never takes it (measured behind the other forms on every shape tried:
-                                11008 x 4096 at 64 rows 19.6 us against 13.3, 28672 x 8192 at 128 rows 56.8 against 49.6) */
+                                of up to 256; split workspace sized as for SLIMK_KERNEL_SKINNY.  SLIMK_KERNEL_AUTO takes
+                                it for 33..48 and 65..80 rows on matrices of 32 MiB and more (where 64-row tiles would be
+                                mostly empty: 8..19 % faster than the tiled kernel there), nowhere else */
 };
 
 /* what the optional int32 verification buffer receives */
@@ -120,7 +121,7 @@ size_t slimk_w2a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int 
 /* Which kernel form SLIMK_KERNEL_AUTO takes for this problem: 1 = skinny, one 64-channel strip per workgroup;
  * 2 = tiled; 3 = skinny, workgroups of several strips that share the activations (12..16 token rows on 384 strips
  * and more, 17..32 rows on matrices of 24 MiB or more, and the problems of 33..256 rows for which it is predicted
- * the fastest of the three).
+ * the fastest of the three); 4 = SLIMK_KERNEL_MID (33..48 and 65..80 rows on matrices of 32 MiB and more).
  * 0 for a shape the library does not take.  A query for tests and tuning; no upstream counterpart (upstream's
  * launcher has one kernel with one fixed tiling, slimkernels/cute/gemm/wgmma_sm90_W2A8.cu:448-450). */
 int slimk_w2a8_gemm_auto_route(int M, int N, int K, int group_size);

@@ -126,7 +126,8 @@ int skinny_plain_split(int N, int K, int group_size) {
     return (G + gps - 1) / gps;
 }
 
-// 33..256 token rows: three kernels can take the problem.
+// 33..256 token rows: three kernels can take the problem (and, for some row counts on large matrices, a fourth: see
+// mid_route).
 //   plain  - the one-strip skinny kernel, 16 rows at a time, the passes side by side as workgroups of their own (each
 //            re-reading weights and activations, all but the first out of L2): the fastest while the workgroups are
 //            few (4096 x 4096: 5.6 us at 33 rows, tiled 17.3).
@@ -144,13 +145,30 @@ int skinny_plain_split(int N, int K, int group_size) {
 // (worst case 33 %; the rule by size it replaces: 4.2 % on the same cases and up to 85 %).
 // Reductions of up to 2048 elements keep the rule they were measured with (plain while its passes over the weights
 // stay under 100 MiB).
-enum MidRoute { kMidPlain, kMidShared, kMidTiled };
+enum MidRoute { kMidPlain, kMidShared, kMidTiled, kMidStrips };
+// Where the tiled kernel would leave most of a 64-row tile empty - 33..48 and 65..80 rows - on a matrix of 32 MiB and
+// more, the kernel with every row in one workgroup (SLIMK_KERNEL_MID) is ahead of it: 28672 x 8192 (groups of 64)
+// 36.7 -> 32.3 us at 33 rows and 57.6 -> 46.4 at 80, 8192 x 28672 41.1 -> 36.2 and 56.1 -> 51.1, 12288 x 12288 (groups
+// of 128) 28.2 -> 25.5 and 37.1 -> 34.3, 16384 x 16384 34.3 -> 31.5 and 51.4 -> 42.4.  At 49..64 and from 81 rows on
+// the tiled kernel keeps the lead (full tiles), and on smaller matrices the skinny forms do.
+bool mid_strips_rows(int M) { return (M >= 33 && M <= 48) || (M >= 65 && M <= 80); }
+MidRoute mid_route_of_three(int M, int N, int K, int group_size);
 MidRoute mid_route(int M, int N, int K, int group_size) {
+    const MidRoute r = mid_route_of_three(M, N, K, group_size);
+    const size_t weight_bytes = (size_t)strips_of(N) * 64 * (K / 4);
+    if (!mid_strips_rows(M) || group_size > 256) return r;
+    if (r == kMidTiled && weight_bytes >= ((size_t)32 << 20)) return kMidStrips;
+    // (long reductions a little below that size, whichever of the three the prediction names: 7168 x 16384, groups of 64,
+    // 32.5 us through the shared-activation workgroups, 29.2 tiled, 26.2 here at 33 rows; 37.5 / 39.1 / 35.9 at 65)
+    if (K >= 16384 && weight_bytes >= ((size_t)24 << 20)) return kMidStrips;
+    return r;
+}
+MidRoute mid_route_of_three(int M, int N, int K, int group_size) {
     if (M > kSkinnyMaxRows) return kMidTiled;
     const int strips = strips_of(N), steps = K / w2a8::kStepK, blocks = (M + 15) / 16;
     const size_t weight_bytes = (size_t)strips * 64 * (K / 4);
     if (K <= 2048) return (size_t)blocks * weight_bytes <= ((size_t)100 << 20) ? kMidPlain : kMidTiled;
-    if (K > 4096 && weight_bytes > ((size_t)32 << 20)) return kMidTiled;  // (28672 x 8192: tiled ahead at every row count)
+    if (K > 4096 && weight_bytes > ((size_t)32 << 20)) return kMidTiled;  // (28672 x 8192: tiled ahead of both skinny forms at every row count)
     const float weight_mib = (float)weight_bytes / 1048576.0f;
     const auto rounds = [](long long wgs, float smooth) {  // between whole rounds and the plain ratio
         const float whole = (float)((wgs + 255) / 256), ratio = std::max(1.0f, (float)wgs / 256.0f);
@@ -180,9 +198,11 @@ MidRoute mid_route(int M, int N, int K, int group_size) {
 }
 
 // The kernel for 33..128 rows (a workgroup = four strips x the rows of a row part): K splits across workgroups in
-// rounds of four pieces (a piece = two 64-element steps, one with groups of 64).  The launch aims at about three
-// workgroups for two CUs and keeps two rounds per workgroup (11008 x 4096 at 64 rows: 33.1 / 25.1 / 19.6 / 22.0 us at
-// 1 / 2 / 4 / 8 splits; 28672 x 8192 at 128 rows, groups of 128: 62.1 / 56.8 / 64.3 us at 1 / 2 / 4).
+// rounds of four pieces (a piece = two 64-element steps, one with groups of 64).  Two workgroups on a CU run side by
+// side in about the time of one, a third waits for a place: the split is the largest power of two (up to 8) that keeps
+// the launch within 512 workgroups and every workgroup at two rounds or more (28672 x 8192 at 33 rows, 112 strip sets:
+// 59.7 / 38.1 / 39.4 / 32.3 / 39.2 / 36.6 us at 1 / 2 / 3 / 4 / 6 / 8 splits; splits that are no power of two measured
+// behind their neighbours on every shape).
 int mid_groups_per_split(int G, int group_size, int split) {
     const int gs = group_size / w2a8::kStepK;
     const int round_groups = std::max(1, w2a8::mid::kPiecesPerRound * w2a8::mid::piece_steps(gs) / gs);  // groups per round
@@ -193,16 +213,18 @@ int mid_split(int M, int N, int K, int group_size) {
     const int units = (strips_of(N) + w2a8::mid::kWaves - 1) / w2a8::mid::kWaves * w2a8::mid_row_parts(M);
     const int G = K / group_size, gs = group_size / w2a8::kStepK;
     const int pieces = K / w2a8::kStepK / w2a8::mid::piece_steps(gs);
-    int split = std::max(1, (384 + units / 2) / units);
-    split = std::min(split, std::max(1, pieces / (2 * w2a8::mid::kPiecesPerRound)));
-    if (split > 32) split = 32;
+    int split = 1;
+    while (split < 8 && units * split * 2 <= 512 && pieces / (split * 2) >= 2 * w2a8::mid::kPiecesPerRound) split *= 2;
     const int gps = mid_groups_per_split(G, group_size, split);
     return (G + gps - 1) / gps;
 }
 
 int resolve_kernel(int M, int N, int K, int group_size, int kernel) {
-    if (kernel == SLIMK_KERNEL_AUTO)
-        return M <= 32 || mid_route(M, N, K, group_size) != kMidTiled ? SLIMK_KERNEL_SKINNY : SLIMK_KERNEL_TILED;
+    if (kernel == SLIMK_KERNEL_AUTO) {
+        if (M <= 32) return SLIMK_KERNEL_SKINNY;
+        const MidRoute r = mid_route(M, N, K, group_size);
+        return r == kMidTiled ? SLIMK_KERNEL_TILED : (r == kMidStrips ? SLIMK_KERNEL_MID : SLIMK_KERNEL_SKINNY);
+    }
     return kernel;
 }
 
@@ -278,7 +300,9 @@ int slimk_w2a8_gemm_auto_split_k(int M, int N, int K, int group_size, int kernel
 
 int slimk_w2a8_gemm_auto_route(int M, int N, int K, int group_size) {
     if (M <= 0 || N <= 0 || !shape_ok(K, group_size)) return 0;
-    if (resolve_kernel(M, N, K, group_size, SLIMK_KERNEL_AUTO) == SLIMK_KERNEL_TILED) return 2;
+    const int kern = resolve_kernel(M, N, K, group_size, SLIMK_KERNEL_AUTO);
+    if (kern == SLIMK_KERNEL_TILED) return 2;
+    if (kern == SLIMK_KERNEL_MID) return 4;
     return skinny_shared_applies(M, N, K, group_size) ? 3 : 1;
 }
 

@@ -102,9 +102,9 @@ __device__ __forceinline__ void mid_body(const GemmParams& p) {
         a_dst[j] = on ? f * 256 : -1;
     }
 
-    // the token scales of the row part, parked in LDS for the end (the first barrier of the loop, or the one after
-    // it, lies between this write and their use)
-    if (tid < MB * 16) sa_lds[tid] = p.s_a[min(row0 + tid, p.M - 1)];
+    // the token scales of the row part: asked for first, parked in LDS for the end once the pipeline's first loads are
+    // out (parking them here would hold those loads back by a trip to memory)
+    const float sa_mine = p.s_a[min(row0 + min(tid, MB * 16 - 1), p.M - 1)];
 
     float t[MB][4][4];
 #pragma unroll
@@ -199,6 +199,8 @@ __device__ __forceinline__ void mid_body(const GemmParams& p) {
         }
     }
 
+    if (tid < MB * 16) sa_lds[tid] = sa_mine;   // (the barrier after the loop lies between this write and its readers)
+
     v4i acc[2][4];
 #pragma unroll
     for (int a = 0; a < 2; ++a)
@@ -249,15 +251,17 @@ __device__ __forceinline__ void mid_body(const GemmParams& p) {
             const uint32_t* const slot = &lds[u * (kFrags * 256) + lane * 4];
             const int g = first_step(piece) / GS;
             // row blocks: MFMAs of block mb into accumulator set mb & 1, the drain of block mb - 1 woven in between; the
-            // fragment after the one in use is read from LDS while the MFMAs of the one in use run
+            // two fragments after the one in use are on their way from LDS while the MFMAs of the one in use run
             v4i a_nxt = *reinterpret_cast<const v4i*>(slot);
+            v4i a_nxt2 = kFrags > 1 ? *reinterpret_cast<const v4i*>(slot + 256) : v4i{0, 0, 0, 0};
 #pragma unroll
             for (int mb = 0; mb <= MB; ++mb) {
                 const int cur = mb & 1, prev = cur ^ 1;
 #pragma unroll
                 for (int s = 0; s < P; ++s) {
                     const v4i a = a_nxt;
-                    if (mb * P + s + 1 < kFrags) a_nxt = *reinterpret_cast<const v4i*>(slot + (mb * P + s + 1) * 256);
+                    a_nxt = a_nxt2;
+                    if (mb * P + s + 2 < kFrags) a_nxt2 = *reinterpret_cast<const v4i*>(slot + (mb * P + s + 2) * 256);
 #pragma unroll
                     for (int pp = 0; pp < 4; ++pp) {
                         if (mb < MB) acc[cur][pp] = mfma_i8_16x16x64(a, b[s][pp], s == 0 ? v4i{0, 0, 0, 0} : acc[cur][pp]);

@@ -186,10 +186,10 @@ def quantize_act_int8(x: torch.Tensor, group_size: int = 128, copies: int = 1, r
 
 def needs_rowsum(M: int, w: "W2A8Weight") -> bool:
     """Whether ``w2a8_gemm(..., kernel="auto")`` of M token rows on this weight reads the activation's group sums:
-    everything but the tiled kernel on the symmetric levels (uniform zero-point 2) does."""
+    everything but the tiled kernel and the kernel for 33..128 rows on the symmetric levels (uniform zero-point 2) does."""
     if w.zp_r is not None or w.zp_const != 2 or w.group_size > 256:
         return True
-    return _lib.lib().slimk_w2a8_gemm_auto_route(M, w.N, w.K, w.group_size) != 2
+    return _lib.lib().slimk_w2a8_gemm_auto_route(M, w.N, w.K, w.group_size) not in (2, 4)
 
 
 def _workspace(w: W2A8Weight, nbytes: int) -> Optional[torch.Tensor]:

@@ -69,7 +69,7 @@ def test_split_heuristic_and_workspace(L):
 
 
 def test_auto_route(L):
-    """Which kernel form AUTO takes: 1 one-strip skinny, 2 tiled, 3 shared-activation skinny."""
+    """Which kernel form AUTO takes: 1 one-strip skinny, 2 tiled, 3 shared-activation skinny, 4 the 33..128-row kernel."""
     route = L.slimk_w2a8_gemm_auto_route
     assert route(1, 4096, 4096, 128) == 1 and route(11, 28672, 8192, 64) == 1 and route(16, 14336, 8192, 64) == 1
     assert route(12, 28672, 8192, 64) == 3 and route(16, 28672, 8192, 64) == 3   # 12..16 rows on 384 strips and more
@@ -79,6 +79,11 @@ def test_auto_route(L):
     assert route(77, 11008, 4096, 128) == 3         # five row blocks on 172 strips: the shared-activation workgroups
     assert route(64, 4096, 14336, 128) == 3         # long reduction, few 256-channel tiles
     assert route(128, 28672, 8192, 64) == 2
+    # rows that would leave a 64-row tile mostly empty, on matrices of 32 MiB and more: every row in one workgroup
+    assert route(33, 28672, 8192, 64) == 4 and route(48, 8192, 28672, 128) == 4 and route(80, 16384, 16384, 128) == 4
+    assert route(49, 28672, 8192, 64) == 2 and route(64, 28672, 8192, 64) == 2 and route(81, 28672, 8192, 64) == 2
+    assert route(40, 7168, 16384, 64) == 4          # a long reduction from 24 MiB on
+    assert route(40, 14336, 4096, 128) in (1, 3) and route(40, 10240, 8192, 128) in (1, 3)   # smaller matrices stay skinny
     assert route(257, 4096, 4096, 128) == 2 and route(2048, 4096, 4096, 128) == 2
     assert route(100, 14336, 2048, 128) in (1, 2)   # reductions of up to 2048 never take the shared form
     assert route(0, 4096, 4096, 128) == 0 and route(16, 4096, 4000, 128) == 0 and route(16, 4096, 4096, 96) == 0

@@ -159,3 +159,31 @@ def test_random_split_k_launches_of_more_workgroups_than_run_at_once(gpu_ops, or
         torch.cuda.synchronize()
         pu.assert_out_close(pu.out_tensor_bits(y), ref4["out_bits"], bf16, pu.reorder_bound(ref4["acc"], scales4, ref4["s_a"]),
                             tag + " W4 one pass")
+
+
+@pytest.mark.parametrize("M,N,K,g,mode,odt", [
+    (40, 6144, 16384, 64, "sym", "bfloat16"),      # 24 MiB, a long reduction: three row blocks
+    (72, 8192, 16384, 128, "asym", "float16"),     # 32 MiB: five row blocks, per-group zero-points
+    (33, 8256, 16384, 256, "ref", "float16"),      # ragged last strip set, groups of 256, one row in the third block
+])
+def test_auto_takes_the_kernel_for_33_to_128_rows_on_large_matrices(gpu_ops, oracle, M, N, K, g, mode, odt):
+    """33..48 and 65..80 token rows on matrices of 24..32 MiB and more go to SLIMK_KERNEL_MID on the library's own
+    choice: every output of every row against the oracle (int32 sums by its exact float product), the int32 sums
+    over K bit for bit, verification and production bits equal."""
+    from slimkernels_amd import _lib
+    assert _lib.lib().slimk_w2a8_gemm_auto_route(M, N, K, g) == 4
+    bf16 = odt == "bfloat16"
+    case = pu.small_case(M, N, K, g, mode, seed=M + N + K, out_dtype=odt)
+    print(case.name, flush=True)
+    packed, scales, zero = workloads.make_quantized_weight(case)
+    x = workloads.make_activation(case)
+    ref = _blas_reference(oracle, x, packed, scales, zero, g, bf16)
+    w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, x)
+    qa = gpu_ops.quantize_act_int8(xd, g)
+    out, acc = gpu_ops.w2a8_gemm(qa, w, pu.torch_dtype(case), kernel="auto", dump="sum")
+    out2 = gpu_ops.w2a8_gemm(qa, w, pu.torch_dtype(case), kernel="auto")
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(qa.q.cpu().numpy(), ref["q"])
+    np.testing.assert_array_equal(acc.cpu().numpy(), ref["acc"].sum(axis=2).astype(np.int64))
+    np.testing.assert_array_equal(pu.out_tensor_bits(out), pu.out_tensor_bits(out2))
+    pu.assert_out_close(pu.out_tensor_bits(out), ref["out_bits"], bf16, pu.reorder_bound(ref["acc"], scales, ref["s_a"]), case.name)
