@@ -149,14 +149,17 @@ enum MidRoute { kMidPlain, kMidShared, kMidTiled, kMidStrips };
 // Where the tiled kernel would leave most of a 64-row tile empty - 33..48 and 65..80 rows - on a matrix of 32 MiB and
 // more, the kernel with every row in one workgroup (SLIMK_KERNEL_MID) is ahead of it: 28672 x 8192 (groups of 64)
 // 36.7 -> 32.3 us at 33 rows and 57.6 -> 46.4 at 80, 8192 x 28672 41.1 -> 36.2 and 56.1 -> 51.1, 12288 x 12288 (groups
-// of 128) 28.2 -> 25.5 and 37.1 -> 34.3, 16384 x 16384 34.3 -> 31.5 and 51.4 -> 42.4.  At 49..64 and from 81 rows on
-// the tiled kernel keeps the lead (full tiles), and on smaller matrices the skinny forms do.
-bool mid_strips_rows(int M) { return (M >= 33 && M <= 48) || (M >= 65 && M <= 80); }
+// of 128) 28.2 -> 25.5 and 37.1 -> 34.3, 16384 x 16384 34.3 -> 31.5 and 51.4 -> 42.4; likewise 129..160 rows (two row
+// parts of five blocks against three tiles: 28672 x 8192, groups of 128, 64.0 -> 58.1 us at 130 rows, 16384 x 16384
+// 68.4 -> 60.2).  At 49..64, 81..128 and from 161 rows on the tiled kernel keeps the lead (fuller tiles), and on smaller
+// matrices the skinny forms do.
+bool mid_strips_rows(int M) { return (M >= 33 && M <= 48) || (M >= 65 && M <= 80) || (M >= 129 && M <= 160); }
 MidRoute mid_route_of_three(int M, int N, int K, int group_size);
 MidRoute mid_route(int M, int N, int K, int group_size) {
     const MidRoute r = mid_route_of_three(M, N, K, group_size);
     const size_t weight_bytes = (size_t)strips_of(N) * 64 * (K / 4);
     if (!mid_strips_rows(M) || group_size > 256) return r;
+    if ((size_t)strips_of(N) * ((M + 15) / 16) > (size_t)kMaxCounters) return r;   // (a split launch needs a counter per tile)
     if (r == kMidTiled && weight_bytes >= ((size_t)32 << 20)) return kMidStrips;
     // (long reductions a little below that size, whichever of the three the prediction names: 7168 x 16384, groups of 64,
     // 32.5 us through the shared-activation workgroups, 29.2 tiled, 26.2 here at 33 rows; 37.5 / 39.1 / 35.9 at 65)
@@ -197,7 +200,7 @@ MidRoute mid_route_of_three(int M, int N, int K, int group_size) {
     return shared_cost <= tiled_cost ? kMidShared : kMidTiled;
 }
 
-// The kernel for 33..128 rows (a workgroup = four strips x the rows of a row part): K splits across workgroups in
+// The kernel for 33..256 rows (a workgroup = four strips x the rows of a row part): K splits across workgroups in
 // rounds of four pieces (a piece = two 64-element steps, one with groups of 64).  Two workgroups on a CU run side by
 // side in about the time of one, a third waits for a place: the split is the largest power of two (up to 8) that keeps
 // the launch within 512 workgroups and every workgroup at two rounds or more (28672 x 8192 at 33 rows, 112 strip sets:
@@ -427,7 +430,7 @@ int gemm_impl(const int8_t* q, int ldq, const float* s_a, const int32_t* rowsum,
     const bool rowsum_unused = !zp_r && zp_const == 2 && group_size <= 256 &&
                                (kern_for_rowsum == SLIMK_KERNEL_TILED || kern_for_rowsum == SLIMK_KERNEL_MID);
     if (!rowsum && !rowsum_unused)
-        return fail(SLIMK_ERR_NULL_POINTER, "gemm: rowsum is NULL (only the tiled kernel and the one for 33..128 rows, with the uniform zero-point 2 and a group size of at most 256, do without)");
+        return fail(SLIMK_ERR_NULL_POINTER, "gemm: rowsum is NULL (only the tiled kernel and SLIMK_KERNEL_MID, with the uniform zero-point 2 and a group size of at most 256, do without)");
     if (!rowsum) ldr = (M + 3) / 4 * 4;
     if (out_dtype != SLIMK_F16 && out_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "out_dtype=%d", out_dtype);
     if (kernel < SLIMK_KERNEL_AUTO || kernel > SLIMK_KERNEL_MID) return fail(SLIMK_ERR_BAD_ENUM, "kernel=%d", kernel);

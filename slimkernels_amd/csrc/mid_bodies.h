@@ -1,9 +1,9 @@
-// The W2A8 GEMM for 33..128 token rows on gfx950: between the weight-streaming kernels for a few rows (which pass over
+// The W2A8 GEMM for 33..256 token rows on gfx950: between the weight-streaming kernels for a few rows (which pass over
 // the weights once per block of 16 rows) and the tiled kernel (whose 64 x 256 tiles are too few, or need K split over
 // many workgroups, while the rows are this few).
 //
-// Workgroup = four strips of 64 channels (one per wave) x up to six blocks of 16 token rows (MB; 97..128 rows run as
-// two row parts of four blocks, blockIdx.z) x a range of K (blockIdx.y).
+// Workgroup = four strips of 64 channels (one per wave) x up to six blocks of 16 token rows (MB; more than 96 rows run
+// as two or three row parts of equal height, blockIdx.z) x a range of K (blockIdx.y).
 //  * Weights: a wave streams the 1 KiB units of its own strip straight into a register ring (buffer loads, scalar
 //    offsets), unpacks a unit ONCE - high bit of every field flipped, field moved to the top of its byte: bytes
 //    64 * (code - 2), no row-sum term for the symmetric levels - and uses the operand for all MB row blocks.

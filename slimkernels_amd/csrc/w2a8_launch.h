@@ -52,11 +52,12 @@ hipError_t launch_skinny_verify(const GemmParams& p, int gs, int waves, bool asy
 hipError_t launch_skinny_shared_verify(const GemmParams& p, int gs, int kparts, bool asym, bool out_bf16, hipStream_t stream);
 hipError_t launch_skinny_grouped_verify(const GroupedParams& gp, int gs, bool asym, bool out_bf16, hipStream_t stream);
 
-// 33..128 token rows: one workgroup per set of four strips (a wave each) and row part (up to six blocks of 16 rows;
-// 97..128 rows run as two parts of four blocks), K split over blockIdx.y in whole groups (p.groups_per_split); the
-// split workspace holds one fp32 tile of 16 x 64 per strip, row block and split and one arrival counter per strip and
-// row block, as the one-strip kernel's does.  launch_mid_verify: the instantiations with the int32 dump.
-constexpr int kMidMaxRows = 128;
+// 33..256 token rows: one workgroup per set of four strips (a wave each) and row part (three to six blocks of 16 rows;
+// more than 96 rows run as two or three parts of equal height), K split over blockIdx.y in whole groups
+// (p.groups_per_split); the split workspace holds one fp32 tile of 16 x 64 per strip, row block and split and one
+// arrival counter per strip and row block, as the one-strip kernel's does.  launch_mid_verify: the instantiations with
+// the int32 dump.
+constexpr int kMidMaxRows = 256;
 namespace mid {
 constexpr int kWaves = 4;           // strips per workgroup
 constexpr int kSlots = 4;           // pieces of activations in LDS
@@ -64,11 +65,12 @@ constexpr int kPiecesPerRound = 4;  // pieces per unrolled round of the main loo
 __host__ __device__ constexpr int piece_steps(int GS) { return GS >= 2 ? 2 : 1; }   // 64-element steps per piece
 __host__ __device__ constexpr int frags_per_wave(int MB, int GS) { return (MB * piece_steps(GS) + kWaves - 1) / kWaves; }
 }  // namespace mid
-// row blocks a launch is instantiated for (3..6) and the row parts it runs as
-inline int mid_row_parts(int M) { return (M + 15) / 16 > 6 ? 2 : 1; }
+// the row parts a launch runs as and the row blocks per part it is instantiated for (3..6)
+inline int mid_row_parts(int M) { return ((M + 15) / 16 + 5) / 6; }
 inline int mid_row_blocks(int M) {
-    const int mb = (M + 15) / 16;
-    return mb > 6 ? 4 : (mb < 3 ? 3 : mb);
+    const int blocks = (M + 15) / 16, parts = mid_row_parts(M);
+    const int mb = (blocks + parts - 1) / parts;
+    return mb < 3 ? 3 : mb;
 }
 
 hipError_t launch_mid(const GemmParams& p, int gs, bool asym, bool out_bf16, hipStream_t stream);

@@ -295,6 +295,8 @@ def test_skinny_shared_more_than_32_rows(gpu_ops, oracle, M, N, K, g, mode, out,
     (20, 192, 2048, 128, "asym", "float16", 2),      # fewer rows than the form is meant for
     (112, 700, 2048, 128, "asym", "bfloat16", 0),    # seven row blocks: row parts of four and three
     (96, 1100, 3072, 256, "sym", "float16", 4),      # six row blocks, groups of 256, ragged last strip set
+    (144, 600, 2048, 128, "sym", "float16", 2),      # nine row blocks: two row parts of five (the second holds four)
+    (200, 320, 1024, 64, "asym", "bfloat16", 0),     # thirteen row blocks: three row parts of five (the third holds three)
 ])
 def test_mid_kernel(gpu_ops, oracle, M, N, K, g, mode, out, split):
     """SLIMK_KERNEL_MID (a workgroup = four strips x up to six blocks of 16 token rows, the activations shared through

@@ -38,7 +38,7 @@ def test_random_single_gemms(gpu_ops, oracle, seed):
         kernel = rng.choice(["auto", "auto", "skinny", "tiled", "mid"])
         if kernel == "skinny" and case.M > 32:
             kernel = "auto"
-        if kernel == "mid" and case.M > 128:
+        if kernel == "mid" and case.M > 256:
             kernel = "auto"
         split = 0 if rng.random() < 0.5 else rng.randint(1, 8)
         tag = f"M={case.M} N={case.N} K={case.K} g={case.group_size} {case.mode} {case.out_dtype} {kernel} split={split}"
@@ -165,9 +165,10 @@ def test_random_split_k_launches_of_more_workgroups_than_run_at_once(gpu_ops, or
     (40, 6144, 16384, 64, "sym", "bfloat16"),      # 24 MiB, a long reduction: three row blocks
     (72, 8192, 16384, 128, "asym", "float16"),     # 32 MiB: five row blocks, per-group zero-points
     (33, 8256, 16384, 256, "ref", "float16"),      # ragged last strip set, groups of 256, one row in the third block
+    (150, 8192, 16384, 128, "sym", "bfloat16"),    # two row parts of five blocks
 ])
 def test_auto_takes_the_kernel_for_33_to_128_rows_on_large_matrices(gpu_ops, oracle, M, N, K, g, mode, odt):
-    """33..48 and 65..80 token rows on matrices of 24..32 MiB and more go to SLIMK_KERNEL_MID on the library's own
+    """33..48, 65..80 and 129..160 token rows on matrices of 24..32 MiB and more go to SLIMK_KERNEL_MID on the library's own
     choice: every output of every row against the oracle (int32 sums by its exact float product), the int32 sums
     over K bit for bit, verification and production bits equal."""
     from slimkernels_amd import _lib
