@@ -374,7 +374,7 @@ __device__ __forceinline__ void mid_body(const GemmParams& p) {
     __syncthreads();
     if (lds[kVerdict] == 0) return;
     // the partial tiles come from memory, not from this XCD's L2: a row block's loads (four channel blocks x up to four
-    // splits) are in flight together
+    // splits) are in flight together, and with up to four row blocks the next block's as well
     const auto fetch = [&](int mb, int sp0, v4u (&dst)[16]) {
 #pragma unroll
         for (int pp = 0; pp < 4; ++pp)
@@ -383,20 +383,26 @@ __device__ __forceinline__ void mid_body(const GemmParams& p) {
                 dst[pp * 4 + u] = __builtin_amdgcn_raw_buffer_load_b128(
                     ws_rsrc, lane_off + mb * kTileBytes + pp * 1024 + min(sp0 + u, p.split - 1) * split_pitch, 0, kCoherent);
     };
+    constexpr bool kTwoDeep = MB <= 4;   // (registers for two row blocks' loads in flight next to the sums)
+    v4u part[kTwoDeep ? 2 : 1][16];
+    if (kTwoDeep) fetch(0, 0, part[0]);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
+        v4u (&mine)[16] = part[kTwoDeep ? mb & 1 : 0];
+        if (kTwoDeep && mb + 1 < MB) {
+            if (mb + 1 < mblocks) fetch(mb + 1, 0, part[kTwoDeep ? (mb + 1) & 1 : 0]);   // (uniform)
+        }
         if (mb < mblocks) {   // (uniform)
-            v4u part[16];
             v4f sum[4];
 #pragma unroll
             for (int pp = 0; pp < 4; ++pp) sum[pp] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
             for (int sp0 = 0; sp0 < p.split; sp0 += 4) {
-                fetch(mb, sp0, part);
+                if (!kTwoDeep || sp0 > 0) fetch(mb, sp0, mine);
 #pragma unroll
                 for (int pp = 0; pp < 4; ++pp)
 #pragma unroll
                     for (int u = 0; u < 4; ++u)
-                        if (sp0 + u < p.split) sum[pp] += __builtin_bit_cast(v4f, part[pp * 4 + u]);
+                        if (sp0 + u < p.split) sum[pp] += __builtin_bit_cast(v4f, mine[pp * 4 + u]);
             }
 #pragma unroll
             for (int pp = 0; pp < 4; ++pp)
