@@ -297,6 +297,8 @@ def flat_fractions(detail):
             flat[f"hbm_frac_{key}"] = r["frac_hbm"]
             flat[f"mfma_frac_{key}"] = r["frac_int8_mfma"]
         flat[f"us_{key}"] = r["us"]
+        if "tiled_kernel_us" in r:
+            flat[f"us_tiled_kernel_{key}"] = r["tiled_kernel_us"]
     if "single_launch" in detail:
         flat["hbm_frac_c2_single_launch"] = detail["single_launch"]["frac_hbm"]
     if "decode_sweep_m_le_16" in detail:
@@ -475,6 +477,9 @@ def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, d
     c4_shapes = ((28672, 8192), (8192, 28672))
     plan = [("c4", N, K, 64, "sym", torch.bfloat16, M) for (N, K) in c4_shapes for M in (1, 16)]
     plan += [("c5", 5120, 13824, 128, "asym", torch.float16, 1), ("c5", 11008, 4096, 128, "asym", torch.float16, 77)]
+    # (33 and 80 rows: row counts that would leave 64-row tiles mostly empty, which the library gives to the kernel
+    # that takes every row in one workgroup on matrices this large; the tiled kernel's time is reported beside it)
+    plan += [("c4", 28672, 8192, 64, "sym", torch.bfloat16, M) for M in (33, 80)]
     plan += [("c4", N, K, 64, "sym", torch.bfloat16, M) for (N, K) in c4_shapes for M in (128, 2048)]
     cache = {}
     for (cfg, N, K, g, mode, odt, M) in plan:
@@ -493,7 +498,15 @@ def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, d
             ops.w2a8_gemm(qa, w, odt, out=out)
         us = time_graph(torch, lambda: [ops.w2a8_gemm(qa, w, odt, out=out) for w in ws], len(ws), replays=4)
         nb, nops = workloads.algorithmic_bytes(c), workloads.algorithmic_ops(c)
+        route = L.slimk_w2a8_gemm_auto_route(M, N, K, g)
+        extra = {}
+        if route == 4:
+            ops.w2a8_gemm(qa, ws[0], odt, out=out, kernel="tiled")
+            extra["tiled_kernel_us"] = round(time_graph(torch, lambda: [ops.w2a8_gemm(qa, w, odt, out=out, kernel="tiled") for w in ws],
+                                                        len(ws), replays=4), 2)
         others.append({"config": cfg, "shape": f"{N}x{K}", "M": M, "group": g, "mode": mode, "weights": "cold" if cold else "warm",
+                       "route": {1: "skinny, one strip per workgroup", 2: "tiled", 3: "skinny, shared activations",
+                                 4: "every row in one workgroup (SLIMK_KERNEL_MID)"}.get(route, str(route)), **extra,
                        "split_k": L.slimk_w2a8_gemm_auto_split_k(M, N, K, g, 0), "us": round(us, 2),
                        "GBps": round(nb / (us * 1e-6) / 1e9, 1), "frac_hbm": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
                        "TOPS": round(nops / (us * 1e-6) / 1e12, 1), "frac_int8_mfma": round(nops / (us * 1e-6) / 1e12 / INT8_PEAK_TOPS, 4)})
