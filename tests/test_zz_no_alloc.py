@@ -1,6 +1,6 @@
 """slimk_w2a8_gemm_static, the GEMM entry point that allocates nothing (its split-K counters and partial sums live
 in a device array inside the library), called through the C ABI and held bit for bit to slimk_w2a8_gemm with a
-caller-owned workspace: calls in a row on one stream, each smaller than the one before, on both kernels."""
+caller-owned workspace: calls in a row on one stream, each smaller than the one before, on every kernel that splits K."""
 import numpy as np
 import pytest
 import torch
@@ -23,6 +23,7 @@ def _call_static(L, qa, w, out, kernel, split_k):
 SEQUENCE = [
     (16, 4096, 14336, 128, "sym", _lib.KERNEL_SKINNY),
     (8, 2048, 14336, 128, "asym", _lib.KERNEL_SKINNY),
+    (80, 2048, 8192, 128, "asym", _lib.KERNEL_MID),
     (64, 4096, 4096, 128, "sym", _lib.KERNEL_TILED),
     (40, 512, 8192, 64, "sym", _lib.KERNEL_TILED),
     (1, 2048, 14336, 128, "sym", _lib.KERNEL_SKINNY),
@@ -39,7 +40,7 @@ def test_gemm_without_allocation_matches_the_workspace_entry_point(gpu_ops, orac
         x = workloads.make_activation(case)
         w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, x)
         qa = gpu_ops.quantize_act_int8(xd, g)
-        kname = "skinny" if kernel == _lib.KERNEL_SKINNY else "tiled"
+        kname = {_lib.KERNEL_SKINNY: "skinny", _lib.KERNEL_TILED: "tiled", _lib.KERNEL_MID: "mid"}[kernel]
         assert L.slimk_w2a8_gemm_auto_split_k(M, N, K, g, kernel) > 1, "the case is meant to split K"
         want = gpu_ops.w2a8_gemm(qa, w, torch.float16, kernel=kname)      # caller-owned workspace
         ref = oracle.reference_forward(x, packed, scales, zero, g, want_acc=True)
