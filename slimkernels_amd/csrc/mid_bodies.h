@@ -122,14 +122,26 @@ __device__ __forceinline__ void mid_body(const GemmParams& p) {
         int rrow[MB];
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) rrow[mb] = min(row0 + mb * 16 + col, p.M - 1);
+        // (the loads of four groups are asked for one turn ahead of their use)
+        v2u zs_n;
+        uint32_t zz_n;
+        int rs_n[MB];
+        const auto fetch_zp = [&](int gb) {
+            const int g = g_lo + min(gb + quad, g_cnt - 1);  // clamped; masked where used
+            zs_n = __builtin_amdgcn_raw_buffer_load_b64(s_rsrc, s_lane_off, g * s_group_stride, 0);
+            zz_n = p.zp_r ? zp32[((size_t)g * p.strips + strip) * 16 + col] : (uint32_t)p.zp_const * 0x01010101u;
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) rs_n[mb] = p.rowsum[(size_t)g * p.ldr + rrow[mb]];
+        };
+        fetch_zp(0);
         for (int gb = 0; gb < g_cnt; gb += 4) {
-            const int g = g_lo + min(gb + quad, g_cnt - 1);  // clamped; masked below
             const bool on = gb + quad < g_cnt;
-            const v2u zs = __builtin_amdgcn_raw_buffer_load_b64(s_rsrc, s_lane_off, g * s_group_stride, 0);
-            const uint32_t zz = p.zp_r ? zp32[((size_t)g * p.strips + strip) * 16 + col] : (uint32_t)p.zp_const * 0x01010101u;
+            const v2u zs = zs_n;
+            const uint32_t zz = zz_n;
             int rs[MB];
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) rs[mb] = p.rowsum[(size_t)g * p.ldr + rrow[mb]];
+            for (int mb = 0; mb < MB; ++mb) rs[mb] = rs_n[mb];
+            fetch_zp(min(gb + 4, g_cnt - 1));
             const v4h sh = __builtin_bit_cast(v4h, zs);
             float zb[4];
 #pragma unroll
