@@ -122,39 +122,40 @@ __device__ __forceinline__ void mid_body(const GemmParams& p) {
         int rrow[MB];
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) rrow[mb] = min(row0 + mb * 16 + col, p.M - 1);
-        // (the loads of four groups are asked for one turn ahead of their use)
-        v2u zs_n;
-        uint32_t zz_n;
-        int rs_n[MB];
-        const auto fetch_zp = [&](int gb) {
-            const int g = g_lo + min(gb + quad, g_cnt - 1);  // clamped; masked where used
-            zs_n = __builtin_amdgcn_raw_buffer_load_b64(s_rsrc, s_lane_off, g * s_group_stride, 0);
-            zz_n = p.zp_r ? zp32[((size_t)g * p.strips + strip) * 16 + col] : (uint32_t)p.zp_const * 0x01010101u;
+        // (sixteen groups' loads are asked for together: a turn of four groups is a dozen MFMAs, far less than a trip to memory)
+        constexpr int kTurns = 4;
+        for (int gb0 = 0; gb0 < g_cnt; gb0 += 4 * kTurns) {
+            v2u zs[kTurns];
+            uint32_t zz[kTurns];
+            int rs[kTurns][MB];
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) rs_n[mb] = p.rowsum[(size_t)g * p.ldr + rrow[mb]];
-        };
-        fetch_zp(0);
-        for (int gb = 0; gb < g_cnt; gb += 4) {
-            const bool on = gb + quad < g_cnt;
-            const v2u zs = zs_n;
-            const uint32_t zz = zz_n;
-            int rs[MB];
+            for (int i = 0; i < kTurns; ++i) {
+                const int g = g_lo + min(gb0 + 4 * i + quad, g_cnt - 1);  // clamped; masked below
+                zs[i] = __builtin_amdgcn_raw_buffer_load_b64(s_rsrc, s_lane_off, g * s_group_stride, 0);
+                zz[i] = p.zp_r ? zp32[((size_t)g * p.strips + strip) * 16 + col] : (uint32_t)p.zp_const * 0x01010101u;
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) rs[mb] = rs_n[mb];
-            fetch_zp(min(gb + 4, g_cnt - 1));
-            const v4h sh = __builtin_bit_cast(v4h, zs);
-            float zb[4];
+                for (int mb = 0; mb < MB; ++mb) rs[i][mb] = p.rowsum[(size_t)g * p.ldr + rrow[mb]];
+            }
 #pragma unroll
-            for (int pp = 0; pp < 4; ++pp) zb[pp] = on ? (2.0f - (float)((zz >> (8 * pp)) & 0xffu)) * (float)sh[pp] : 0.0f;
+            for (int i = 0; i < kTurns; ++i) {
+                const int gb = gb0 + 4 * i;
+                if (gb < g_cnt) {   // (uniform)
+                    const bool on = gb + quad < g_cnt;
+                    const v4h sh = __builtin_bit_cast(v4h, zs[i]);
+                    float zb[4];
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) {
-                const float rsf = (float)rs[mb];
+                    for (int pp = 0; pp < 4; ++pp) zb[pp] = on ? (2.0f - (float)((zz[i] >> (8 * pp)) & 0xffu)) * (float)sh[pp] : 0.0f;
 #pragma unroll
-                for (int pp = 0; pp < 4; ++pp) {
-                    v4f c = {t[mb][pp][0], t[mb][pp][1], t[mb][pp][2], t[mb][pp][3]};
-                    c = __builtin_amdgcn_mfma_f32_16x16x4f32(rsf, zb[pp], c, 0, 0, 0);
+                    for (int mb = 0; mb < MB; ++mb) {
+                        const float rsf = (float)rs[i][mb];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) t[mb][pp][j] = c[j];
+                        for (int pp = 0; pp < 4; ++pp) {
+                            v4f c = {t[mb][pp][0], t[mb][pp][1], t[mb][pp][2], t[mb][pp][3]};
+                            c = __builtin_amdgcn_mfma_f32_16x16x4f32(rsf, zb[pp], c, 0, 0, 0);
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) t[mb][pp][j] = c[j];
+                        }
+                    }
                 }
             }
         }
