@@ -112,9 +112,9 @@ def _blas_reference(oracle, x, packed, scales, zero, g, bf16):
 
 @pytest.mark.parametrize("seed", range(2))
 def test_random_split_k_launches_of_more_workgroups_than_run_at_once(gpu_ops, oracle, seed):
-    """Split-K of the tiled kernel (W2 and the one-pass W4 form) on launches of 600 workgroups and more, one or two
-    stages per workgroup: the last workgroups to start publish their partial sums into a memory pipeline that is
-    backed up.  Every output of every row against the oracle (not against the verification instantiation)."""
+    """Split-K of the tiled kernel (W2 and the one-pass W4 form) and of the kernel for 33..256 rows on launches of 600
+    workgroups and more, one or two stages (rounds) per workgroup: the last workgroups to start publish their partial
+    sums into a memory pipeline that is backed up.  Every output of every row against the oracle (not against the verification instantiation)."""
     from slimkernels_amd import w4
     from slimkernels_amd.torch import w4 as tw4
     rng = random.Random(3000 + seed)
@@ -145,6 +145,28 @@ def test_random_split_k_launches_of_more_workgroups_than_run_at_once(gpu_ops, or
         np.testing.assert_array_equal(pu.out_tensor_bits(out), pu.out_tensor_bits(out2))
         pu.assert_out_close(pu.out_tensor_bits(out), ref["out_bits"], bf16, pu.reorder_bound(ref["acc"], scales, ref["s_a"]), tag)
         del w, qa, out, out2
+        # a launch of the same class through the kernel for 33..256 rows (its partial tiles leave as 16-byte stores too):
+        # four strips x one row part per workgroup, one or two rounds of four pieces per split
+        msplit = rng.choice([4, 8])
+        mM = rng.choice([40, 77, 100, 150])
+        parts = ((mM + 15) // 16 + 5) // 6
+        mK = 64 * 4 * (1 if g == 64 else 2) * rng.choice([1, 2]) * msplit
+        sets = -(-(600 + rng.randrange(300)) // (parts * msplit))
+        mN = 256 * sets - rng.choice([0, 8, 64, 200])
+        mcase = pu.small_case(mM, mN, mK, g, mode, seed=rng.randrange(1 << 20), out_dtype=odt)
+        mtag = f"M={mM} N={mN} K={mK} g={g} {mode} {odt} mid split={msplit} workgroups={sets * parts * msplit}"
+        print(mtag, flush=True)
+        mpacked, mscales, mzero = workloads.make_quantized_weight(mcase)
+        mx = workloads.make_activation(mcase)
+        mref = _blas_reference(oracle, mx, mpacked, mscales, mzero, g, bf16)
+        mw, mxd = pu.device_inputs(gpu_ops, mcase, mpacked, mscales, mzero, mx)
+        mqa = gpu_ops.quantize_act_int8(mxd, g)
+        mout = gpu_ops.w2a8_gemm(mqa, mw, pu.torch_dtype(mcase), kernel="mid", split_k=msplit)
+        mout2 = gpu_ops.w2a8_gemm(mqa, mw, pu.torch_dtype(mcase), kernel="mid", split_k=msplit)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(pu.out_tensor_bits(mout), pu.out_tensor_bits(mout2))
+        pu.assert_out_close(pu.out_tensor_bits(mout), mref["out_bits"], bf16, pu.reorder_bound(mref["acc"], mscales, mref["s_a"]), mtag)
+        del mw, mqa, mout, mout2
         if g == 256:
             continue
         # the same launch shape through the one-pass 4-bit form of the body (uniform zero-point 8)
