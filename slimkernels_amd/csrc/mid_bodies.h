@@ -463,4 +463,11 @@ static hipError_t launch_mid_impl(const GemmParams& p, int gs, bool asym, bool o
     return hipGetLastError();
 }
 
+// one group size of the verification instantiations (a translation unit each: they build side by side)
+template <int GS>
+static hipError_t launch_mid_verify_one(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
+    launch_mid_gs<GS, true>(p, asym || p.zp_const != 2, out_bf16, stream);
+    return hipGetLastError();
+}
+
 }  // namespace w2a8
