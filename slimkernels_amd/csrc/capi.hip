@@ -158,7 +158,10 @@ MidRoute mid_route_of_three(int M, int N, int K, int group_size);
 MidRoute mid_route(int M, int N, int K, int group_size) {
     const MidRoute r = mid_route_of_three(M, N, K, group_size);
     const size_t weight_bytes = (size_t)strips_of(N) * 64 * (K / 4);
-    if (!mid_strips_rows(M) || group_size > 256) return r;
+    // (six row blocks against two 64-row tiles: ahead only on wide matrices, 256 strips and more - 28672 x 8192 at 96 rows,
+    // groups of 64, 58.0 -> 54.6 us, 16384 x 16384 53.1 -> 48.9, 53248 x 16384 at 88 rows 148 -> 120; 8192 x 28672 56.2 -> 59.6)
+    const bool six_blocks_wide = M >= 81 && M <= 96 && strips_of(N) >= 256;
+    if (!(mid_strips_rows(M) || six_blocks_wide) || group_size > 256) return r;
     if ((size_t)strips_of(N) * ((M + 15) / 16) > (size_t)kMaxCounters) return r;   // (a split launch needs a counter per tile)
     if (r == kMidTiled && weight_bytes >= ((size_t)32 << 20)) return kMidStrips;
     // (long reductions a little below that size, whichever of the three the prediction names: 7168 x 16384, groups of 64,

@@ -81,7 +81,8 @@ def test_auto_route(L):
     assert route(128, 28672, 8192, 64) == 2
     # rows that would leave a 64-row tile mostly empty, on matrices of 32 MiB and more: every row in one workgroup
     assert route(33, 28672, 8192, 64) == 4 and route(48, 8192, 28672, 128) == 4 and route(80, 16384, 16384, 128) == 4
-    assert route(49, 28672, 8192, 64) == 2 and route(64, 28672, 8192, 64) == 2 and route(81, 28672, 8192, 64) == 2
+    assert route(49, 28672, 8192, 64) == 2 and route(64, 28672, 8192, 64) == 2 and route(97, 28672, 8192, 64) == 2
+    assert route(88, 28672, 8192, 64) == 4 and route(88, 8192, 28672, 64) == 2      # 81..96 rows: on 256 strips and more
     assert route(144, 28672, 8192, 128) == 4 and route(161, 28672, 8192, 128) == 2
     assert route(40, 7168, 16384, 64) == 4          # a long reduction from 24 MiB on
     assert route(40, 14336, 4096, 128) in (1, 3) and route(40, 10240, 8192, 128) in (1, 3)   # smaller matrices stay skinny
