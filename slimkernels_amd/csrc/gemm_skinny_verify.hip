@@ -1,7 +1,8 @@
 // Verification instantiations of the skinny-M kernels: the production bodies (skinny_bodies.h) with the int32 dump
 // switched on.  A verification launch takes the same instantiation choices as the production launch of the same
 // problem; its outputs are bit-identical with the production launch's.  The one-problem kernel's instantiations are
-// spread over three more translation units, one per group size (gemm_skinny_verify_gs*.hip), to build in parallel.
+// spread over three more translation units, one per group size (gemm_skinny_verify_gs*.hip), and the grouped kernel's
+// sit in gemm_skinny_grouped_verify.hip, to build in parallel.
 #include "skinny_bodies.h"
 
 namespace w2a8 {
@@ -18,10 +19,6 @@ hipError_t launch_skinny_verify(const GemmParams& p, int gs, int waves, bool asy
 
 hipError_t launch_skinny_shared_verify(const GemmParams& p, int gs, int kparts, bool asym, bool out_bf16, hipStream_t stream) {
     return launch_skinny_shared_impl<true>(p, gs, kparts, asym, out_bf16, stream);
-}
-
-hipError_t launch_skinny_grouped_verify(const GroupedParams& gp, int gs, bool asym, bool out_bf16, hipStream_t stream) {
-    return launch_skinny_grouped_impl<true>(gp, gs, asym, out_bf16, stream);
 }
 
 }  // namespace w2a8
