@@ -82,10 +82,9 @@ enum slimk_kernel {
     SLIMK_KERNEL_MID = 3     /* workgroups of four 64-channel strips x up to 96 token rows (more rows: two or three row
                                 parts), activations shared through LDS, weights streamed once per row part straight to
                                 registers, K split across workgroups: M <= 256, groups of up to 256; split workspace
-                                sized as for SLIMK_KERNEL_SKINNY.  SLIMK_KERNEL_AUTO takes it for 33..48, 65..80 and
-                                129..160 rows (81..96 too from 256 strips on) on matrices of 32 MiB and more, where
-                                64-row tiles would be mostly empty (3..30 % faster than the tiled kernel there),
-                                nowhere else */
+                                sized as for SLIMK_KERNEL_SKINNY.  SLIMK_KERNEL_AUTO takes it where it is predicted the
+                                fastest of the four forms: row counts that leave 64-row tiles partly empty (33..48,
+                                65..96, 129..160) on large matrices (3..30 % faster than the tiled kernel there) */
 };
 
 /* what the optional int32 verification buffer receives */
@@ -123,8 +122,9 @@ size_t slimk_w2a8_gemm_workspace_bytes(int M, int N, int K, int group_size, int 
 /* Which kernel form SLIMK_KERNEL_AUTO takes for this problem: 1 = skinny, one 64-channel strip per workgroup;
  * 2 = tiled; 3 = skinny, workgroups of several strips that share the activations (12..16 token rows on 384 strips
  * and more, 17..32 rows on matrices of 24 MiB or more, and the problems of 33..256 rows for which it is predicted
- * the fastest of the three); 4 = SLIMK_KERNEL_MID (33..48, 65..80 and 129..160 rows, 81..96 too from 256 strips on,
- * on matrices of 32 MiB and more).
+ * the fastest of the four); 4 = SLIMK_KERNEL_MID (the problems of 33..256 rows for which it is predicted the fastest:
+ * row counts that leave 64-row tiles partly empty, on large matrices).  For 33..256 rows the prediction is a cost
+ * formula per form, fitted to timings of all four on 32 matrices; it picks within 0.5 % of the best form on average.
  * 0 for a shape the library does not take.  A query for tests and tuning; no upstream counterpart (upstream's
  * launcher has one kernel with one fixed tiling, slimkernels/cute/gemm/wgmma_sm90_W2A8.cu:448-450). */
 int slimk_w2a8_gemm_auto_route(int M, int N, int K, int group_size);

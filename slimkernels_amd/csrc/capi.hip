@@ -126,68 +126,54 @@ int skinny_plain_split(int N, int K, int group_size) {
     return (G + gps - 1) / gps;
 }
 
-// 33..256 token rows: three kernels can take the problem (and, for some row counts on large matrices, a fourth: see
-// mid_route).
+// 33..256 token rows: four kernels can take the problem.
 //   plain  - the one-strip skinny kernel, 16 rows at a time, the passes side by side as workgroups of their own (each
 //            re-reading weights and activations, all but the first out of L2): the fastest while the workgroups are
 //            few (4096 x 4096: 5.6 us at 33 rows, tiled 17.3).
 //   shared - the shared-activation workgroups (four strips x two k-parts fetch a row block's activations once): a
 //            quarter of the plain kernel's workgroups at a higher cost each (11008 x 4096 at 80 rows: 13.5 us, plain
-//            16.0, tiled 20.8; 4096 x 11008 at 33..80 rows: 15.1..15.4 us, tiled 20.1..25.7, plain 15.6..21.4).
+//            16.0, tiled 20.8; 4096 x 28672 at 33..80 rows: 24.3..33.1 us, tiled 39.5..40.7).
 //   tiled  - 64 x 256 tiles through LDS: the cheapest per row once the rows fill its tiles and the reduction is long
 //            enough to amortise its start-up.
-// The choice is the smallest of three predicted times.  Each prediction is a start-up cost, a cost of splitting K
-// across workgroups, and rounds of 256 workgroups (one per CU) times a cost per round that grows with the steps a
-// workgroup (plain, tiled) or a wave (shared) runs through; plain and shared also pay for the weights' first trip
-// from HBM.  The coefficients are a least-squares fit (on the logarithm of predicted / measured) to timings of all
-// three kernels on 23 matrices (1024..28672 channels, K = 3072..28672) at 33, 48, 64, 80, 96, 128, 160 and 256 rows,
-// weights streamed from HBM: picking by the prediction costs 1.1 % over the best kernel of each case on average
-// (worst case 33 %; the rule by size it replaces: 4.2 % on the same cases and up to 85 %).
+//   strips - SLIMK_KERNEL_MID, four strips x every row of a row part per workgroup: ahead where 64-row tiles would run
+//            mostly empty on a large matrix (28672 x 8192, groups of 64: 36.7 -> 32.3 us at 33 rows, 57.6 -> 46.4 at 80;
+//            16384 x 16384: 51.4 -> 42.4 at 80, 68.4 -> 60.2 at 130).
+// The choice is the smallest of four predicted times.  Each prediction is a start-up cost, a cost of splitting K
+// across workgroups, and rounds of workgroups (256: one per CU; the strips form runs two per CU side by side) times a
+// cost per round that grows with the steps a workgroup (plain, tiled, strips) or a wave (shared) runs through; plain and
+// shared also pay for the weights' first trip from HBM, groups of 64 cost every form more per step.  The coefficients
+// are a least-squares fit (on the logarithm of predicted / measured) to 615 timed cases: all four kernels on 32
+// matrices (1024..28672 channels, K = 3072..28672, 1..64 MiB) at 33, 48, 64, 80, 96, 128, 160 and 256 rows in groups of
+// 128, eight of them also in groups of 64 and of 256, and further row counts (40..240) on twelve, weights streamed from
+// HBM: picking by the prediction costs 0.5 % over the best kernel of each case on average (worst case 15 %; fitted
+// on two thirds of the matrices and judged on the rest: 0.4..1.0 %; a three-way prediction with size rules for the
+// strips form, which this replaces: 2.2 %, up to 47 %).
 // Reductions of up to 2048 elements keep the rule they were measured with (plain while its passes over the weights
 // stay under 100 MiB).
 enum MidRoute { kMidPlain, kMidShared, kMidTiled, kMidStrips };
-// Where the tiled kernel would leave most of a 64-row tile empty - 33..48 and 65..80 rows - on a matrix of 32 MiB and
-// more, the kernel with every row in one workgroup (SLIMK_KERNEL_MID) is ahead of it: 28672 x 8192 (groups of 64)
-// 36.7 -> 32.3 us at 33 rows and 57.6 -> 46.4 at 80, 8192 x 28672 41.1 -> 36.2 and 56.1 -> 51.1, 12288 x 12288 (groups
-// of 128) 28.2 -> 25.5 and 37.1 -> 34.3, 16384 x 16384 34.3 -> 31.5 and 51.4 -> 42.4; likewise 129..160 rows (two row
-// parts of five blocks against three tiles: 28672 x 8192, groups of 128, 64.0 -> 58.1 us at 130 rows, 16384 x 16384
-// 68.4 -> 60.2).  At 49..64, 81..128 and from 161 rows on the tiled kernel keeps the lead (fuller tiles), and on smaller
-// matrices the skinny forms do.
-bool mid_strips_rows(int M) { return (M >= 33 && M <= 48) || (M >= 65 && M <= 80) || (M >= 129 && M <= 160); }
-MidRoute mid_route_of_three(int M, int N, int K, int group_size);
+int mid_split(int M, int N, int K, int group_size);
 MidRoute mid_route(int M, int N, int K, int group_size) {
-    const MidRoute r = mid_route_of_three(M, N, K, group_size);
-    const size_t weight_bytes = (size_t)strips_of(N) * 64 * (K / 4);
-    // (six row blocks against two 64-row tiles: ahead only on wide matrices, 256 strips and more - 28672 x 8192 at 96 rows,
-    // groups of 64, 58.0 -> 54.6 us, 16384 x 16384 53.1 -> 48.9, 53248 x 16384 at 88 rows 148 -> 120; 8192 x 28672 56.2 -> 59.6)
-    const bool six_blocks_wide = M >= 81 && M <= 96 && strips_of(N) >= 256;
-    if (!(mid_strips_rows(M) || six_blocks_wide) || group_size > 256) return r;
-    if ((size_t)strips_of(N) * ((M + 15) / 16) > (size_t)kMaxCounters) return r;   // (a split launch needs a counter per tile)
-    if (r == kMidTiled && weight_bytes >= ((size_t)32 << 20)) return kMidStrips;
-    // (long reductions a little below that size, whichever of the three the prediction names: 7168 x 16384, groups of 64,
-    // 32.5 us through the shared-activation workgroups, 29.2 tiled, 26.2 here at 33 rows; 37.5 / 39.1 / 35.9 at 65)
-    if (K >= 16384 && weight_bytes >= ((size_t)24 << 20)) return kMidStrips;
-    return r;
-}
-MidRoute mid_route_of_three(int M, int N, int K, int group_size) {
     if (M > kSkinnyMaxRows) return kMidTiled;
     const int strips = strips_of(N), steps = K / w2a8::kStepK, blocks = (M + 15) / 16;
     const size_t weight_bytes = (size_t)strips * 64 * (K / 4);
     if (K <= 2048) return (size_t)blocks * weight_bytes <= ((size_t)100 << 20) ? kMidPlain : kMidTiled;
-    if (K > 4096 && weight_bytes > ((size_t)32 << 20)) return kMidTiled;  // (28672 x 8192: tiled ahead of both skinny forms at every row count)
     const float weight_mib = (float)weight_bytes / 1048576.0f;
+    // a step costs more in groups of 64 and less in groups of 256 and more than in groups of 128: factors per form
+    const auto by_group = [&](float of64, float of256) { return group_size == 64 ? of64 : (group_size >= 256 ? of256 : 1.0f); };
     const auto rounds = [](long long wgs, float smooth) {  // between whole rounds and the plain ratio
         const float whole = (float)((wgs + 255) / 256), ratio = std::max(1.0f, (float)wgs / 256.0f);
         return smooth * ratio + (1.0f - smooth) * whole;
     };
     const int plain_split = skinny_plain_split(N, K, group_size);
-    const float plain_cost = 1.786f + (plain_split > 1 ? 3.684f : 0.0f) + 0.1085f * weight_mib +
-                             rounds((long long)strips * plain_split * blocks, 0.475f) * (1.050f + 0.0369f * (float)steps / (float)plain_split);
+    const float plain_cost = 2.569f + (plain_split > 1 ? 3.476f : 0.0f) + 0.1133f * weight_mib +
+                             rounds((long long)strips * plain_split * blocks, 0.473f) *
+                                 (0.961f + 0.0356f * (float)steps / (float)plain_split) * by_group(1.086f, 0.939f);
     const int shared_split = skinny_shared_split(M, N, K, group_size);
     const int units = (strips + 3) / 4 * blocks;
-    const float shared_cost = 5.066f + (shared_split > 1 ? 2.920f : 0.0f) + 0.1165f * weight_mib +
-                              rounds((long long)units * shared_split, 0.386f) * (-1.437f + 0.2702f * (float)steps / (2.0f * (float)shared_split));
-    float tiled_cost = 1e30f;
+    const float shared_cost = 6.125f + (shared_split > 1 ? 2.584f : 0.0f) + 0.0599f * weight_mib +
+                              rounds((long long)units * shared_split, 0.318f) *
+                                  (-0.321f + 0.2239f * (float)steps / (2.0f * (float)shared_split)) * by_group(1.337f, 0.805f);
+    float tiled_cost = 1e30f, strips_cost = 1e30f;
     if (group_size <= 256) {
         const int gs = group_size / w2a8::kStepK;
         const int tiled_split = w2a8::tiled_fast_auto_split(M, strips, steps, gs);
@@ -195,13 +181,26 @@ MidRoute mid_route_of_three(int M, int N, int K, int group_size) {
         const int stages = (steps + 1) / 2;
         const int per = (stages + tiled_split - 1) / tiled_split;
         const int n = (tiles * tiled_split + 255) / 256;  // workgroups per CU: up to three run side by side
-        const float together = n == 1 ? 1.0f : (n == 2 ? 1.424f : (n == 3 ? 1.860f : 0.608f * (float)n));
-        tiled_cost = -10.21f + (tiled_split > 1 ? 6.384f : 0.0f) +
-                     ((float)per + 23.97f) * 0.6773f * together * (group_size == 64 ? 1.184f : 1.0f);
+        const float together = n == 1 ? 1.0f : (n == 2 ? 1.515f : (n == 3 ? 2.136f : 0.695f * (float)n));
+        tiled_cost = -0.846f + (tiled_split > 1 ? 7.117f : 0.0f) +
+                     ((float)per + 8.09f) * 0.7121f * together * by_group(1.245f, 0.915f);
+        // (a split launch of the strips form needs an arrival counter per strip and row block)
+        if (M <= w2a8::kMidMaxRows && (size_t)strips * blocks <= (size_t)kMaxCounters) {
+            const int split = mid_split(M, N, K, group_size);
+            const int mb = w2a8::mid_row_blocks(M), piece_steps = w2a8::mid::piece_steps(gs);
+            const long long wgs = (long long)((strips + w2a8::mid::kWaves - 1) / w2a8::mid::kWaves) * w2a8::mid_row_parts(M) * split;
+            const float turns = (float)(((wgs + 255) / 256 + 1) / 2);   // two workgroups of a CU run side by side ...
+            const float pair = wgs > 256 ? 1.730f : 1.0f;                // ... each slower than one alone
+            const float pieces = (float)((steps / piece_steps + split - 1) / split);
+            const float piece = (0.3812f + 0.0786f * (float)mb) * by_group(0.675f, 1.014f);   // (a piece of groups of 64 is one step)
+            strips_cost = 5.845f + (split > 1 ? 3.211f * (float)mb - 3.363f : 0.0f) + turns * pair * pieces * piece;
+        }
     }
-    if (plain_cost <= shared_cost && plain_cost <= tiled_cost) return kMidPlain;
-    return shared_cost <= tiled_cost ? kMidShared : kMidTiled;
+    const float skinny_cost = std::min(plain_cost, shared_cost), other_cost = std::min(tiled_cost, strips_cost);
+    if (skinny_cost <= other_cost) return plain_cost <= shared_cost ? kMidPlain : kMidShared;
+    return tiled_cost <= strips_cost ? kMidTiled : kMidStrips;
 }
+
 
 // The kernel for 33..256 rows (a workgroup = four strips x the rows of a row part): K splits across workgroups in
 // rounds of four pieces (a piece = two 64-element steps, one with groups of 64).  Two workgroups on a CU run side by

@@ -1172,35 +1172,40 @@ __global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_grouped_kernel(c
     }
 }
 
-// One problem through the shared-activation body: grid.x = sets of strips (in whole sets of eight per
-// row block, as in the grouped kernel), grid.y = K splits.  For 17..32 token rows on matrices big
+// One problem through the shared-activation body.  For 17..32 token rows on matrices big
 // enough to be bound by bandwidth (measured 8..27 % faster than one strip per workgroup there), for the problems of
 // 33..256 rows the host predicts it fastest for, and with four k-parts x two strips for 12..16 rows on very wide
 // matrices (more strips than the CUs take as one-strip workgroups at a time).
+// The grid is one-dimensional and placed by xcd_place: a set is a (unit, K split) pair, its members are its row
+// blocks.  (Dealing whole units out instead, K splits in blockIdx.y, left 5120 channels = 20 units at 96 rows in two
+// splits with 36 workgroups on four XCDs of 32 CUs and 24 on the others: 30.6 us, now 22.3 us.)
 template <int GS, int NK, bool ASYM, typename OutT, bool DUMP = false>
 __global__ __launch_bounds__(kGroupedWaves * 64, 4) void skinny_shared_kernel(const GemmParams p) {
     __shared__ __attribute__((aligned(16))) GroupedSmem sm;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int local = blockIdx.x;
     const int mblocks = (p.M + 15) >> 4;
-    const int mblk = (local >> 3) % mblocks;
-    const int unit = (local / (8 * mblocks)) * 8 + (local & 7);
-    if (unit * (kGroupedWaves / NK) >= p.strips) return;  // padding workgroup (uniform)
+    constexpr int kPerUnit = kGroupedWaves / NK;
+    const int units = (p.strips + kPerUnit - 1) / kPerUnit;
+    struct { int unit, mblk, split; } at;
+    int pair;
+    if (!xcd_place(blockIdx.x, units * (p.split > 1 ? p.split : 1), mblocks, pair, at.mblk)) return;  // (uniform)
+    at.unit = pair % units;
+    at.split = pair / units;
     if (mblocks == 1) {  // one row block: every weight byte is used once (loads marked stream-once)
-        if (p.split > 1) shared_body<4, GS, NK, true, ASYM, true, true, OutT, DUMP>(p, unit, mblk, wave, sm, blockIdx.y);
-        else shared_body<4, GS, NK, true, ASYM, true, false, OutT, DUMP>(p, unit, mblk, wave, sm);
+        if (p.split > 1) shared_body<4, GS, NK, true, ASYM, true, true, OutT, DUMP>(p, at.unit, at.mblk, wave, sm, at.split);
+        else shared_body<4, GS, NK, true, ASYM, true, false, OutT, DUMP>(p, at.unit, at.mblk, wave, sm);
         return;
     }
     // several row blocks: all but the first read of the weights come from L2
-    if (p.split > 1) shared_body<4, GS, NK, true, ASYM, false, true, OutT, DUMP>(p, unit, mblk, wave, sm, blockIdx.y);
-    else shared_body<4, GS, NK, true, ASYM, false, false, OutT, DUMP>(p, unit, mblk, wave, sm);
+    if (p.split > 1) shared_body<4, GS, NK, true, ASYM, false, true, OutT, DUMP>(p, at.unit, at.mblk, wave, sm, at.split);
+    else shared_body<4, GS, NK, true, ASYM, false, false, OutT, DUMP>(p, at.unit, at.mblk, wave, sm);
 }
 
 template <int GS, int NK, bool DUMP>
 static void launch_shared_nk(const GemmParams& p, bool asym, bool out_bf16, hipStream_t stream) {
     const int per_unit = kGroupedWaves / NK;
     const int units = (p.strips + per_unit - 1) / per_unit;
-    const dim3 grid((units + 7) / 8 * 8 * ((p.M + 15) / 16), p.split > 1 ? p.split : 1), block(kGroupedWaves * 64);
+    const dim3 grid(xcd_grid(units * (p.split > 1 ? p.split : 1), (p.M + 15) / 16)), block(kGroupedWaves * 64);
     if (asym) {
         if (out_bf16) skinny_shared_kernel<GS, NK, true, OutBF16, DUMP><<<grid, block, 0, stream>>>(p);
         else skinny_shared_kernel<GS, NK, true, OutF16, DUMP><<<grid, block, 0, stream>>>(p);

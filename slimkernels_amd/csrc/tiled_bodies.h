@@ -81,7 +81,10 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
     // L2.  When the channel tiles divide by eight, every XCD owns one band of channel tiles for all
     // token tiles: its share of the weights then stays in its L2 for the whole kernel and only the
     // activations stream through (token tile major, so concurrent tiles share activation rows).
-    // Otherwise every XCD gets one contiguous run of tiles, channel tile fastest.
+    // Otherwise, with two to four token tiles, the token tiles of a channel tile stay on one XCD and the channel tiles
+    // are dealt out evenly (xcd_place: 11008 x 14336 at 80..128 rows 44.8..48.8 -> 40.8..43.1 us); with one token tile or
+    // more than four, every XCD gets one contiguous run of tiles, channel tile fastest (one token tile dealt out by
+    // xcd_place, neighbouring channel tiles on different XCDs, measured 17 % slower on that matrix: 29.9 -> 34.9 us).
     const int tiles_n = (p.strips + kStrips - 1) / kStrips;
     const int tiles_m = (p.M + kBM - 1) / kBM;
     const int total = tiles_m * tiles_n;
@@ -91,6 +94,10 @@ __device__ __forceinline__ void tiled_body(const GemmParams& p) {
     if (tiles_n % 8 == 0) {
         const int band = tiles_n / 8;
         tile = (local / band) * tiles_n + xcd * band + local % band;
+    } else if (tiles_m >= 2 && tiles_m <= 4) {
+        int n_tile, m_tile_i;
+        if (!xcd_place((int)blockIdx.x, tiles_n, tiles_m, n_tile, m_tile_i)) return;
+        tile = m_tile_i * tiles_n + n_tile;
     } else {
         tile = xcd * per_xcd + local;
     }

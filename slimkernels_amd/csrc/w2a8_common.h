@@ -155,4 +155,26 @@ struct OutBF16 {
     }
 };
 
+// Placement of a one-dimensional grid on the eight XCDs.  Workgroups go to the XCDs in turn, so blockIdx.x & 7 names
+// the XCD and blockIdx.x >> 3 the workgroup's place in that XCD's queue.  The work is `sets` sets of `members`
+// workgroups each, the members of a set reading the same weights: they take consecutive places in one XCD's queue
+// (all but the first read come from its L2), and the sets are dealt out to the XCDs evenly; what is left when their
+// number is no multiple of eight goes round the XCDs member by member, so no XCD gets more than one workgroup more than
+// another.  The grid is xcd_grid(sets, members) workgroups; false: a padding workgroup.
+__device__ __forceinline__ bool xcd_place(const int local, const int sets, const int members, int& set, int& member) {
+    const int even = sets >> 3, rest = sets & 7;
+    const int xcd = local & 7, slot = local >> 3;
+    if (slot < even * members) {
+        set = (slot / members) * 8 + xcd;
+        member = slot % members;
+        return true;
+    }
+    const int t = (slot - even * members) * 8 + xcd;
+    if (t >= rest * members) return false;
+    set = even * 8 + t % rest;
+    member = t / rest;
+    return true;
+}
+inline int xcd_grid(const int sets, const int members) { return (sets * members + 7) / 8 * 8; }
+
 }  // namespace w2a8

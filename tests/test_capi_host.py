@@ -79,12 +79,12 @@ def test_auto_route(L):
     assert route(77, 11008, 4096, 128) == 3         # five row blocks on 172 strips: the shared-activation workgroups
     assert route(64, 4096, 14336, 128) == 3         # long reduction, few 256-channel tiles
     assert route(128, 28672, 8192, 64) == 2
-    # rows that would leave a 64-row tile mostly empty, on matrices of 32 MiB and more: every row in one workgroup
+    # 33..256 rows: the smallest of four predicted times.  Rows that leave 64-row tiles partly empty on a large matrix:
+    # every row of a row part in one workgroup; tiles that fill: the tiled kernel
     assert route(33, 28672, 8192, 64) == 4 and route(48, 8192, 28672, 128) == 4 and route(80, 16384, 16384, 128) == 4
     assert route(49, 28672, 8192, 64) == 2 and route(64, 28672, 8192, 64) == 2 and route(97, 28672, 8192, 64) == 2
-    assert route(88, 28672, 8192, 64) == 4 and route(88, 8192, 28672, 64) == 2      # 81..96 rows: on 256 strips and more
-    assert route(144, 28672, 8192, 128) == 4 and route(161, 28672, 8192, 128) == 2
-    assert route(40, 7168, 16384, 64) == 4          # a long reduction from 24 MiB on
+    assert route(88, 28672, 8192, 64) == 4 and route(144, 28672, 8192, 128) == 4 and route(161, 28672, 8192, 128) == 2
+    assert route(40, 7168, 16384, 64) == 3 and route(72, 20480, 8192, 64) == 3       # a set of strips per CU or fewer, long reduction
     assert route(40, 14336, 4096, 128) in (1, 3) and route(40, 10240, 8192, 128) in (1, 3)   # smaller matrices stay skinny
     assert route(257, 4096, 4096, 128) == 2 and route(2048, 4096, 4096, 128) == 2
     assert route(100, 14336, 2048, 128) in (1, 2)   # reductions of up to 2048 never take the shared form

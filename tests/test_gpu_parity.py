@@ -266,11 +266,11 @@ def test_skinny_shared_12_to_16_rows_on_wide_matrices(gpu_ops, oracle, M, N, K, 
 
 
 @pytest.mark.parametrize("M,N,K,g,mode,out,split", [
-    (100, 6200, 2304, 64, "asym", "bfloat16", 0),   # short reduction: seven row blocks, the last ragged, ragged last strip
+    (100, 7400, 2304, 64, "asym", "bfloat16", 0),   # short reduction: seven row blocks, the last ragged, ragged last strip
     (130, 1000, 12288, 128, "sym", "float16", 0),   # long reduction, few strips: nine row blocks, K split across workgroups
     (33, 4000, 12288, 256, "ref", "float16", 0),    # the third row block holds one row
     (50, 4000, 12288, 128, "sym", "float16", 2),    # explicit split
-    (250, 3000, 2304, 128, "asym", "float16", 0),   # sixteen row blocks
+    (250, 4000, 2304, 128, "asym", "float16", 0),   # sixteen row blocks
 ])
 def test_skinny_shared_more_than_32_rows(gpu_ops, oracle, M, N, K, g, mode, out, split):
     """33..256 token rows where the library sends them through the shared-activation workgroups (one workgroup per
