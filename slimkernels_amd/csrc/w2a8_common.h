@@ -161,7 +161,7 @@ struct OutBF16 {
 // (all but the first read come from its L2), and the sets are dealt out to the XCDs evenly; what is left when their
 // number is no multiple of eight goes round the XCDs member by member, so no XCD gets more than one workgroup more than
 // another.  The grid is xcd_grid(sets, members) workgroups; false: a padding workgroup.
-__device__ __forceinline__ bool xcd_place(const int local, const int sets, const int members, int& set, int& member) {
+__host__ __device__ __forceinline__ bool xcd_place(const int local, const int sets, const int members, int& set, int& member) {
     const int even = sets >> 3, rest = sets & 7;
     const int xcd = local & 7, slot = local >> 3;
     if (slot < even * members) {
