@@ -152,11 +152,12 @@ int skinny_plain_split(int N, int K, int group_size) {
 // stay under 100 MiB).
 enum MidRoute { kMidPlain, kMidShared, kMidTiled, kMidStrips };
 int mid_split(int M, int N, int K, int group_size);
-MidRoute mid_route(int M, int N, int K, int group_size) {
-    if (M > kSkinnyMaxRows) return kMidTiled;
+// skinny_only: the faster of the two skinny forms (what an explicit request for the skinny kernel runs)
+MidRoute mid_route(int M, int N, int K, int group_size, bool skinny_only = false) {
+    if (M > kSkinnyMaxRows) return skinny_only ? kMidPlain : kMidTiled;
     const int strips = strips_of(N), steps = K / w2a8::kStepK, blocks = (M + 15) / 16;
     const size_t weight_bytes = (size_t)strips * 64 * (K / 4);
-    if (K <= 2048) return (size_t)blocks * weight_bytes <= ((size_t)100 << 20) ? kMidPlain : kMidTiled;
+    if (K <= 2048) return skinny_only || (size_t)blocks * weight_bytes <= ((size_t)100 << 20) ? kMidPlain : kMidTiled;
     const float weight_mib = (float)weight_bytes / 1048576.0f;
     // a step costs more in groups of 64 and less in groups of 256 and more than in groups of 128: factors per form
     const auto by_group = [&](float of64, float of256) { return group_size == 64 ? of64 : (group_size >= 256 ? of256 : 1.0f); };
@@ -173,6 +174,7 @@ MidRoute mid_route(int M, int N, int K, int group_size) {
     const float shared_cost = 6.125f + (shared_split > 1 ? 2.584f : 0.0f) + 0.0599f * weight_mib +
                               rounds((long long)units * shared_split, 0.318f) *
                                   (-0.321f + 0.2239f * (float)steps / (2.0f * (float)shared_split)) * by_group(1.337f, 0.805f);
+    if (skinny_only) return plain_cost <= shared_cost ? kMidPlain : kMidShared;
     float tiled_cost = 1e30f, strips_cost = 1e30f;
     if (group_size <= 256) {
         const int gs = group_size / w2a8::kStepK;
@@ -235,13 +237,13 @@ int resolve_kernel(int M, int N, int K, int group_size, int kernel) {
 
 // One problem with 17..32 token rows on a matrix big enough to be bound by bandwidth goes through the shared-activation
 // workgroups: 8..27 % faster there than one strip per workgroup (at 16 rows and below the one-strip kernel is as fast
-// or faster); with more rows, where mid_route says so (an explicit request for the skinny kernel on a shape
-// that mid_route gives to the tiled one runs one strip per workgroup, whichever skinny form would be the faster there).
+// or faster); with more rows, where it is predicted the faster of the two skinny forms (which is also what an explicit
+// request for the skinny kernel runs on a shape that SLIMK_KERNEL_AUTO gives to another kernel).
 bool skinny_shared_applies(int M, int N, int K, int group_size) {
     if (M >= kWideSharedRows && M <= 16) return strips_of(N) >= kWideSharedStrips;
     if (M <= 16 || M > kSkinnyMaxRows) return false;
     if (M <= 32) return (size_t)strips_of(N) * 64 * (K / 4) >= kSharedMinWeightBytes;
-    return mid_route(M, N, K, group_size) == kMidShared;
+    return mid_route(M, N, K, group_size, true) == kMidShared;
 }
 
 int auto_split(int M, int N, int K, int group_size, int kernel) {

@@ -87,6 +87,9 @@ def test_auto_route(L):
     assert route(40, 7168, 16384, 64) == 3 and route(72, 20480, 8192, 64) == 3       # a set of strips per CU or fewer, long reduction
     assert route(40, 14336, 4096, 128) in (1, 3) and route(40, 10240, 8192, 128) in (1, 3)   # smaller matrices stay skinny
     assert route(257, 4096, 4096, 128) == 2 and route(2048, 4096, 4096, 128) == 2
+    # an explicit request for the skinny kernel on a shape AUTO gives to the tiled one takes the faster skinny form:
+    # here the shared-activation workgroups (unsplit; the one-strip form would split K three ways)
+    assert route(256, 5120, 13824, 128) == 2 and L.slimk_w2a8_gemm_auto_split_k(256, 5120, 13824, 128, _lib.KERNEL_SKINNY) == 1
     assert route(100, 14336, 2048, 128) in (1, 2)   # reductions of up to 2048 never take the shared form
     assert route(0, 4096, 4096, 128) == 0 and route(16, 4096, 4000, 128) == 0 and route(16, 4096, 4096, 96) == 0
 
