@@ -94,6 +94,44 @@ def test_auto_route(L):
     assert route(0, 4096, 4096, 128) == 0 and route(16, 4096, 4000, 128) == 0 and route(16, 4096, 4096, 96) == 0
 
 
+def test_auto_route_only_names_kernels_that_take_the_shape(L):
+    """Whatever kernel the fitted choice names for a random shape of 1..300 rows, that kernel accepts the shape: an
+    explicit request for it with two K splits and a workspace of 16 bytes passes validation: it stops at the workspace
+    check (error 5) or, where two splits come to one, at the launch (error 6 on a machine without a GPU, which is why
+    the test only runs there: the pointers are fake).  The workspace size the library quotes for its own choice agrees
+    with its split."""
+    import random
+    import torch
+    if torch.cuda.device_count() > 0:
+        pytest.skip("fake pointers: only where a launch cannot happen")
+    rng = random.Random(20)
+    explicit = {1: _lib.KERNEL_SKINNY, 3: _lib.KERNEL_SKINNY, 2: _lib.KERNEL_TILED, 4: _lib.KERNEL_MID}
+    seen = set()
+    for _ in range(3000):
+        g = rng.choice([64, 128, 256])
+        K = g * rng.randint(4, 28672 // g)
+        N = rng.choice([rng.randint(1, 4096), rng.randint(4096, 65536)])
+        M = rng.choice([rng.randint(1, 300), rng.choice([16, 17, 32, 33, 96, 97, 256, 257])])
+        if M * K > (1 << 31) - 1 or N * (K // 4) > (1 << 31) - 1:
+            continue
+        r = L.slimk_w2a8_gemm_auto_route(M, N, K, g)
+        assert r in (1, 2, 3, 4), (M, N, K, g, r)
+        if M <= 32:
+            assert r in (1, 3)
+        if M > 256:
+            assert r == 2
+        seen.add(r)
+        ldq = (K + 15) // 16 * 16
+        rc = _gemm(L, M=M, N=N, K=K, g=g, ldq=ldq, ldo=N, ldr=(M + 3) // 4 * 4, kernel=explicit[r], split=2, ws=FAKE, wsb=16)
+        assert rc in (5, 6), (M, N, K, g, r, rc, L.slimk_w2a8_last_error())
+        if rc == 6:   # the launch itself, not a launcher that refuses the shape
+            assert b"no ROCm-capable device" in L.slimk_w2a8_last_error(), (M, N, K, g, r, L.slimk_w2a8_last_error())
+        split = L.slimk_w2a8_gemm_auto_split_k(M, N, K, g, _lib.KERNEL_AUTO)
+        assert split >= 1
+        assert (L.slimk_w2a8_gemm_workspace_bytes(M, N, K, g, _lib.KERNEL_AUTO, 0) > 0) == (split > 1), (M, N, K, g, r, split)
+    assert seen == {1, 2, 3, 4}
+
+
 def _gemm(L, **kw):
     a = dict(q=FAKE, ldq=4096, s_a=FAKE, rowsum=FAKE, ldr=16, w_r=FAKE, s_r=FAKE, zp_r=None, zp_const=2,
              M=16, N=4096, K=4096, g=128, out=FAKE, ldo=4096, odt=0, acc=None, dump=0, ws=None, wsb=0,
