@@ -579,9 +579,13 @@ def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, d
             for w in ws16:
                 ops.w2a16_gemm(x, w, torch.float16, out=out)
             us = time_graph(torch, lambda: [ops.w2a16_gemm(x, w, torch.float16, out=out) for w in ws16], len(ws16), replays=4)
+            xb = x.to(torch.bfloat16)   # the same rows as bf16 activations (the bf16 matrix cores, a fifth MFMA per 32 k)
+            for w in ws16:
+                ops.w2a16_gemm(xb, w, torch.float16, out=out)
+            us_b = time_graph(torch, lambda: [ops.w2a16_gemm(xb, w, torch.float16, out=out) for w in ws16], len(ws16), replays=4)
             nb = N * K // 4 + 2 * N * (K // g) + 2 * M * K + 2 * M * N
             a16rows.append({"shape": f"{N}x{K}", "M": M, "group": g, "weights": "cold",
-                            "split_k": L.slimk_w2a16_gemm_auto_split_k(M, N, K, g), "us": round(us, 2),
+                            "split_k": L.slimk_w2a16_gemm_auto_split_k(M, N, K, g), "us": round(us, 2), "us_bf16_activations": round(us_b, 2),
                             "GBps": round(nb / (us * 1e-6) / 1e9, 1), "frac_hbm": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)})
         del ws16
     detail["w2a16"] = a16rows

@@ -360,12 +360,14 @@ int slimk_w4a8_gemm(const int8_t* q, int ldq, const float* s_a, const int32_t* r
                     void* out, int ldo, int out_dtype,
                     void* workspace, size_t workspace_bytes, int split_k, void* stream);
 
-/* Weight-only form: x [M][ldx] fp16 activations are NOT quantised; the 2-bit codes are widened to fp16 in
- * front of the fp16 matrix cores and every scale group's fp32 sum is scaled into the fp32 result:
+/* Weight-only form: x [M][ldx] fp16 or bf16 activations are NOT quantised; the 2-bit codes are widened to the
+ * activations' type in front of the fp16 resp. bf16 matrix cores and every scale group's fp32 sum is scaled into the
+ * fp32 result:
  *   out[m][n] = cast( sum_g scales[g][n] * sum_{k in g} x[m][k] * (code[n][k] - zp[g][n]) ).
  * Same repacked weight operands as slimk_w2a8_gemm (w_r, s_r, zp_r / zp_const).  Built for few token rows
  * (the weight stream bounds the time); any M works, 16 rows at a time, each re-reading the weights.
- * K % 128 == 0; x_dtype must be SLIMK_F16 (bf16 activations: SLIMK_ERR_UNSUPPORTED); x 16-byte aligned,
+ * K % 128 == 0; x_dtype SLIMK_F16 or SLIMK_BF16 (bf16: the codes enter the matrix core as 1 + code / 4 and the
+ * group's activation sum, a fifth MFMA, takes the offset and the zero-point off in fp32); x 16-byte aligned,
  * ldx % 8 == 0.  split_k: K splits across workgroups, 0 = choose; with more than one the caller supplies
  * slimk_w2a16_gemm_workspace_bytes(...) bytes of workspace (fp32 partial sums, summed in split order by a
  * second kernel: results do not depend on timing).  The workspace needs no initialisation.

@@ -331,13 +331,17 @@ def w4_reference_forward(x_half: np.ndarray, codes_nk: np.ndarray, scale_half: n
 
 
 def w2a16_reference_forward(x_half: np.ndarray, codes_nk: np.ndarray, scale_half: np.ndarray, zp: np.ndarray,
-                            group_size: int):
+                            group_size: int, x_bf16: bool = False):
     """The weight-only form in float64: out[m, n] = sum_g scale[g, n] * sum_{k in g} x[m, k] * (code[n, k] - zp[g, n])
     with the fp16 activations as they are (the notebook kernel w2matmul, gemm_splitk.ipynb cell 1, widens the
     2-bit fields to fp16 in front of an fp32-accumulating dot; it has no scales and no zero-point, which are
     this path's own).  Returns (out float64 [M, N], mag float64 [M, N]) where mag = sum_g |scale| * sum_k |x| * |code - zp|
-    bounds the terms, for a tolerance on an fp32 accumulation in any order."""
-    x = np.asarray(x_half, np.float16).astype(np.float64)
+    bounds the terms, for a tolerance on an fp32 accumulation in any order.  With x_bf16 the activations are uint16
+    bf16 bit patterns instead of a float16 array."""
+    if x_bf16:
+        x = (np.asarray(x_half, np.uint16).astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    else:
+        x = np.asarray(x_half, np.float16).astype(np.float64)
     codes = np.asarray(codes_nk, np.uint8)
     N, K = codes.shape
     M = x.shape[0]

@@ -919,7 +919,6 @@ int slimk_w2a16_gemm(const void* x, int ldx, int x_dtype,
     if (int rc = check_kg(K, group_size)) return rc;
     if (K % 128 != 0) return fail(SLIMK_ERR_UNSUPPORTED, "w2a16_gemm: K=%d must be a multiple of 128", K);
     if (x_dtype != SLIMK_F16 && x_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "x_dtype=%d", x_dtype);
-    if (x_dtype != SLIMK_F16) return fail(SLIMK_ERR_UNSUPPORTED, "w2a16_gemm: activations must be fp16");
     if (out_dtype != SLIMK_F16 && out_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "out_dtype=%d", out_dtype);
     if (zp_const < 0 || zp_const > 3) return fail(SLIMK_ERR_BAD_SHAPE, "zp_const=%d must be 0..3", zp_const);
     if (ldx < K || ldo < N) return fail(SLIMK_ERR_BAD_SHAPE, "ldx=%d / ldo=%d too small for K=%d / N=%d", ldx, ldo, K, N);
@@ -937,7 +936,7 @@ int slimk_w2a16_gemm(const void* x, int ldx, int x_dtype,
     p.x = reinterpret_cast<const uint16_t*>(x); p.ldx = ldx;
     p.w_r = w_r; p.s_r = s_r; p.zp_r = zp_r; p.out = out; p.ldo = ldo;
     p.M = M; p.N = N; p.K = K; p.G = K / group_size; p.steps = steps; p.strips = strips_of(N);
-    p.zp_const = zp_const; p.split = split_k;
+    p.zp_const = zp_const; p.split = split_k; p.x_bf16 = x_dtype == SLIMK_BF16;
     if (split_k > 1) {
         const size_t need = (size_t)split_k * (size_t)M * (size_t)N * sizeof(float);
         if (!workspace) return fail(SLIMK_ERR_WORKSPACE, "split_k=%d needs a workspace of %zu bytes", split_k, need);

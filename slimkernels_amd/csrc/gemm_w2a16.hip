@@ -20,6 +20,14 @@
 // kernel: deterministic).  Activations are read straight from global memory (they stay in L2; rows past M
 // are out of range of the buffer descriptor and read as zero without a memory access).  Every wave keeps
 // three chunks of 128 reduction elements of weights in flight while it works on a fourth.
+//
+// bf16 activations (XBF) go to v_mfma_f32_16x16x32_bf16.  The vector ALU has no bf16 arithmetic, so the codes are not
+// centred in front of the matrix core: a field shifted to mantissa bits 6:5 and OR-ed onto 0x3f80 is the bf16 number
+// 1 + code / 4 (one shift and one v_and_or_b32 per register), a fifth MFMA per 32 reduction elements against ones sums
+// the activations of the group, and at the group's end
+//   sum_k x * (code - zp) = 4 * sum_k x * (1 + code / 4) - (4 + zp) * sum_k x
+// is put together in fp32 (every product is exact; the two sums are a few times larger than their difference, which
+// costs an fp32 accumulation a few of its 24 bits).
 #include "w2a8_launch.h"
 
 namespace w2a8 {
@@ -35,8 +43,13 @@ constexpr int kChunkSteps = 2;   // steps (of 64) per loop iteration
 
 // GS = steps per scale group (1, 2 or 4); kWaves = K-parts per workgroup (4, 8 or 16); ZP = per-group
 // zero-points; PARTIAL = write fp32 partial sums instead of the output
-template <int GS, int kWaves, bool ZP, bool PARTIAL, typename OutT>
-__global__ __launch_bounds__(kWaves * 64) void w2a16_kernel(const W2A16Params p) {
+typedef __bf16 v8b __attribute__((ext_vector_type(8)));
+
+// (The bf16 form is held to 128 registers, two eight-wave workgroups per CU: left alone it takes 162 and one
+// workgroup, 35.7 instead of 22.0 us at 28672 x 8192, one row; groups of 256 would spill 252 bytes at that limit and
+// keep the compiler's own choice, as every fp16 instantiation does.)
+template <int GS, int kWaves, bool ZP, bool PARTIAL, typename OutT, bool XBF = false>
+__global__ __launch_bounds__(kWaves * 64, XBF && GS < 4 ? 4 : 1) void w2a16_kernel(const W2A16Params p) {
     __shared__ float red[kWaves][16][64];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -98,6 +111,7 @@ __global__ __launch_bounds__(kWaves * 64) void w2a16_kernel(const W2A16Params p)
 
     float t[4][4];
     v4f acc[4];
+    v4f acc_x = {0.f, 0.f, 0.f, 0.f};   // XBF: the group's activation sums per token row
 #pragma unroll
     for (int pp = 0; pp < 4; ++pp) {
         acc[pp] = v4f{0.f, 0.f, 0.f, 0.f};
@@ -124,6 +138,21 @@ __global__ __launch_bounds__(kWaves * 64) void w2a16_kernel(const W2A16Params p)
                 const v4u ap = {__builtin_amdgcn_perm(d[1], d[0], 0x05040100u), __builtin_amdgcn_perm(d[1], d[0], 0x07060302u),
                                 __builtin_amdgcn_perm(d[3], d[2], 0x05040100u), __builtin_amdgcn_perm(d[3], d[2], 0x07060302u)};
                 const uint32_t e0 = (uint32_t)wf[2 * h], e1 = (uint32_t)wf[2 * h + 1];
+                if constexpr (XBF) {
+                    constexpr uint32_t kOne = 0x3f803f80u, kField = 0x00600060u;
+                    const v4u ones = {kOne, kOne, kOne, kOne};
+                    acc_x = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8b, ap), __builtin_bit_cast(v8b, ones), acc_x, 0, 0, 0);
+#pragma unroll
+                    for (int pp = 0; pp < 4; ++pp) {
+                        // field p of a half-word's low byte (even bytes) resp. high byte (odd bytes) -> mantissa bits 6:5
+                        const int up = 5 - 2 * pp;   // 5, 3, 1, -1
+                        const auto even = [&](uint32_t v) { return pp < 3 ? v << (up & 31) : v >> 1; };
+                        const v4u b = {(even(e0) & kField) | kOne, ((e0 >> (8 - up)) & kField) | kOne,
+                                       (even(e1) & kField) | kOne, ((e1 >> (8 - up)) & kField) | kOne};
+                        acc[pp] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8b, ap), __builtin_bit_cast(v8b, b), acc[pp], 0, 0, 0);
+                    }
+                    continue;
+                }
                 const uint32_t o0 = e0 >> 8, o1 = e1 >> 8;
 #pragma unroll
                 for (int pp = 0; pp < 4; ++pp) {
@@ -142,7 +171,19 @@ __global__ __launch_bounds__(kWaves * 64) void w2a16_kernel(const W2A16Params p)
             // end of a scale group: fold the group's sums into the running sums
             const bool group_ends = GS <= kChunkSteps ? ((s + 1) % GS == 0)
                                                       : (((step0 + c * kChunkSteps + s + 1) % GS) == 0);
-            if (group_ends) {
+            if (group_ends && XBF) {
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) {
+                    const uint32_t raw = pp < 2 ? cur.s[gi].x : cur.s[gi].y;
+                    const float sc4 = half_bits_to_float((uint16_t)((pp & 1) ? raw >> 16 : raw & 0xffffu)) * 4.0f;
+                    const uint32_t z = ZP ? (cur.z[gi] >> (8 * pp)) & 0xffu : (uint32_t)p.zp_const;
+                    const float off = -(4.0f + (float)z) * 0.25f;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) t[pp][j] = __builtin_fmaf(__builtin_fmaf(off, acc_x[j], acc[pp][j]), sc4, t[pp][j]);
+                    acc[pp] = v4f{0.f, 0.f, 0.f, 0.f};
+                }
+                acc_x = v4f{0.f, 0.f, 0.f, 0.f};
+            } else if (group_ends) {
 #pragma unroll
                 for (int pp = 0; pp < 4; ++pp) {
                     const uint32_t raw = pp < 2 ? cur.s[gi].x : cur.s[gi].y;
@@ -225,6 +266,11 @@ __global__ __launch_bounds__(256) void w2a16_reduce_kernel(const float* __restri
 
 template <int GS, int W, bool ZP, bool PARTIAL>
 void launch_one(const W2A16Params& p, bool out_bf16, dim3 grid, hipStream_t stream) {
+    if (p.x_bf16) {
+        if (out_bf16) w2a16_kernel<GS, W, ZP, PARTIAL, OutBF16, true><<<grid, dim3(W * 64), 0, stream>>>(p);
+        else w2a16_kernel<GS, W, ZP, PARTIAL, OutF16, true><<<grid, dim3(W * 64), 0, stream>>>(p);
+        return;
+    }
     if (out_bf16) w2a16_kernel<GS, W, ZP, PARTIAL, OutBF16><<<grid, dim3(W * 64), 0, stream>>>(p);
     else w2a16_kernel<GS, W, ZP, PARTIAL, OutF16><<<grid, dim3(W * 64), 0, stream>>>(p);
 }

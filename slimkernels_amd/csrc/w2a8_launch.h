@@ -99,7 +99,7 @@ int tiled_fast_effective_split(int steps, int gs, int split, int* groups_per_spl
 size_t tiled_fast_workspace_tiles(int M, int strips, int gs);
 // Weight-only form (fp16 activations on the fp16 matrix cores, gemm_w2a16.hip).
 struct W2A16Params {
-    const uint16_t* x;      // [M][ldx] fp16 bits
+    const uint16_t* x;      // [M][ldx] fp16 bits (bf16 bits with x_bf16)
     const uint32_t* w_r;    // repacked codes
     const uint16_t* s_r;    // [G][strips][16][4] fp16 bits
     const uint8_t* zp_r;    // [G][strips][16][4] or nullptr
@@ -110,6 +110,7 @@ struct W2A16Params {
     int G, steps, strips;
     int zp_const;
     int split;              // K splits across workgroups (grid.y)
+    bool x_bf16;            // bf16 activations: the bf16 matrix cores
 };
 int w2a16_auto_split(int M, int strips, int steps, int gs);
 hipError_t launch_w2a16(const W2A16Params& p, int gs, bool out_bf16, hipStream_t stream);

@@ -289,13 +289,13 @@ def w2a8_linear_fused(x: torch.Tensor, w: W2A8Weight, out_dtype=torch.float16, *
 
 def w2a16_gemm(x: torch.Tensor, w: W2A8Weight, out_dtype=torch.float16, *, split_k: int = 0,
                out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The weight-only form: out[M, N] = x @ dequant(W)^T with the fp16 activations x [M, K] as they are (no
-    activation quantisation), the 2-bit codes widened to fp16 in front of the fp16 matrix cores, fp32 sums.
+    """The weight-only form: out[M, N] = x @ dequant(W)^T with the fp16 or bf16 activations x [M, K] as they are (no
+    activation quantisation), the 2-bit codes widened in front of the fp16 resp. bf16 matrix cores, fp32 sums.
     Built for few token rows; K must be a multiple of 128."""
     L = _lib.lib()
     _require_cuda(x, "x")
-    if x.dim() != 2 or x.dtype != torch.float16:
-        raise ValueError("x must be a 2-D float16 tensor [M, K]")
+    if x.dim() != 2 or x.dtype not in _DT:
+        raise ValueError("x must be a 2-D float16 or bfloat16 tensor [M, K]")
     if out_dtype not in _DT:
         raise ValueError("out_dtype must be torch.float16 or torch.bfloat16")
     M, K = x.shape
@@ -466,13 +466,13 @@ class W2A8Linear(torch.nn.Module):
 
 
 class W2A16Linear(W2A8Linear):
-    """The same layer with the activations left in fp16 (weight-only quantisation): forward runs the
+    """The same layer with the activations left in fp16 or bf16 (weight-only quantisation): forward runs the
     weight-only kernel, meant for a few token rows; the weight object and the constructors are W2A8Linear's."""
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         lead = x.shape[:-1]
         x2 = x.reshape(-1, x.shape[-1])
-        if x2.dtype != torch.float16:
+        if x2.dtype not in _DT:
             x2 = x2.to(torch.float16)
         y = w2a16_gemm(x2, self.weight, self.out_dtype)
         if self.bias is not None:

@@ -1,4 +1,4 @@
-"""The weight-only form (fp16 activations times 2-bit weights on the fp16 matrix cores).
+"""The weight-only form (fp16 or bf16 activations times 2-bit weights on the fp16 resp. bf16 matrix cores).
 
 Upstream's sketch is the notebook kernel ``w2matmul`` (slimkernels/triton/gemm_splitk.ipynb cell 1): 2-bit
 fields widened to fp16 in front of an fp32-accumulating ``tl.dot``; it carries no scales and no zero-point and has
@@ -76,8 +76,7 @@ def test_w2a16_validation():
     assert call(x=None) == 1
     assert call(M=0) == 2
     assert call(K=4096 + 64, ldx=4160, g=64) == 7 and b"multiple of 128" in L.slimk_w2a8_last_error()
-    assert call(xdt=1) == 7 and b"fp16" in L.slimk_w2a8_last_error()      # bf16 activations
-    assert call(xdt=2) == 4 and call(odt=5) == 4
+    assert call(xdt=2) == 4 and call(odt=5) == 4                          # fp16 (0) and bf16 (1) activations only
     assert call(zpc=4) == 2
     assert call(ldx=4000) == 2 and call(ldo=100) == 2
     assert call(ldx=4100) == 3 and call(x=FAKE + 2) == 3
@@ -142,6 +141,50 @@ def test_w2a16_gemm_against_the_oracle(gpu_ops, oracle, M, N, K, g, mode, out, s
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K,g,mode,out,split", [
+    (1, 4096, 4096, 128, "sym", "bfloat16", 0),
+    (3, 200, 512, 64, "asym", "bfloat16", 1),      # N not a multiple of 64, per-group zero-points, group 64
+    (16, 1024, 2048, 128, "asym", "float16", 0),
+    (5, 320, 2048, 256, "sym", "bfloat16", 2),     # group 256: a group spans two loop iterations
+    (7, 192, 1792, 64, "ref", "bfloat16", 3),      # K-parts of unequal length, uniform zero-point 1
+    (40, 448, 1024, 128, "sym", "bfloat16", 0),    # several blocks of 16 token rows
+    (2, 14336, 4096, 128, "sym", "bfloat16", 0),
+])
+def test_w2a16_gemm_with_bf16_activations_against_the_oracle(gpu_ops, oracle, M, N, K, g, mode, out, split):
+    """bf16 activations as they are (the bf16 matrix cores; the codes enter as 1 + code / 4 and the group's activation sum
+    takes the offset and the zero-point off): the oracle's float64 result from the same bf16 values, to the tolerance
+    of the fp16 form.  A row of large activations with a non-zero mean is the case that costs this form bits."""
+    print(f"W2A16 bf16 activations M={M} N={N} K={K} g={g} {mode} {out} split={split}", flush=True)
+    case = pu.small_case(M, N, K, g, mode, seed=M * 11 + N, out_dtype=out)
+    packed, scales, zero = pu.quantized_weight(case)
+    x = workloads.make_activation(case).astype(np.float32)
+    x[0] = x[0] * 30.0 + 17.0                                             # large, far from zero mean
+    w, _ = pu.device_inputs(gpu_ops, case, packed, scales, zero, workloads.make_activation(case))
+    xd = torch.from_numpy(x).cuda().to(torch.bfloat16)
+    x_bits = xd.view(torch.int16).cpu().numpy().view(np.uint16)
+    want, mag = oracle.w2a16_reference_forward(x_bits, oracle.np_unpack(packed), scales, zero, g, x_bf16=True)
+    y = gpu_ops.w2a16_gemm(xd, w, pu.torch_dtype(case), split_k=split)
+    assert y.shape == (M, N)
+    _check(y, want, mag, out == "bfloat16", "W2A16 bf16 activations")
+    y2 = gpu_ops.w2a16_gemm(xd.clone(), w, pu.torch_dtype(case), split_k=split)
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
+
+
+@pytest.mark.gpu
+def test_w2a16_linear_layer_keeps_bf16_activations(gpu_ops, oracle):
+    case = pu.small_case(6, 256, 512, 128, "asym", seed=31, out_dtype="bfloat16")
+    packed, scales, zero = pu.quantized_weight(case)
+    w, _ = pu.device_inputs(gpu_ops, case, packed, scales, zero, workloads.make_activation(case))
+    layer = gpu_ops.W2A16Linear(w, out_dtype=torch.bfloat16)
+    x = torch.randn(2, 3, 512, device="cuda").to(torch.bfloat16)
+    y = layer(x)
+    x_bits = x.reshape(6, 512).view(torch.int16).cpu().numpy().view(np.uint16)
+    want, mag = oracle.w2a16_reference_forward(x_bits, oracle.np_unpack(packed), scales, zero, 128, x_bf16=True)
+    assert y.shape == (2, 3, 256) and y.dtype == torch.bfloat16
+    _check(y.reshape(6, 256), want, mag, True, "W2A16Linear bf16")
+
+
+@pytest.mark.gpu
 def test_w2a16_agrees_with_the_int8_path_to_the_activation_quantisation(gpu_ops):
     """Same weights, same activations: the W2A8 result differs from the weight-only one only by the int8
     rounding of the activations (per-token scale absmax / 127: relative error of a sum of K terms ~ 1 %)."""
@@ -202,6 +245,12 @@ def test_w2a16_seeded_random_shapes(gpu_ops, oracle, seed):
         want, mag = oracle.w2a16_reference_forward(x, oracle.np_unpack(packed), scales, zero, g)
         y = gpu_ops.w2a16_gemm(xd, w, pu.torch_dtype(case), split_k=split)
         _check(y, want, mag, out == "bfloat16", f"W2A16 seed {seed} case {i}")
+        # the same draw as bf16 activations (rounded from the fp16 values, shifted off zero mean in every other case)
+        xb = (xd.float() + (0.75 if i % 2 else 0.0)).to(torch.bfloat16)
+        x_bits = xb.view(torch.int16).cpu().numpy().view(np.uint16)
+        want, mag = oracle.w2a16_reference_forward(x_bits, oracle.np_unpack(packed), scales, zero, g, x_bf16=True)
+        y = gpu_ops.w2a16_gemm(xb, w, pu.torch_dtype(case), split_k=split)
+        _check(y, want, mag, out == "bfloat16", f"W2A16 bf16 activations seed {seed} case {i}")
 
 
 @pytest.mark.gpu
