@@ -589,6 +589,24 @@ def collect_detail(torch, np, ops, L, workloads, shapes, acts, cases, name_of, d
                             "GBps": round(nb / (us * 1e-6) / 1e9, 1), "frac_hbm": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)})
         del ws16
     detail["w2a16"] = a16rows
+    # one decode step's four linears (the c2 shapes) at one token row, weight-only: one grouped launch against four
+    layer = ((4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336))
+    sets = [[random_weight(N, K, 128, False) for (N, K) in layer] for _ in range(12)]
+    xs = {K: torch.randn(1, K, device=dev, dtype=torch.float16) for K in (4096, 14336)}
+    outs = [torch.empty((1, N), dtype=torch.float16, device=dev) for (N, K) in layer]
+    def single():
+        for ws in sets:
+            for w, o in zip(ws, outs):
+                ops.w2a16_gemm(xs[w.K], w, torch.float16, out=o)
+    def grouped():
+        for ws in sets:
+            ops.w2a16_gemm_grouped([(xs[w.K], w, o) for w, o in zip(ws, outs)], torch.float16)
+    us_single = time_graph(torch, single, len(sets), replays=4)
+    us_grouped = time_graph(torch, grouped, len(sets), replays=4)
+    nb = sum(N * K // 4 + 2 * N * (K // 128) + 2 * K + 2 * N for (N, K) in layer)
+    detail["w2a16_layer_m1"] = {"shapes": [f"{N}x{K}" for (N, K) in layer], "group": 128, "weights": "cold",
+                                "us_four_launches": round(us_single, 2), "us_one_grouped_launch": round(us_grouped, 2),
+                                "frac_hbm_grouped": round(nb / (us_grouped * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
     return detail
 
 

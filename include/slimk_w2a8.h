@@ -382,6 +382,29 @@ int slimk_w2a16_gemm(const void* x, int ldx, int x_dtype,
                      void* out, int ldo, int out_dtype,
                      void* workspace, size_t workspace_bytes, int split_k, void* stream);
 
+/* One problem of a grouped weight-only launch: the arguments of slimk_w2a16_gemm that describe data. */
+typedef struct slimk_w2a16_problem {
+    const void* x;       /* [M][ldx] fp16 or bf16 (the launch's x_dtype) */
+    const uint32_t* w_r;
+    const uint16_t* s_r;
+    const uint8_t* zp_r; /* NULL: uniform zero-point zp_const */
+    void* out;
+    int ldx, ldo;
+    int M, N, K;
+    int zp_const;
+} slimk_w2a16_problem;
+
+/* Several independent weight-only GEMMs in ONE kernel launch (the linears of a decode step that do not depend on one
+ * another): `problems` is a HOST array of `count` (1..SLIMK_W2A8_MAX_GROUP) entries, copied into the kernel arguments
+ * (graph-capturable, the array may be reused at once).  All problems share group_size, x_dtype and out_dtype, and
+ * either all carry per-group zero-points or none does; M, N, K may differ (K % 128 == 0 each).  No K splits across
+ * workgroups and no workspace: every problem runs as slimk_w2a16_gemm with split_k = 1 would, the number of K-parts
+ * inside a workgroup chosen once for the launch (so the fp32 summation order can differ from a single launch's).
+ * Inside the launch the problems run longest reduction first.
+ * No upstream counterpart (the notebook kernel w2matmul is one GEMM per launch). */
+int slimk_w2a16_gemm_grouped(const slimk_w2a16_problem* problems, int count, int group_size, int x_dtype, int out_dtype,
+                             void* stream);
+
 /* Streaming-read calibration kernel: sums `bytes` (multiple of 16) of device memory into
  * sink[0..] so that a profiler can relate its FETCH_SIZE counter to a known byte count and
  * the benchmark can quote the achievable HBM read rate next to the GEMM's. */

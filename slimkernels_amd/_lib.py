@@ -49,6 +49,7 @@ SIGNATURES = {
     "slimk_w2a16_gemm_auto_split_k": (_i, [_i, _i, _i, _i]),
     "slimk_w2a16_gemm_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "slimk_w2a16_gemm": (_i, [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _i, _vp, _sz, _i, _vp]),
+    "slimk_w2a16_gemm_grouped": (_i, [_vp, _i, _i, _i, _i, _vp]),
     "slimk_w2a8_read_probe": (_i, [_vp, _sz, _vp, _vp]),
 }
 MAX_GROUP = 24
@@ -59,6 +60,12 @@ class Problem(ctypes.Structure):
     """struct slimk_w2a8_problem"""
     _fields_ = [("q", _vp), ("s_a", _vp), ("rowsum", _vp), ("w_r", _vp), ("s_r", _vp), ("zp_r", _vp), ("out", _vp),
                 ("ldq", _i), ("ldr", _i), ("ldo", _i), ("M", _i), ("N", _i), ("K", _i), ("zp_const", _i)]
+
+
+class Problem16(ctypes.Structure):
+    """struct slimk_w2a16_problem"""
+    _fields_ = [("x", _vp), ("w_r", _vp), ("s_r", _vp), ("zp_r", _vp), ("out", _vp),
+                ("ldx", _i), ("ldo", _i), ("M", _i), ("N", _i), ("K", _i), ("zp_const", _i)]
 
 
 class SlimkError(RuntimeError):

@@ -948,6 +948,58 @@ int slimk_w2a16_gemm(const void* x, int ldx, int x_dtype,
     return hip_result(w2a8::launch_w2a16(p, gs, out_dtype == SLIMK_BF16, (hipStream_t)stream), "w2a16_gemm");
 }
 
+int slimk_w2a16_gemm_grouped(const slimk_w2a16_problem* problems, int count, int group_size, int x_dtype, int out_dtype,
+                             void* stream) {
+    if (!problems) return fail(SLIMK_ERR_NULL_POINTER, "w2a16_gemm_grouped: problems is NULL");
+    if (count < 1 || count > SLIMK_W2A8_MAX_GROUP)
+        return fail(SLIMK_ERR_BAD_SHAPE, "w2a16_gemm_grouped: count=%d must be 1..%d", count, SLIMK_W2A8_MAX_GROUP);
+    if (x_dtype != SLIMK_F16 && x_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "x_dtype=%d", x_dtype);
+    if (out_dtype != SLIMK_F16 && out_dtype != SLIMK_BF16) return fail(SLIMK_ERR_BAD_ENUM, "out_dtype=%d", out_dtype);
+    if (group_size != 64 && group_size != 128 && group_size != 256)
+        return fail(SLIMK_ERR_BAD_SHAPE, "group_size=%d must be 64, 128 or 256", group_size);
+    // longest reductions first, so that the workgroups that run longest do not start last
+    int order[SLIMK_W2A8_MAX_GROUP];
+    for (int i = 0; i < count; ++i) order[i] = i;
+    for (int i = 1; i < count; ++i)
+        for (int j = i; j > 0 && problems[order[j]].K > problems[order[j - 1]].K; --j) {
+            const int t = order[j]; order[j] = order[j - 1]; order[j - 1] = t;
+        }
+    w2a8::W2A16Group gp{};
+    gp.count = count;
+    int zm = -1;
+    long long wgs = 0;
+    for (int i = 0; i < count; ++i) {
+        const slimk_w2a16_problem& pr = problems[order[i]];
+        if (!pr.x || !pr.w_r || !pr.s_r || !pr.out)
+            return fail(SLIMK_ERR_NULL_POINTER, "w2a16_gemm_grouped: problem %d has a NULL buffer", order[i]);
+        if (pr.M <= 0 || pr.N <= 0) return fail(SLIMK_ERR_BAD_SHAPE, "w2a16_gemm_grouped: problem %d: M=%d, N=%d", order[i], pr.M, pr.N);
+        if (int rc = check_kg(pr.K, group_size)) return rc;
+        if (pr.K % 128 != 0) return fail(SLIMK_ERR_UNSUPPORTED, "w2a16_gemm_grouped: problem %d: K=%d must be a multiple of 128", order[i], pr.K);
+        if (pr.zp_const < 0 || pr.zp_const > 3) return fail(SLIMK_ERR_BAD_SHAPE, "w2a16_gemm_grouped: problem %d: zp_const=%d", order[i], pr.zp_const);
+        if (pr.ldx < pr.K || pr.ldo < pr.N)
+            return fail(SLIMK_ERR_BAD_SHAPE, "w2a16_gemm_grouped: problem %d: a leading dimension is too small", order[i]);
+        if (int rc = check_extent(pr.M, pr.N, pr.K, 2 * pr.ldx)) return rc;
+        if (!aligned16(pr.x) || pr.ldx % 8 != 0 || !aligned16(pr.w_r) || !aligned16(pr.s_r) || (pr.zp_r && !aligned16(pr.zp_r)) ||
+            (reinterpret_cast<uintptr_t>(pr.out) & 1u))
+            return fail(SLIMK_ERR_MISALIGNED, "w2a16_gemm_grouped: problem %d breaks an alignment rule of slimk_w2a16_gemm", order[i]);
+        const int this_zm = pr.zp_r ? 1 : 0;
+        if (zm >= 0 && this_zm != zm)
+            return fail(SLIMK_ERR_UNSUPPORTED, "w2a16_gemm_grouped: problems mix uniform and per-group zero-points");
+        zm = this_zm;
+        w2a8::W2A16Params& g = gp.prob[i];
+        g.x = reinterpret_cast<const uint16_t*>(pr.x); g.ldx = pr.ldx;
+        g.w_r = pr.w_r; g.s_r = pr.s_r; g.zp_r = pr.zp_r; g.out = pr.out; g.ldo = pr.ldo;
+        g.M = pr.M; g.N = pr.N; g.K = pr.K; g.G = pr.K / group_size; g.steps = pr.K / w2a8::kStepK; g.strips = strips_of(pr.N);
+        g.zp_const = pr.zp_const; g.split = 1; g.x_bf16 = x_dtype == SLIMK_BF16;
+        gp.wg_begin[i] = (int)wgs;
+        wgs += (long long)g.strips * ((pr.M + 15) / 16);
+        if (wgs > (1 << 24)) return fail(SLIMK_ERR_UNSUPPORTED, "w2a16_gemm_grouped: more than 2^24 workgroups");
+    }
+    gp.wg_begin[count] = (int)wgs;
+    return hip_result(w2a8::launch_w2a16_grouped(gp, group_size / w2a8::kStepK, zm == 1, out_dtype == SLIMK_BF16,
+                                                 x_dtype == SLIMK_BF16, (hipStream_t)stream), "w2a16 grouped gemm");
+}
+
 int slimk_w2a8_read_probe(const void* src, size_t bytes, uint32_t* sink, void* stream) {
     if (!src || !sink) return fail(SLIMK_ERR_NULL_POINTER, "read_probe: NULL buffer");
     if (bytes == 0 || bytes % 16 != 0 || !aligned16(src))

@@ -28,6 +28,8 @@
 //   sum_k x * (code - zp) = 4 * sum_k x * (1 + code / 4) - (4 + zp) * sum_k x
 // is put together in fp32 (every product is exact; the two sums are a few times larger than their difference, which
 // costs an fp32 accumulation a few of its 24 bits).
+#include <algorithm>
+
 #include "w2a8_launch.h"
 
 namespace w2a8 {
@@ -48,21 +50,21 @@ typedef __bf16 v8b __attribute__((ext_vector_type(8)));
 // (The bf16 form is held to 128 registers, two eight-wave workgroups per CU: left alone it takes 162 and one
 // workgroup, 35.7 instead of 22.0 us at 28672 x 8192, one row; groups of 256 would spill 252 bytes at that limit and
 // keep the compiler's own choice, as every fp16 instantiation does.)
-template <int GS, int kWaves, bool ZP, bool PARTIAL, typename OutT, bool XBF = false>
-__global__ __launch_bounds__(kWaves * 64, XBF && GS < 4 ? 4 : 1) void w2a16_kernel(const W2A16Params p) {
-    __shared__ float red[kWaves][16][64];
+// strip, split_idx, mblk: the workgroup's strip of 64 channels, its K split (PARTIAL) and its block of 16 token rows
+template <int GS, int kWaves, bool ZP, bool PARTIAL, typename OutT, bool XBF>
+__device__ __forceinline__ void w2a16_body(const W2A16Params& p, const int strip, const int split_idx, const int mblk,
+                                           float (&red)[kWaves][16][64]) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 15, quad = lane >> 4;
-    const int strip = blockIdx.x;
-    const int m0 = (int)blockIdx.z * 16;
+    const int m0 = mblk * 16;
 
     // K-parts in granules of max(GS, 2) steps, dealt out evenly over split * kWaves parts (a part may be empty)
     constexpr int kGranule = GS > kChunkSteps ? GS : kChunkSteps;
     const int n_gran = p.steps / kGranule;
     const int parts = p.split * kWaves;
-    const int part = (int)blockIdx.y * kWaves + wave;
+    const int part = split_idx * kWaves + wave;
     const int gr0 = (int)((long long)part * n_gran / parts), gr1 = (int)((long long)(part + 1) * n_gran / parts);
     const int step0 = gr0 * kGranule;
     const int n_chunks = (gr1 - gr0) * (kGranule / kChunkSteps);
@@ -247,10 +249,31 @@ __global__ __launch_bounds__(kWaves * 64, XBF && GS < 4 ? 4 : 1) void w2a16_kern
         const int m = m0 + quad * 4 + j;
         const int n = strip * kStripN + pp * 16 + col;
         if (m < p.M && n < p.N) {
-            if (PARTIAL) p.ws[((size_t)blockIdx.y * p.M + m) * p.N + n] = v;
+            if (PARTIAL) p.ws[((size_t)split_idx * p.M + m) * p.N + n] = v;
             else reinterpret_cast<uint16_t*>(p.out)[(size_t)m * p.ldo + n] = OutT::cast(v);
         }
     }
+}
+
+template <int GS, int kWaves, bool ZP, bool PARTIAL, typename OutT, bool XBF = false>
+__global__ __launch_bounds__(kWaves * 64, XBF && GS < 4 ? 4 : 1) void w2a16_kernel(const W2A16Params p) {
+    __shared__ float red[kWaves][16][64];
+    w2a16_body<GS, kWaves, ZP, PARTIAL, OutT, XBF>(p, (int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z, red);
+}
+
+// Several problems in one launch (no K splits across workgroups): workgroup ids are cut into runs, one per problem,
+// strip fastest within a run; the problem table travels in the kernel arguments.
+template <int GS, int kWaves, bool ZP, typename OutT, bool XBF>
+__global__ __launch_bounds__(kWaves * 64, XBF && GS < 4 ? 4 : 1) void w2a16_grouped_kernel(const W2A16Group gp) {
+    __shared__ float red[kWaves][16][64];
+    const int wg = (int)blockIdx.x;
+    // problem index = number of run boundaries at or below this workgroup id: one lane per boundary, one ballot
+    const int bl = min((int)(threadIdx.x & 63), kMaxGroup - 1);
+    const bool past = bl + 1 < gp.count && wg >= gp.wg_begin[bl + 1];
+    const int i = __builtin_amdgcn_readfirstlane(__builtin_popcountll(__ballot(past)));
+    const W2A16Params& p = gp.prob[i];
+    const int local = wg - gp.wg_begin[i];
+    w2a16_body<GS, kWaves, ZP, false, OutT, XBF>(p, local % p.strips, 0, local / p.strips, red);
 }
 
 template <typename OutT>
@@ -320,6 +343,44 @@ static int w2a16_waves(int M, int strips, int steps, int gs, int split) {
     int waves = wanted >= 12 ? 16 : wanted >= 6 ? 8 : 4;
     while (waves > 4 && (long long)waves * split * 4 > chunks) waves /= 2;
     return waves;
+}
+
+namespace {
+template <int GS, int W>
+void launch_group_w(const W2A16Group& gp, bool zp, bool out_bf16, bool x_bf16, dim3 grid, hipStream_t stream) {
+#define SLIMK_W2A16_GROUP(ZPV, OUT, XB) w2a16_grouped_kernel<GS, W, ZPV, OUT, XB><<<grid, dim3(W * 64), 0, stream>>>(gp)
+    if (zp) {
+        if (x_bf16) { if (out_bf16) SLIMK_W2A16_GROUP(true, OutBF16, true); else SLIMK_W2A16_GROUP(true, OutF16, true); }
+        else { if (out_bf16) SLIMK_W2A16_GROUP(true, OutBF16, false); else SLIMK_W2A16_GROUP(true, OutF16, false); }
+    } else {
+        if (x_bf16) { if (out_bf16) SLIMK_W2A16_GROUP(false, OutBF16, true); else SLIMK_W2A16_GROUP(false, OutF16, true); }
+        else { if (out_bf16) SLIMK_W2A16_GROUP(false, OutBF16, false); else SLIMK_W2A16_GROUP(false, OutF16, false); }
+    }
+#undef SLIMK_W2A16_GROUP
+}
+template <int GS>
+void launch_group_gs(const W2A16Group& gp, int waves, bool zp, bool out_bf16, bool x_bf16, dim3 grid, hipStream_t stream) {
+    if (waves == 16) launch_group_w<GS, 16>(gp, zp, out_bf16, x_bf16, grid, stream);
+    else if (waves == 8) launch_group_w<GS, 8>(gp, zp, out_bf16, x_bf16, grid, stream);
+    else launch_group_w<GS, 4>(gp, zp, out_bf16, x_bf16, grid, stream);
+}
+}  // namespace
+
+// The K-parts inside a workgroup are one choice for the whole launch: towards 16 wavefronts per CU over all its
+// workgroups, every part of the shortest reduction at least four chunks long where K allows.
+hipError_t launch_w2a16_grouped(const W2A16Group& gp, int gs, bool zp, bool out_bf16, bool x_bf16, hipStream_t stream) {
+    const int total = gp.wg_begin[gp.count];
+    int min_steps = gp.prob[0].steps;
+    for (int i = 1; i < gp.count; ++i) min_steps = std::min(min_steps, gp.prob[i].steps);
+    const int chunks = min_steps / kChunkSteps;
+    const long long wanted = 4096 / (total < 1 ? 1 : total);
+    int waves = wanted >= 12 ? 16 : wanted >= 6 ? 8 : 4;
+    while (waves > 4 && waves * 4 > chunks) waves /= 2;
+    const dim3 grid((unsigned)total);
+    if (gs == 1) launch_group_gs<1>(gp, waves, zp, out_bf16, x_bf16, grid, stream);
+    else if (gs == 2) launch_group_gs<2>(gp, waves, zp, out_bf16, x_bf16, grid, stream);
+    else launch_group_gs<4>(gp, waves, zp, out_bf16, x_bf16, grid, stream);
+    return hipGetLastError();
 }
 
 hipError_t launch_w2a16(const W2A16Params& p, int gs, bool out_bf16, hipStream_t stream) {

@@ -322,6 +322,48 @@ def w2a16_gemm(x: torch.Tensor, w: W2A8Weight, out_dtype=torch.float16, *, split
     return out
 
 
+def w2a16_gemm_grouped(problems, out_dtype=torch.float16):
+    """Several independent weight-only GEMMs in one kernel launch.
+
+    ``problems`` is a sequence of (x, W2A8Weight) or (x, w, out) tuples whose activations share one type (float16 or
+    bfloat16) and whose weights share group size and zero-point mode; returns the list of outputs.  More than 24
+    problems are issued as several launches."""
+    L = _lib.lib()
+    probs = [(p[0], p[1], p[2] if len(p) > 2 else None) for p in problems]
+    if not probs:
+        return []
+    dev = probs[0][0].device
+    xdt = probs[0][0].dtype
+    g = probs[0][1].group_size
+    if xdt not in _DT or out_dtype not in _DT:
+        raise ValueError("activations and out_dtype must be torch.float16 or torch.bfloat16")
+    outs, keep = [], []
+    with torch.cuda.device(dev):
+        for lo in range(0, len(probs), _lib.MAX_GROUP):
+            chunk = probs[lo:lo + _lib.MAX_GROUP]
+            arr = (_lib.Problem16 * len(chunk))()
+            for i, (x, w, out) in enumerate(chunk):
+                _require_cuda(x, "x")
+                if x.dim() != 2 or x.dtype != xdt or x.shape[1] != w.K or w.group_size != g:
+                    raise ValueError("grouped problems must share the activation type and group size and match their weights' K")
+                M, K = x.shape
+                if x.stride(1) != 1 or x.stride(0) % 8 != 0 or x.stride(0) < K or x.data_ptr() % 16 != 0:
+                    x = x.contiguous()
+                    if x.data_ptr() % 16 != 0:
+                        x = x.clone()
+                keep.append(x)
+                if out is None:
+                    out = torch.empty((M, w.N), dtype=out_dtype, device=dev)
+                if out.dtype != out_dtype:
+                    raise ValueError("every output must have dtype out_dtype")
+                outs.append(out)
+                arr[i] = _lib.Problem16(x.data_ptr(), w.w_r.data_ptr(), w.s_r.data_ptr(),
+                                        w.zp_r.data_ptr() if w.zp_r is not None else None, out.data_ptr(),
+                                        x.stride(0), out.stride(0), M, w.N, K, w.zp_const)
+            _lib.check(L.slimk_w2a16_gemm_grouped(ctypes.byref(arr), len(chunk), g, _DT[xdt], _DT[out_dtype], _stream_ptr(dev)))
+    return outs
+
+
 def w2a8_gemm_grouped(problems, out_dtype=torch.float16, *, dump: Optional[str] = None):
     """Several independent skinny (M <= 32) GEMMs in one kernel launch.
 

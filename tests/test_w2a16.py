@@ -184,6 +184,60 @@ def test_w2a16_linear_layer_keeps_bf16_activations(gpu_ops, oracle):
     _check(y.reshape(6, 256), want, mag, True, "W2A16Linear bf16")
 
 
+def test_w2a16_grouped_validation():
+    L = _lib.lib()
+    P = _lib.Problem16
+    def arr(*ps):
+        a = (P * len(ps))(*ps)
+        return ctypes.byref(a), len(ps)
+    ok = dict(x=FAKE, w_r=FAKE, s_r=FAKE, zp_r=None, out=FAKE, ldx=4096, ldo=4096, M=1, N=4096, K=4096, zp_const=2)
+    def prob(**kw):
+        d = dict(ok); d.update(kw)
+        return P(d["x"], d["w_r"], d["s_r"], d["zp_r"], d["out"], d["ldx"], d["ldo"], d["M"], d["N"], d["K"], d["zp_const"])
+    g = L.slimk_w2a16_gemm_grouped
+    a, n = arr(prob())
+    assert g(None, 1, 128, 0, 0, None) == 1
+    assert g(a, 0, 128, 0, 0, None) == 2 and g(a, 25, 128, 0, 0, None) == 2
+    assert g(a, n, 128, 2, 0, None) == 4 and g(a, n, 128, 0, 3, None) == 4 and g(a, n, 100, 0, 0, None) == 2
+    for bad, code in ((dict(x=None), 1), (dict(M=0), 2), (dict(K=4096 + 64, ldx=4160), 7), (dict(ldx=4000), 2), (dict(ldo=8), 2),
+                      (dict(x=FAKE + 2), 3), (dict(ldx=4100), 3), (dict(zp_const=4), 2)):
+        a, n = arr(prob(), prob(**bad))
+        assert g(a, n, 64, 0, 0, None) == code, (bad, L.slimk_w2a8_last_error())
+    a, n = arr(prob(), prob(zp_r=FAKE))
+    assert g(a, n, 128, 1, 1, None) == 7 and b"mix" in L.slimk_w2a8_last_error()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("xdt,mode,out,g", [("float16", "sym", "float16", 128), ("bfloat16", "asym", "bfloat16", 64),
+                                             ("bfloat16", "ref", "float16", 256), ("float16", "asym", "bfloat16", 128)])
+def test_w2a16_grouped_launch_against_the_oracle(gpu_ops, oracle, xdt, mode, out, g):
+    """Problems of different M, N (ragged) and K in one launch: every output against the oracle to the single launch's
+    tolerance, a second launch bit-identical, and a launch of one problem."""
+    shapes = [(1, 512, 1024), (3, 200, 512), (16, 1000, 2048), (17, 64, 256), (40, 320, 1536), (2, 4096, 4096)]
+    dt = torch.bfloat16 if xdt == "bfloat16" else torch.float16
+    odt = torch.bfloat16 if out == "bfloat16" else torch.float16
+    probs, wants = [], []
+    for i, (M, N, K) in enumerate(shapes):
+        case = pu.small_case(M, N, K, g, mode, seed=500 + i, out_dtype=out)
+        packed, scales, zero = pu.quantized_weight(case)
+        w, xd = pu.device_inputs(gpu_ops, case, packed, scales, zero, workloads.make_activation(case))
+        xd = (xd.float() + (0.5 if i % 2 else 0.0)).to(dt)
+        x_np = xd.view(torch.int16).cpu().numpy().view(np.uint16) if dt == torch.bfloat16 else xd.cpu().numpy()
+        wants.append(oracle.w2a16_reference_forward(x_np, oracle.np_unpack(packed), scales, zero, g, x_bf16=dt == torch.bfloat16))
+        probs.append((xd, w))
+    outs = gpu_ops.w2a16_gemm_grouped(probs, odt)
+    torch.cuda.synchronize()
+    for i, (y, (want, mag)) in enumerate(zip(outs, wants)):
+        assert y.shape == (shapes[i][0], shapes[i][1]) and y.dtype == odt
+        _check(y, want, mag, out == "bfloat16", f"W2A16 grouped problem {i} {shapes[i]}")
+    again = gpu_ops.w2a16_gemm_grouped(probs, odt)
+    assert all(torch.equal(a.view(torch.int16), b.view(torch.int16)) for a, b in zip(outs, again))
+    one = gpu_ops.w2a16_gemm_grouped(probs[2:3], odt)
+    _check(one[0], wants[2][0], wants[2][1], out == "bfloat16", "W2A16 grouped launch of one problem")
+    with pytest.raises(ValueError):
+        gpu_ops.w2a16_gemm_grouped([probs[0], (probs[1][0].to(torch.float16 if dt == torch.bfloat16 else torch.bfloat16), probs[1][1])], odt)
+
+
 @pytest.mark.gpu
 def test_w2a16_agrees_with_the_int8_path_to_the_activation_quantisation(gpu_ops):
     """Same weights, same activations: the W2A8 result differs from the weight-only one only by the int8
