@@ -47,6 +47,9 @@ def test_replays_repeat_the_eager_calls(gpu_ops):
         case, w, xd = _prepare(gpu_ops, M, N, K, 128, "sym", 970 + i)
         fused.append((case, w, xd))
 
+    a16_xb = fused[0][2].to(torch.bfloat16)
+    a16_outs = [torch.empty((1, 2048), dtype=torch.float16, device="cuda") for _ in range(2)] + \
+               [torch.empty((c[0].M, c[0].N), dtype=torch.float16, device="cuda") for c in grouped]
     qas = {}
     static_outs = [torch.empty((p[0].M, p[0].N), dtype=torch.float16, device="cuda") for p in prepared[:1] + prepared[3:4]]
 
@@ -65,6 +68,12 @@ def test_replays_repeat_the_eager_calls(gpu_ops):
         outs += gpu_ops.w2a8_gemm_grouped(probs, torch.float16)
         for case, w, xd in fused:
             outs.append(gpu_ops.w2a8_linear_fused(xd, w, torch.float16))
+        # the weight-only form: one launch with K split through its own partial-sum buffer, bf16 activations, and the
+        # grouped launch
+        case, w, xd = fused[0][0], fused[0][1], fused[0][2]
+        outs.append(gpu_ops.w2a16_gemm(xd, w, torch.float16, split_k=2, out=a16_outs[0]))
+        outs.append(gpu_ops.w2a16_gemm(a16_xb, w, torch.float16, out=a16_outs[1]))
+        outs += gpu_ops.w2a16_gemm_grouped([(c[2], c[1], o) for c, o in zip(grouped, a16_outs[2:])], torch.float16)
         # the entry point that allocates nothing (split-K through the library-owned array): its first call on the
         # device is the eager one below, outside the capture
         for (case, w, xd, kernel, _), out in zip(prepared[:1] + prepared[3:4], static_outs):
