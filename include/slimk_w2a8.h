@@ -398,8 +398,8 @@ typedef struct slimk_w2a16_problem {
  * another): `problems` is a HOST array of `count` (1..SLIMK_W2A8_MAX_GROUP) entries, copied into the kernel arguments
  * (graph-capturable, the array may be reused at once).  All problems share group_size, x_dtype and out_dtype, and
  * either all carry per-group zero-points or none does; M, N, K may differ (K % 128 == 0 each).  No K splits across
- * workgroups and no workspace: every problem runs as slimk_w2a16_gemm with split_k = 1 would, the number of K-parts
- * inside a workgroup chosen once for the launch (so the fp32 summation order can differ from a single launch's).
+ * workgroups and no workspace: a workgroup holds one or several strips of a problem, each in as many K-parts as its
+ * reduction length suggests (so the fp32 summation order can differ from a single launch's).
  * Inside the launch the problems run longest reduction first.
  * No upstream counterpart (the notebook kernel w2matmul is one GEMM per launch). */
 int slimk_w2a16_gemm_grouped(const slimk_w2a16_problem* problems, int count, int group_size, int x_dtype, int out_dtype,

@@ -966,6 +966,12 @@ int slimk_w2a16_gemm_grouped(const slimk_w2a16_problem* problems, int count, int
         }
     w2a8::W2A16Group gp{};
     gp.count = count;
+    // Sixteen waves per workgroup when a reduction of the launch is long enough to occupy them (128 steps and more),
+    // eight otherwise; a problem's strips take as many K-parts as leave a part eight steps (four chunks, one trip of
+    // the kernel's main loop), the rest of the workgroup's waves go to neighbouring strips.
+    int max_steps = 0;
+    for (int i = 0; i < count; ++i) max_steps = std::max(max_steps, problems[i].K / w2a8::kStepK);
+    gp.waves = max_steps >= 128 ? 16 : 8;
     int zm = -1;
     long long wgs = 0;
     for (int i = 0; i < count; ++i) {
@@ -991,8 +997,12 @@ int slimk_w2a16_gemm_grouped(const slimk_w2a16_problem* problems, int count, int
         g.w_r = pr.w_r; g.s_r = pr.s_r; g.zp_r = pr.zp_r; g.out = pr.out; g.ldo = pr.ldo;
         g.M = pr.M; g.N = pr.N; g.K = pr.K; g.G = pr.K / group_size; g.steps = pr.K / w2a8::kStepK; g.strips = strips_of(pr.N);
         g.zp_const = pr.zp_const; g.split = 1; g.x_bf16 = x_dtype == SLIMK_BF16;
+        int lp = 0;
+        while ((2 << lp) <= gp.waves && g.steps / (2 << lp) >= 8) ++lp;
+        gp.log_parts[i] = lp;
+        const int per = gp.waves >> lp;
         gp.wg_begin[i] = (int)wgs;
-        wgs += (long long)g.strips * ((pr.M + 15) / 16);
+        wgs += (long long)((g.strips + per - 1) / per) * ((pr.M + 15) / 16);
         if (wgs > (1 << 24)) return fail(SLIMK_ERR_UNSUPPORTED, "w2a16_gemm_grouped: more than 2^24 workgroups");
     }
     gp.wg_begin[count] = (int)wgs;

@@ -50,21 +50,27 @@ typedef __bf16 v8b __attribute__((ext_vector_type(8)));
 // (The bf16 form is held to 128 registers, two eight-wave workgroups per CU: left alone it takes 162 and one
 // workgroup, 35.7 instead of 22.0 us at 28672 x 8192, one row; groups of 256 would spill 252 bytes at that limit and
 // keep the compiler's own choice, as every fp16 instantiation does.)
-// strip, split_idx, mblk: the workgroup's strip of 64 channels, its K split (PARTIAL) and its block of 16 token rows
+// unit, split_idx, mblk: the workgroup's set of strips, its K split (PARTIAL) and its block of 16 token rows.
+// lp: log2 of the K-parts per strip inside the workgroup, P; the workgroup holds kWaves / P strips (unit * kWaves / P
+// onwards), wave w works on strip w / P, part w % P.  One launch of one problem runs P = kWaves (one strip).
 template <int GS, int kWaves, bool ZP, bool PARTIAL, typename OutT, bool XBF>
-__device__ __forceinline__ void w2a16_body(const W2A16Params& p, const int strip, const int split_idx, const int mblk,
-                                           float (&red)[kWaves][16][64]) {
+__device__ __forceinline__ void w2a16_body(const W2A16Params& p, const int unit, const int split_idx, const int mblk,
+                                           const int lp, float (&red)[kWaves][16][64]) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 15, quad = lane >> 4;
     const int m0 = mblk * 16;
+    const int P = 1 << lp, sidx = wave >> lp, kp = wave & (P - 1);
+    const int strip_raw = unit * (kWaves >> lp) + sidx;
+    const bool strip_ok = strip_raw < p.strips;     // a surplus wave streams the last strip and stores nothing
+    const int strip = min(strip_raw, p.strips - 1);
 
     // K-parts in granules of max(GS, 2) steps, dealt out evenly over split * kWaves parts (a part may be empty)
     constexpr int kGranule = GS > kChunkSteps ? GS : kChunkSteps;
     const int n_gran = p.steps / kGranule;
-    const int parts = p.split * kWaves;
-    const int part = split_idx * kWaves + wave;
+    const int parts = p.split * P;
+    const int part = split_idx * P + kp;
     const int gr0 = (int)((long long)part * n_gran / parts), gr1 = (int)((long long)(part + 1) * n_gran / parts);
     const int step0 = gr0 * kGranule;
     const int n_chunks = (gr1 - gr0) * (kGranule / kChunkSteps);
@@ -239,16 +245,15 @@ __device__ __forceinline__ void w2a16_body(const W2A16Params& p, const int strip
 #pragma unroll
         for (int j = 0; j < 4; ++j) red[wave][pp * 4 + j][lane] = t[pp][j];
     __syncthreads();
-    constexpr int kRows = 16 / kWaves;
-#pragma unroll
-    for (int i = 0; i < kRows; ++i) {
-        const int r = wave * kRows + i, pp = r >> 2, j = r & 3;
-        float v = red[0][r][lane];
-#pragma unroll
-        for (int w = 1; w < kWaves; ++w) v += red[w][r][lane];
+    // wave (strip s, part k) finishes rows k * 16 / P onwards of strip s: the parts' sums in part order
+    const int rows = 16 >> lp;
+    for (int i = 0; i < rows; ++i) {
+        const int r = kp * rows + i, pp = r >> 2, j = r & 3;
+        float v = red[sidx << lp][r][lane];
+        for (int w = 1; w < P; ++w) v += red[(sidx << lp) + w][r][lane];
         const int m = m0 + quad * 4 + j;
         const int n = strip * kStripN + pp * 16 + col;
-        if (m < p.M && n < p.N) {
+        if (strip_ok && m < p.M && n < p.N) {
             if (PARTIAL) p.ws[((size_t)split_idx * p.M + m) * p.N + n] = v;
             else reinterpret_cast<uint16_t*>(p.out)[(size_t)m * p.ldo + n] = OutT::cast(v);
         }
@@ -258,11 +263,14 @@ __device__ __forceinline__ void w2a16_body(const W2A16Params& p, const int strip
 template <int GS, int kWaves, bool ZP, bool PARTIAL, typename OutT, bool XBF = false>
 __global__ __launch_bounds__(kWaves * 64, XBF && GS < 4 ? 4 : 1) void w2a16_kernel(const W2A16Params p) {
     __shared__ float red[kWaves][16][64];
-    w2a16_body<GS, kWaves, ZP, PARTIAL, OutT, XBF>(p, (int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z, red);
+    constexpr int kLogWaves = kWaves == 16 ? 4 : kWaves == 8 ? 3 : 2;
+    w2a16_body<GS, kWaves, ZP, PARTIAL, OutT, XBF>(p, (int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z, kLogWaves, red);
 }
 
 // Several problems in one launch (no K splits across workgroups): workgroup ids are cut into runs, one per problem,
-// strip fastest within a run; the problem table travels in the kernel arguments.
+// set of strips fastest within a run; every problem has its own number of K-parts per strip (a long reduction all the
+// waves of a workgroup on one strip, a short one several strips side by side); the problem table travels in the kernel
+// arguments.
 template <int GS, int kWaves, bool ZP, typename OutT, bool XBF>
 __global__ __launch_bounds__(kWaves * 64, XBF && GS < 4 ? 4 : 1) void w2a16_grouped_kernel(const W2A16Group gp) {
     __shared__ float red[kWaves][16][64];
@@ -273,7 +281,9 @@ __global__ __launch_bounds__(kWaves * 64, XBF && GS < 4 ? 4 : 1) void w2a16_grou
     const int i = __builtin_amdgcn_readfirstlane(__builtin_popcountll(__ballot(past)));
     const W2A16Params& p = gp.prob[i];
     const int local = wg - gp.wg_begin[i];
-    w2a16_body<GS, kWaves, ZP, false, OutT, XBF>(p, local % p.strips, 0, local / p.strips, red);
+    const int lp = gp.log_parts[i];
+    const int per = kWaves >> lp, units = (p.strips + per - 1) / per;
+    w2a16_body<GS, kWaves, ZP, false, OutT, XBF>(p, local % units, 0, local / units, lp, red);
 }
 
 template <typename OutT>
@@ -366,20 +376,12 @@ void launch_group_gs(const W2A16Group& gp, int waves, bool zp, bool out_bf16, bo
 }
 }  // namespace
 
-// The K-parts inside a workgroup are one choice for the whole launch: towards 16 wavefronts per CU over all its
-// workgroups, every part of the shortest reduction at least four chunks long where K allows.
+// gp.waves wavefronts per workgroup (4, 8 or 16), gp.log_parts[i] the K-parts per strip of problem i
 hipError_t launch_w2a16_grouped(const W2A16Group& gp, int gs, bool zp, bool out_bf16, bool x_bf16, hipStream_t stream) {
-    const int total = gp.wg_begin[gp.count];
-    int min_steps = gp.prob[0].steps;
-    for (int i = 1; i < gp.count; ++i) min_steps = std::min(min_steps, gp.prob[i].steps);
-    const int chunks = min_steps / kChunkSteps;
-    const long long wanted = 4096 / (total < 1 ? 1 : total);
-    int waves = wanted >= 12 ? 16 : wanted >= 6 ? 8 : 4;
-    while (waves > 4 && waves * 4 > chunks) waves /= 2;
-    const dim3 grid((unsigned)total);
-    if (gs == 1) launch_group_gs<1>(gp, waves, zp, out_bf16, x_bf16, grid, stream);
-    else if (gs == 2) launch_group_gs<2>(gp, waves, zp, out_bf16, x_bf16, grid, stream);
-    else launch_group_gs<4>(gp, waves, zp, out_bf16, x_bf16, grid, stream);
+    const dim3 grid((unsigned)gp.wg_begin[gp.count]);
+    if (gs == 1) launch_group_gs<1>(gp, gp.waves, zp, out_bf16, x_bf16, grid, stream);
+    else if (gs == 2) launch_group_gs<2>(gp, gp.waves, zp, out_bf16, x_bf16, grid, stream);
+    else launch_group_gs<4>(gp, gp.waves, zp, out_bf16, x_bf16, grid, stream);
     return hipGetLastError();
 }
 

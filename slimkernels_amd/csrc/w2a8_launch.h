@@ -115,11 +115,14 @@ struct W2A16Params {
 int w2a16_auto_split(int M, int strips, int steps, int gs);
 hipError_t launch_w2a16(const W2A16Params& p, int gs, bool out_bf16, hipStream_t stream);
 // Several weight-only problems in one launch (each unsplit; the activation type, zero-point mode and output type are
-// the launch's): problem i owns workgroups wg_begin[i] .. wg_begin[i+1]-1, strips x blocks of 16 token rows.
+// the launch's): problem i owns workgroups wg_begin[i] .. wg_begin[i+1]-1, sets of strips x blocks of 16 token rows;
+// a workgroup of `waves` wavefronts holds waves >> log_parts[i] strips of problem i, each in 1 << log_parts[i] K-parts.
 struct W2A16Group {
     W2A16Params prob[kMaxGroup];
     int wg_begin[kMaxGroup + 1];
+    int log_parts[kMaxGroup];
     int count;
+    int waves;
 };
 hipError_t launch_w2a16_grouped(const W2A16Group& gp, int gs, bool zp, bool out_bf16, bool x_bf16, hipStream_t stream);
 
